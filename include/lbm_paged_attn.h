@@ -1,0 +1,170 @@
+/*
+ * lbm_paged_attn.h - C ABI of the MI355X (gfx950) streaming paged-KV attention library.
+ *
+ * The reference (Robbyant/lingbot-map) has no FFI on this path: its boundary is the Python
+ * KV-cache manager lingbot_map/layers/flashinfer_cache.py:55 and the third-party FlashInfer
+ * wrapper it drives.  Each entry point below names the reference interface it stands in for.
+ * All pointers are raw device pointers unless marked "host"; all sizes are plain integers;
+ * `stream` is a hipStream_t passed as void* (NULL = the null stream).  Every function returns
+ * LBM_OK or an LBM_ERR_* code and never throws; lbm_last_error() gives the text of the last
+ * failure on the calling thread.  No function synchronises the device.
+ *
+ * Data layout (flashinfer_cache.py:141-148): one pool per transformer block,
+ *   pool[page][2][page_size][num_heads][head_dim]      dim 1: 0 = K, 1 = V
+ * A "row" is one token's [num_heads][head_dim] vector; the K row index of (page, slot) is
+ * page * 2 * page_size + slot and the matching V row is page_size rows later.
+ */
+#ifndef LBM_PAGED_ATTN_H
+#define LBM_PAGED_ATTN_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define LBM_ABI_VERSION 1
+
+#define LBM_OK 0
+#define LBM_ERR_INVALID 1     /* bad argument (null pointer, negative size, bad enum)      */
+#define LBM_ERR_UNSUPPORTED 2 /* shape the kernels do not cover (head_dim != 64, ...)       */
+#define LBM_ERR_WORKSPACE 3   /* workspace too small; see lbm_attn_workspace_bytes          */
+#define LBM_ERR_HIP 4         /* a HIP runtime call failed                                  */
+
+#define LBM_DTYPE_BF16 0
+#define LBM_DTYPE_F32 1
+
+#define LBM_LAYOUT_TWO_STREAM 0  /* reference: patch pages + packed special stream         */
+#define LBM_LAYOUT_FRAME_PAGES 1 /* whole frame in pages; eviction compacts index-only     */
+
+#define LBM_MAX_STREAMS 16
+
+/* Table operations, executed in this fixed order when several bits are set. */
+#define LBM_OP_RESET 1
+#define LBM_OP_ROLLBACK 2
+#define LBM_OP_APPEND 4
+#define LBM_OP_EVICT 8
+#define LBM_OP_PLAN 16
+
+/* Sticky bits of the device-side error word (header word LBM_HDR_ERROR). */
+#define LBM_TERR_PATCH_POOL 1   /* flashinfer_cache.py:489-494 */
+#define LBM_TERR_SPECIAL_POOL 2 /* flashinfer_cache.py:533-537 */
+#define LBM_TERR_WINDOW_RING 4
+#define LBM_TERR_MEMORY_FULL 8
+#define LBM_TERR_ROLLBACK 16    /* flashinfer_cache.py:276-278,290-293 */
+#define LBM_TERR_KV_COUNT 32    /* host and device disagree on the visible token count */
+
+/* Header words at the start of each stream's table block. */
+#define LBM_HDR_FRAME_COUNT 0
+#define LBM_HDR_N_ANCHOR 1
+#define LBM_HDR_WIN_HEAD 2
+#define LBM_HDR_WIN_COUNT 3
+#define LBM_HDR_N_FREE_PATCH 4
+#define LBM_HDR_N_FREE_SPECIAL 5
+#define LBM_HDR_N_SPECIAL_PAGES 6
+#define LBM_HDR_SPECIAL_TOKENS 7
+#define LBM_HDR_N_MEMORY 8
+#define LBM_HDR_N_MEMORY_PAGES 9
+#define LBM_HDR_ERROR 10
+#define LBM_HDR_PLAN_KV_TOKENS 11
+#define LBM_HDR_PLAN_N_PAGES 12
+#define LBM_HDR_WORDS 16
+
+/* Geometry of one stream's cache; the same for every stream of a batch.
+ * Mirrors the constructor arguments of FlashInferKVCacheManager
+ * (flashinfer_cache.py:75-138) with the page size made a free parameter. */
+typedef struct lbm_cache_geom {
+  int32_t layout;             /* LBM_LAYOUT_*                                             */
+  int32_t tokens_per_frame;   /* specials first, then patches (flashinfer_cache.py:206)   */
+  int32_t num_special_tokens;
+  int32_t page_size;          /* tokens per page                                          */
+  int32_t scale_frames;       /* anchor frames, never evicted                             */
+  int32_t patch_pages;        /* recyclable page ids [0, patch_pages) of each stream      */
+  int32_t special_pages;      /* append-only ids after them (two_stream), else 0          */
+  int32_t memory_frames;      /* capacity of the compacted-frame list (frame_pages)       */
+  int32_t pages_per_stream;   /* id distance between streams (>= patch + special pages)   */
+} lbm_cache_geom;
+
+/* One stream's share of a lbm_tables_step call. */
+typedef struct lbm_step_op {
+  int32_t ops;              /* LBM_OP_* bits; 0 = leave this stream alone                  */
+  int32_t sliding_window;   /* EVICT: frames the window may keep                           */
+  int32_t keep_tokens;      /* EVICT, frame_pages: leading tokens kept per evicted frame   */
+  int32_t self_tokens;      /* PLAN: >0 appends the current frame's own K/V (read from the
+                               caller's tensors, never stored) after the cached tokens     */
+  int32_t q_begin;          /* first row of this stream in the batched q/k/v tensors       */
+  int32_t kv_row_begin;     /* PLAN: first entry of this stream in kv_rows                 */
+  int32_t expect_kv_tokens; /* PLAN: the host's count of visible tokens                    */
+  int32_t page_out_begin;   /* PLAN: first entry of this stream in kv_page_ids/_lens       */
+} lbm_step_op;
+
+/* One stream's share of an attention call (host memory). */
+typedef struct lbm_attn_stream {
+  int32_t q_begin;      /* first query row                                                 */
+  int32_t q_rows;       /* number of query rows                                            */
+  int32_t kv_row_begin; /* first entry in kv_rows                                          */
+  int32_t kv_tokens;    /* number of entries                                               */
+} lbm_attn_stream;
+
+int lbm_abi_version(void);
+const char* lbm_last_error(void);
+
+/* int32 words of device memory one stream's tables need; 0 if the geometry is invalid. */
+int64_t lbm_tables_words(const lbm_cache_geom* geom);
+
+/* Index-only table maintenance, one launch for all streams of a batch.  Replaces the host
+ * deque/list bookkeeping of FlashInferKVCacheManager: reset (flashinfer_cache.py:423-432),
+ * rollback_last_frame (:268-301), the allocation half of append_frame (:474-553),
+ * evict_frames / execute_deferred_eviction (:229-266), and build_visible_page_table +
+ * compute_last_page_len + the three table uploads before plan() (:385-400, :438-470).
+ *   tables        [n_streams * lbm_tables_words]           in/out
+ *   ops           host, n_streams entries
+ *   append_rows   APPEND: K row of every token of the new frame, -1 if the stream does not
+ *                 append (indexed q_begin + t); may be NULL without APPEND
+ *   kv_rows       PLAN: K row of every visible token; entries < 0 name row (-1 - e) of the
+ *                 caller's own k/v tensors; may be NULL without PLAN
+ *   kv_page_ids, kv_page_lens   PLAN: FlashInfer-style page table with a valid length per
+ *                 page (optional, NULL to skip) */
+int lbm_tables_step(int32_t* tables, const lbm_cache_geom* geom, int32_t n_streams,
+                    const lbm_step_op* ops, int32_t* append_rows, int32_t* kv_rows,
+                    int32_t* kv_page_ids, int32_t* kv_page_lens, void* stream);
+
+/* Expand a FlashInfer-style page table (any page order, any valid length per page) into
+ * the row table the attention kernel reads.  Stands in for the index half of
+ * BatchPrefillWithPagedKVCacheWrapper.plan (flashinfer_cache.py:402-414).
+ *   kv_indptr  host, n_streams + 1 offsets into kv_page_ids / kv_page_lens
+ *   kv_tokens  host, n_streams visible token counts (sum of the stream's page lens)
+ *   kv_row_begin host, n_streams offsets into kv_rows */
+int lbm_rows_from_pages(const int32_t* kv_page_ids, const int32_t* kv_page_lens,
+                        const int32_t* kv_indptr, const int32_t* kv_tokens,
+                        const int32_t* kv_row_begin, int32_t n_streams, int32_t page_size,
+                        int32_t* kv_rows, void* stream);
+
+/* Keyframe-gated paged append: scatter one batch of new K/V rows into the pool.  Replaces
+ * the slice assignments and dtype casts of append_frame (flashinfer_cache.py:215-218,
+ * :504-505, :548-549).  Rows whose append_rows entry is negative are not written. */
+int lbm_kv_append(const void* k, const void* v, int32_t src_dtype, void* pool,
+                  int32_t pool_dtype, const int32_t* append_rows, int32_t n_tokens,
+                  int32_t num_heads, int32_t head_dim, int32_t page_size, void* stream);
+
+/* Bytes of workspace lbm_attn_run needs for this batch (split-KV partial results). */
+size_t lbm_attn_workspace_bytes(const lbm_attn_stream* streams, int32_t n_streams,
+                                int32_t num_heads, int32_t head_dim);
+
+/* Ragged gather + softmax(q k^T * sm_scale) v over the rows kv_rows names, non-causal, MHA.
+ * Replaces BatchPrefillWithPagedKVCacheWrapper.run (flashinfer_cache.py:418-421) and the
+ * gather + F.scaled_dot_product_attention bridge (:324-347, :372-383).
+ *   q, out         [rows][num_heads][head_dim], dtype = pool dtype
+ *   self_k, self_v the caller's K/V of the current frames, same indexing as q (only read
+ *                  for negative kv_rows entries; may be NULL otherwise) */
+int lbm_attn_run(const void* q, const void* pool, void* out, const void* self_k,
+                 const void* self_v, const int32_t* kv_rows, const lbm_attn_stream* streams,
+                 int32_t n_streams, int32_t num_heads, int32_t head_dim, int32_t page_size,
+                 int32_t dtype, float sm_scale, void* workspace, size_t workspace_bytes,
+                 void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* LBM_PAGED_ATTN_H */

@@ -1,0 +1,128 @@
+// extern "C" entry points: argument checks, then the launch helpers of the kernel files.
+#include <hip/hip_runtime.h>
+#include <cstdarg>
+#include <cstdio>
+#include "lbm_internal.h"
+#include "tables_logic.h"
+
+namespace {
+thread_local char g_last_error[512] = "";
+}
+
+int lbm_fail(int code, const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_last_error, sizeof(g_last_error), fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+int lbm_check_launch(const char* kernel_name) {
+  const hipError_t e = hipGetLastError();
+  if (e == hipSuccess) return LBM_OK;
+  return lbm_fail(LBM_ERR_HIP, "%s: %s", kernel_name, hipGetErrorString(e));
+}
+
+extern "C" {
+
+int lbm_abi_version(void) { return LBM_ABI_VERSION; }
+
+const char* lbm_last_error(void) { return g_last_error; }
+
+int64_t lbm_tables_words(const lbm_cache_geom* geom) {
+  if (!geom || !lbm_geom_valid(*geom)) return 0;
+  return lbm_tables_layout(*geom).words;
+}
+
+int lbm_tables_step(int32_t* tables, const lbm_cache_geom* geom, int32_t n_streams,
+                    const lbm_step_op* ops, int32_t* append_rows, int32_t* kv_rows,
+                    int32_t* kv_page_ids, int32_t* kv_page_lens, void* stream) {
+  if (!tables || !geom || !ops) return lbm_fail(LBM_ERR_INVALID, "lbm_tables_step: null tables, geom or ops");
+  if (!lbm_geom_valid(*geom)) return lbm_fail(LBM_ERR_INVALID, "lbm_tables_step: invalid cache geometry");
+  if (n_streams < 1 || n_streams > LBM_MAX_STREAMS)
+    return lbm_fail(LBM_ERR_INVALID, "lbm_tables_step: n_streams %d outside [1, %d]", n_streams, LBM_MAX_STREAMS);
+  for (int i = 0; i < n_streams; ++i) {
+    const lbm_step_op& o = ops[i];
+    if (o.ops & ~(LBM_OP_RESET | LBM_OP_ROLLBACK | LBM_OP_APPEND | LBM_OP_EVICT | LBM_OP_PLAN))
+      return lbm_fail(LBM_ERR_INVALID, "lbm_tables_step: stream %d has unknown op bits 0x%x", i, o.ops);
+    if ((o.ops & LBM_OP_PLAN) && !kv_rows && !(kv_page_ids && kv_page_lens))
+      return lbm_fail(LBM_ERR_INVALID, "lbm_tables_step: PLAN needs kv_rows or the page table outputs");
+    if ((o.ops & LBM_OP_PLAN) && (o.expect_kv_tokens < 0 || o.kv_row_begin < 0 || o.page_out_begin < 0))
+      return lbm_fail(LBM_ERR_INVALID, "lbm_tables_step: stream %d has a negative plan offset or count", i);
+    if ((o.ops & LBM_OP_EVICT) && o.sliding_window < 0)
+      return lbm_fail(LBM_ERR_INVALID, "lbm_tables_step: stream %d has a negative sliding_window", i);
+    if (o.q_begin < 0) return lbm_fail(LBM_ERR_INVALID, "lbm_tables_step: stream %d has a negative q_begin", i);
+  }
+  return lbm_launch_tables(tables, *geom, n_streams, ops, append_rows, kv_rows, kv_page_ids,
+                           kv_page_lens, (hipStream_t)stream);
+}
+
+int lbm_rows_from_pages(const int32_t* kv_page_ids, const int32_t* kv_page_lens,
+                        const int32_t* kv_indptr, const int32_t* kv_tokens,
+                        const int32_t* kv_row_begin, int32_t n_streams, int32_t page_size,
+                        int32_t* kv_rows, void* stream) {
+  if (!kv_page_ids || !kv_page_lens || !kv_indptr || !kv_tokens || !kv_row_begin || !kv_rows)
+    return lbm_fail(LBM_ERR_INVALID, "lbm_rows_from_pages: null argument");
+  if (n_streams < 1 || n_streams > LBM_MAX_STREAMS || page_size <= 0)
+    return lbm_fail(LBM_ERR_INVALID, "lbm_rows_from_pages: bad n_streams %d or page_size %d", n_streams, page_size);
+  for (int i = 0; i < n_streams; ++i)
+    if (kv_indptr[i + 1] < kv_indptr[i] || kv_tokens[i] < 0 || kv_row_begin[i] < 0)
+      return lbm_fail(LBM_ERR_INVALID, "lbm_rows_from_pages: stream %d has a decreasing indptr or a negative count", i);
+  return lbm_launch_rows_from_pages(kv_page_ids, kv_page_lens, kv_indptr, kv_tokens, kv_row_begin,
+                                    n_streams, page_size, kv_rows, (hipStream_t)stream);
+}
+
+int lbm_kv_append(const void* k, const void* v, int32_t src_dtype, void* pool, int32_t pool_dtype,
+                  const int32_t* append_rows, int32_t n_tokens, int32_t num_heads,
+                  int32_t head_dim, int32_t page_size, void* stream) {
+  if (n_tokens == 0) return LBM_OK;
+  if (!k || !v || !pool || !append_rows) return lbm_fail(LBM_ERR_INVALID, "lbm_kv_append: null argument");
+  if (n_tokens < 0 || num_heads <= 0 || head_dim <= 0 || page_size <= 0)
+    return lbm_fail(LBM_ERR_INVALID, "lbm_kv_append: non-positive size");
+  if ((src_dtype != LBM_DTYPE_BF16 && src_dtype != LBM_DTYPE_F32) ||
+      (pool_dtype != LBM_DTYPE_BF16 && pool_dtype != LBM_DTYPE_F32))
+    return lbm_fail(LBM_ERR_INVALID, "lbm_kv_append: unknown dtype");
+  if ((num_heads * head_dim) % 8 != 0)
+    return lbm_fail(LBM_ERR_UNSUPPORTED, "lbm_kv_append: num_heads * head_dim must be a multiple of 8");
+  return lbm_launch_append(k, v, src_dtype, pool, pool_dtype, append_rows, n_tokens, num_heads,
+                           head_dim, page_size, (hipStream_t)stream);
+}
+
+static int lbm_check_attn_streams(const lbm_attn_stream* s, int n, const char* who) {
+  if (!s) return lbm_fail(LBM_ERR_INVALID, "%s: null streams", who);
+  if (n < 1 || n > LBM_MAX_STREAMS) return lbm_fail(LBM_ERR_INVALID, "%s: n_streams %d outside [1, %d]", who, n, LBM_MAX_STREAMS);
+  for (int i = 0; i < n; ++i)
+    if (s[i].q_begin < 0 || s[i].q_rows < 0 || s[i].kv_row_begin < 0 || s[i].kv_tokens < 0)
+      return lbm_fail(LBM_ERR_INVALID, "%s: stream %d has a negative field", who, i);
+  return LBM_OK;
+}
+
+size_t lbm_attn_workspace_bytes(const lbm_attn_stream* streams, int32_t n_streams,
+                                int32_t num_heads, int32_t head_dim) {
+  if (lbm_check_attn_streams(streams, n_streams, "lbm_attn_workspace_bytes") != LBM_OK) return 0;
+  if (num_heads <= 0 || head_dim <= 0) return 0;
+  LbmAttnSchedule sch;
+  lbm_attn_schedule(streams, n_streams, num_heads, &sch);
+  return lbm_attn_schedule_bytes(sch, num_heads, head_dim);
+}
+
+int lbm_attn_run(const void* q, const void* pool, void* out, const void* self_k,
+                 const void* self_v, const int32_t* kv_rows, const lbm_attn_stream* streams,
+                 int32_t n_streams, int32_t num_heads, int32_t head_dim, int32_t page_size,
+                 int32_t dtype, float sm_scale, void* workspace, size_t workspace_bytes,
+                 void* stream) {
+  int rc = lbm_check_attn_streams(streams, n_streams, "lbm_attn_run");
+  if (rc != LBM_OK) return rc;
+  if (!q || !pool || !out || !kv_rows) return lbm_fail(LBM_ERR_INVALID, "lbm_attn_run: null q, pool, out or kv_rows");
+  if (num_heads <= 0 || head_dim <= 0 || page_size <= 0) return lbm_fail(LBM_ERR_INVALID, "lbm_attn_run: non-positive size");
+  if ((self_k == nullptr) != (self_v == nullptr)) return lbm_fail(LBM_ERR_INVALID, "lbm_attn_run: self_k and self_v go together");
+  LbmAttnSchedule sch;
+  lbm_attn_schedule(streams, n_streams, num_heads, &sch);
+  const size_t need = lbm_attn_schedule_bytes(sch, num_heads, head_dim);
+  if (need > 0 && (!workspace || workspace_bytes < need))
+    return lbm_fail(LBM_ERR_WORKSPACE, "lbm_attn_run: workspace of %zu bytes, %zu needed", workspace_bytes, need);
+  return lbm_launch_attention(q, pool, out, self_k, self_v, kv_rows, sch, num_heads, head_dim,
+                              page_size, dtype, sm_scale, workspace, (hipStream_t)stream);
+}
+
+}  // extern "C"

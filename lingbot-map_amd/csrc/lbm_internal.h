@@ -1,0 +1,48 @@
+// Declarations shared by the translation units of the library (not part of the C ABI).
+#ifndef LBM_INTERNAL_H
+#define LBM_INTERNAL_H
+
+#include <hip/hip_runtime.h>
+#include <stddef.h>
+#include <stdint.h>
+#include "../../include/lbm_paged_attn.h"
+
+// Records `msg` as the calling thread's last error and returns `code`.
+int lbm_fail(int code, const char* fmt, ...);
+// hipGetLastError() after a launch; LBM_OK or LBM_ERR_HIP with the kernel's name recorded.
+int lbm_check_launch(const char* kernel_name);
+
+int lbm_launch_tables(int32_t* tables, const lbm_cache_geom& g, int n_streams,
+                      const lbm_step_op* ops, int32_t* append_rows, int32_t* kv_rows,
+                      int32_t* page_ids, int32_t* page_lens, hipStream_t stream);
+int lbm_launch_rows_from_pages(const int32_t* page_ids, const int32_t* page_lens,
+                               const int32_t* indptr, const int32_t* kv_tokens,
+                               const int32_t* row_begin, int n_streams, int page_size,
+                               int32_t* kv_rows, hipStream_t stream);
+int lbm_launch_append(const void* k, const void* v, int src_dtype, void* pool, int pool_dtype,
+                      const int32_t* append_rows, int n_tokens, int num_heads, int head_dim,
+                      int page_size, hipStream_t stream);
+
+// Split-KV schedule of one attention call, computed on the host from token counts only.
+struct LbmAttnStreamPlan {
+  int32_t q_begin, q_rows, kv_row_begin, kv_tokens;
+  int32_t n_qtiles, n_splits, tiles_per_split;
+  int32_t wg_begin;    // first workgroup of this stream
+  int32_t part_begin;  // first partial-result row (unit: q row of one split) in the workspace
+};
+struct LbmAttnSchedule {
+  int32_t n_streams;
+  int32_t total_wgs;
+  int64_t part_rows;   // rows of partial results over all streams (0 when nothing is split)
+  LbmAttnStreamPlan s[LBM_MAX_STREAMS];
+};
+void lbm_attn_schedule(const lbm_attn_stream* streams, int n_streams, int num_heads,
+                       LbmAttnSchedule* out);
+size_t lbm_attn_schedule_bytes(const LbmAttnSchedule& sch, int num_heads, int head_dim);
+
+int lbm_launch_attention(const void* q, const void* pool, void* out, const void* self_k,
+                         const void* self_v, const int32_t* kv_rows, const LbmAttnSchedule& sch,
+                         int num_heads, int head_dim, int page_size, int dtype, float sm_scale,
+                         void* workspace, hipStream_t stream);
+
+#endif  // LBM_INTERNAL_H

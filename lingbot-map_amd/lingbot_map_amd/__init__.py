@@ -1,0 +1,11 @@
+"""MI355X-native streaming paged-KV attention for LingBot-Map's global blocks.
+
+``HipPagedKVCacheManager`` stands in for the reference's ``FlashInferKVCacheManager``
+(lingbot_map/layers/flashinfer_cache.py:55); ``HipPagedBlock`` for its ``FlashInferBlock``
+(lingbot_map/layers/block.py:151).  Importing this package loads the HIP library and raises
+if it has not been built: there is no CPU path.
+"""
+from . import _native  # noqa: F401  (loads the library, fails loudly when missing)
+from .manager import HipPagedKVCacheManager
+
+__all__ = ["HipPagedKVCacheManager"]

@@ -1,0 +1,84 @@
+"""ctypes binding of the C ABI declared in include/lbm_paged_attn.h.
+
+There is no CPU fallback: importing this module without the built library raises."""
+from __future__ import annotations
+
+import ctypes as C
+import os
+
+from .build import LIB_PATH
+
+OK, ERR_INVALID, ERR_UNSUPPORTED, ERR_WORKSPACE, ERR_HIP = 0, 1, 2, 3, 4
+DTYPE_BF16, DTYPE_F32 = 0, 1
+LAYOUT_TWO_STREAM, LAYOUT_FRAME_PAGES = 0, 1
+MAX_STREAMS = 16
+OP_RESET, OP_ROLLBACK, OP_APPEND, OP_EVICT, OP_PLAN = 1, 2, 4, 8, 16
+TERR_NAMES = {1: "patch page pool exhausted", 2: "special page pool exhausted", 4: "window ring full",
+              8: "trajectory memory full", 16: "rollback underflow", 32: "visible token count mismatch"}
+HDR = {"frame_count": 0, "n_anchor": 1, "win_head": 2, "win_count": 3, "n_free_patch": 4,
+       "n_free_special": 5, "n_special_pages": 6, "special_tokens": 7, "n_memory": 8,
+       "n_memory_pages": 9, "error": 10, "plan_kv_tokens": 11, "plan_n_pages": 12}
+HDR_WORDS = 16
+ABI_VERSION = 1
+
+
+class CacheGeom(C.Structure):
+    _fields_ = [(n, C.c_int32) for n in (
+        "layout", "tokens_per_frame", "num_special_tokens", "page_size", "scale_frames",
+        "patch_pages", "special_pages", "memory_frames", "pages_per_stream")]
+
+
+class StepOp(C.Structure):
+    _fields_ = [(n, C.c_int32) for n in (
+        "ops", "sliding_window", "keep_tokens", "self_tokens", "q_begin", "kv_row_begin",
+        "expect_kv_tokens", "page_out_begin")]
+
+
+class AttnStream(C.Structure):
+    _fields_ = [(n, C.c_int32) for n in ("q_begin", "q_rows", "kv_row_begin", "kv_tokens")]
+
+
+SYMBOLS = ("lbm_abi_version", "lbm_last_error", "lbm_tables_words", "lbm_tables_step",
+           "lbm_rows_from_pages", "lbm_kv_append", "lbm_attn_workspace_bytes", "lbm_attn_run")
+
+
+def _load():
+    if not os.path.exists(LIB_PATH):
+        raise RuntimeError(
+            f"HIP library {LIB_PATH} is not built; run `python -c 'import __graft_entry__ as g; g.build()'` "
+            "(there is no CPU fallback for this path)")
+    lib = C.CDLL(LIB_PATH)
+    p, i32, vp = C.POINTER, C.c_int32, C.c_void_p
+    lib.lbm_abi_version.restype = C.c_int
+    lib.lbm_last_error.restype = C.c_char_p
+    lib.lbm_tables_words.restype = C.c_int64
+    lib.lbm_tables_words.argtypes = [p(CacheGeom)]
+    lib.lbm_tables_step.restype = C.c_int
+    lib.lbm_tables_step.argtypes = [vp, p(CacheGeom), i32, p(StepOp), vp, vp, vp, vp, vp]
+    lib.lbm_rows_from_pages.restype = C.c_int
+    lib.lbm_rows_from_pages.argtypes = [vp, vp, p(i32), p(i32), p(i32), i32, i32, vp, vp]
+    lib.lbm_kv_append.restype = C.c_int
+    lib.lbm_kv_append.argtypes = [vp, vp, i32, vp, i32, vp, i32, i32, i32, i32, vp]
+    lib.lbm_attn_workspace_bytes.restype = C.c_size_t
+    lib.lbm_attn_workspace_bytes.argtypes = [p(AttnStream), i32, i32, i32]
+    lib.lbm_attn_run.restype = C.c_int
+    lib.lbm_attn_run.argtypes = [vp, vp, vp, vp, vp, vp, p(AttnStream), i32, i32, i32, i32, i32,
+                                 C.c_float, vp, C.c_size_t, vp]
+    if lib.lbm_abi_version() != ABI_VERSION:
+        raise RuntimeError(f"{LIB_PATH}: ABI version {lib.lbm_abi_version()}, binding expects {ABI_VERSION}")
+    return lib
+
+
+lib = _load()
+
+
+class LbmError(RuntimeError):
+    pass
+
+
+def check(rc: int) -> None:
+    if rc != OK:
+        msg = lib.lbm_last_error().decode("utf-8", "replace")
+        if rc == ERR_INVALID:
+            raise ValueError(msg)
+        raise LbmError(f"lbm error {rc}: {msg}")

@@ -1,0 +1,177 @@
+"""GPU parity of the three HIP kernels, called through the C ABI, against the CPU oracle.
+
+Tolerances (attention): bf16 max-abs <= 2e-2 and mean-abs <= 2e-3 against fp32 SDPA on the
+same bf16 inputs.  Page tables, append rows and pool contents: bit-exact."""
+import ctypes as C
+import math
+
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+BF16_MAX_ABS, BF16_MEAN_ABS = 2e-2, 2e-3
+
+
+def _native():
+    from lingbot_map_amd import _native as N
+    return N
+
+
+def ptr(t):
+    return C.c_void_p(t.data_ptr())
+
+
+def run_attention(q, pool, kv_rows, streams, page_size, self_k=None, self_v=None):
+    """q [rows,H,D]; streams: list of (q_begin, q_rows, kv_row_begin, kv_tokens)."""
+    N = _native()
+    H, D = q.shape[1], q.shape[2]
+    arr = (N.AttnStream * len(streams))(*[N.AttnStream(*s) for s in streams])
+    need = N.lib.lbm_attn_workspace_bytes(arr, len(streams), H, D)
+    ws = torch.empty(max(int(need), 16), dtype=torch.uint8, device=q.device)
+    out = torch.full_like(q, float("nan"))
+    N.check(N.lib.lbm_attn_run(ptr(q), ptr(pool), ptr(out), ptr(self_k) if self_k is not None else None,
+                               ptr(self_v) if self_v is not None else None, ptr(kv_rows), arr, len(streams), H, D,
+                               page_size, N.DTYPE_BF16, 1.0 / math.sqrt(D), ptr(ws), ws.numel(), None))
+    torch.cuda.synchronize()
+    return out
+
+
+def rows_from_pages(page_ids, page_lens, page_size, dev):
+    N = _native()
+    n_tok = int(sum(page_lens))
+    ids = torch.tensor(page_ids, dtype=torch.int32, device=dev)
+    lens = torch.tensor(page_lens, dtype=torch.int32, device=dev)
+    rows = torch.full((n_tok + 8,), -12345, dtype=torch.int32, device=dev)
+    i32 = C.c_int32
+    N.check(N.lib.lbm_rows_from_pages(ptr(ids), ptr(lens), (i32 * 2)(0, len(page_ids)), (i32 * 1)(n_tok),
+                                      (i32 * 1)(0), 1, page_size, ptr(rows), None))
+    torch.cuda.synchronize()
+    return rows, n_tok
+
+
+def check_bf16(out, ref):
+    err = (out.float() - ref.float()).abs()
+    assert torch.isfinite(out.float()).all()
+    assert err.max().item() <= BF16_MAX_ABS, f"max-abs {err.max().item()}"
+    assert err.mean().item() <= BF16_MEAN_ABS, f"mean-abs {err.mean().item()}"
+
+
+@pytest.mark.parametrize("tq,n_pages,page_size,H", [(7, 3, 4, 2), (64, 9, 16, 16), (300, 70, 16, 4), (1004, 140, 16, 16)])
+def test_attention_matches_oracle_ragged_pages(tq, n_pages, page_size, H):
+    from oracle.sdpa_cache import gather_paged, sdpa_nhd
+    dev = torch.device("cuda:0")
+    g = torch.Generator().manual_seed(tq * 31 + n_pages)
+    D = 64
+    total_pages = n_pages + 5
+    pool = torch.randn(total_pages, 2, page_size, H, D, generator=g).to(torch.bfloat16)
+    q = torch.randn(tq, H, D, generator=g).to(torch.bfloat16)
+    page_ids = torch.randperm(total_pages, generator=g)[:n_pages].tolist()       # shuffled, non-contiguous
+    page_lens = torch.randint(1, page_size + 1, (n_pages,), generator=g).tolist()  # partial pages anywhere
+    kk, vv = gather_paged(pool, page_ids, page_lens)
+    ref = sdpa_nhd(q, kk, vv)
+    rows, n_tok = rows_from_pages(page_ids, page_lens, page_size, dev)
+    expect_rows = [p * 2 * page_size + s for p, n in zip(page_ids, page_lens) for s in range(n)]
+    assert rows[:n_tok].cpu().tolist() == expect_rows
+    assert (rows[n_tok:] == -12345).all()
+    out = run_attention(q.to(dev), pool.to(dev), rows, [(0, tq, 0, n_tok)], page_size)
+    check_bf16(out.cpu(), ref)
+
+
+def test_attention_config2_shape_split_kv():
+    """1004 queries x 17,068 KV tokens, 16 heads: the shape the headline metric is quoted on."""
+    from oracle.sdpa_cache import sdpa_nhd
+    dev = torch.device("cuda:0")
+    g = torch.Generator().manual_seed(1)
+    T, H, D, S, frames = 1004, 16, 64, 16, 17
+    ppf = math.ceil(T / S)
+    pool = torch.zeros(frames * ppf + 3, 2, S, H, D, dtype=torch.bfloat16)
+    perm = torch.randperm(pool.shape[0], generator=g)[: frames * ppf].tolist()
+    ks, vs, ids, lens = [], [], [], []
+    for f in range(frames):
+        k = torch.randn(T, H, D, generator=g).to(torch.bfloat16)
+        v = torch.randn(T, H, D, generator=g).to(torch.bfloat16)
+        ks.append(k); vs.append(v)
+        for j in range(ppf):
+            p = perm[f * ppf + j]
+            n = min(S, T - j * S)
+            pool[p, 0, :n] = k[j * S: j * S + n]
+            pool[p, 1, :n] = v[j * S: j * S + n]
+            ids.append(p); lens.append(n)
+    q = torch.randn(T, H, D, generator=g).to(torch.bfloat16)
+    ref = sdpa_nhd(q, torch.cat(ks), torch.cat(vs))
+    rows, n_tok = rows_from_pages(ids, lens, S, dev)
+    assert n_tok == 17068
+    out = run_attention(q.to(dev), pool.to(dev), rows, [(0, T, 0, n_tok)], S)
+    check_bf16(out.cpu(), ref)
+
+
+def test_attention_read_only_tail_and_two_streams():
+    """Negative row entries read the caller's own K/V (non-keyframe); two ragged streams in one launch."""
+    from oracle.sdpa_cache import sdpa_nhd
+    dev = torch.device("cuda:0")
+    g = torch.Generator().manual_seed(5)
+    T, H, D, S = 40, 4, 64, 16
+    pool = torch.randn(12, 2, S, H, D, generator=g).to(torch.bfloat16)
+    q = torch.randn(2 * T, H, D, generator=g).to(torch.bfloat16)
+    sk = torch.randn(2 * T, H, D, generator=g).to(torch.bfloat16)
+    sv = torch.randn(2 * T, H, D, generator=g).to(torch.bfloat16)
+    flat_k = pool[:, 0].reshape(-1, H, D)
+    flat_v = pool[:, 1].reshape(-1, H, D)
+    slots0 = torch.randperm(12 * S, generator=g)[:70].tolist()
+    slots1 = torch.randperm(12 * S, generator=g)[:129].tolist()
+    to_row = lambda s: (s // S) * 2 * S + s % S
+    rows0 = [to_row(s) for s in slots0]
+    rows1 = [to_row(s) for s in slots1] + [-1 - (T + t) for t in range(T)]   # stream 1 also sees its own frame
+    rows = torch.tensor(rows0 + [0] * 3 + rows1, dtype=torch.int32, device=dev)
+    out = run_attention(q.to(dev), pool.to(dev), rows, [(0, T, 0, len(rows0)), (T, T, len(rows0) + 3, len(rows1))],
+                        S, sk.to(dev), sv.to(dev)).cpu()
+    ref0 = sdpa_nhd(q[:T], flat_k[slots0], flat_v[slots0])
+    ref1 = sdpa_nhd(q[T:], torch.cat([flat_k[slots1], sk[T:]]), torch.cat([flat_v[slots1], sv[T:]]))
+    check_bf16(out[:T], ref0)
+    check_bf16(out[T:], ref1)
+
+
+def test_attention_closed_forms():
+    dev = torch.device("cuda:0")
+    H, D, S = 2, 64, 16
+    g = torch.Generator().manual_seed(9)
+    q = torch.randn(33, H, D, generator=g).to(torch.bfloat16).to(dev)
+    pool = torch.randn(4, 2, S, H, D, generator=g).to(torch.bfloat16).to(dev)
+    # one KV token: the output is that token's V
+    rows = torch.tensor([1 * 2 * S + 5], dtype=torch.int32, device=dev)
+    out = run_attention(q, pool, rows, [(0, 33, 0, 1)], S)
+    assert torch.equal(out, pool[1, 1, 5].expand(33, H, D))
+    # identical keys: the output is the mean of V
+    pool[2, 0] = pool[2, 0, 0]
+    rows = torch.arange(2 * 2 * S, 2 * 2 * S + S, dtype=torch.int32, device=dev)
+    out = run_attention(q, pool, rows, [(0, 33, 0, S)], S)
+    mean = pool[2, 1].float().mean(0)
+    assert (out.float() - mean).abs().max().item() <= 1e-2
+
+
+@pytest.mark.parametrize("src,dst", [(torch.bfloat16, torch.bfloat16), (torch.float32, torch.bfloat16),
+                                     (torch.float32, torch.float32), (torch.bfloat16, torch.float32)])
+def test_append_is_exact_and_gated(src, dst):
+    N = _native()
+    dev = torch.device("cuda:0")
+    g = torch.Generator().manual_seed(3)
+    T, H, D, S, pages = 37, 16, 64, 16, 9
+    k = torch.randn(T, H, D, generator=g).to(src)
+    v = torch.randn(T, H, D, generator=g).to(src)
+    slots = torch.randperm(pages * S, generator=g)[:T]
+    rows = ((slots // S) * 2 * S + slots % S).to(torch.int32)
+    rows[5] = -1
+    rows[20] = -1
+    pool = torch.full((pages, 2, S, H, D), 7.0, dtype=dst, device=dev)
+    code = {torch.bfloat16: N.DTYPE_BF16, torch.float32: N.DTYPE_F32}
+    kd, vd, rd = k.to(dev), v.to(dev), rows.to(dev)
+    N.check(N.lib.lbm_kv_append(ptr(kd), ptr(vd), code[src], ptr(pool), code[dst], ptr(rd), T, H, D, S, None))
+    torch.cuda.synchronize()
+    expect = torch.full((pages, 2, S, H, D), 7.0, dtype=dst)
+    for t in range(T):
+        if rows[t] >= 0:
+            p, s = int(slots[t]) // S, int(slots[t]) % S
+            expect[p, 0, s] = k[t].to(dst)
+            expect[p, 1, s] = v[t].to(dst)
+    assert torch.equal(pool.cpu(), expect)

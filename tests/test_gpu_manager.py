@@ -1,0 +1,161 @@
+"""The drop-in manager on the GPU against the oracle: device page tables bit-exact after
+every operation, pool contents exact, attention within the bf16 tolerance."""
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+BF16_MAX_ABS, BF16_MEAN_ABS = 2e-2, 2e-3
+
+
+def make(layout, page_size, T=7, n_sp=3, scale=1, window=2, max_total=6, H=2, blocks=2, **kw):
+    from lingbot_map_amd import HipPagedKVCacheManager
+    return HipPagedKVCacheManager(blocks, scale + window + 16, T, H, 64, torch.bfloat16, torch.device("cuda:0"),
+                                  num_special_tokens=n_sp, scale_frames=scale, sliding_window=window,
+                                  max_total_frames=max_total, page_size=page_size, layout=layout, **kw)
+
+
+def frame(T, H, g):
+    return tuple(torch.randn(T, H, 64, generator=g).to(torch.bfloat16) for _ in range(3))
+
+
+def test_six_frame_trace_on_device():
+    """Hand-derived ids for tokens_per_frame 7 (see tests/test_oracle_policy.py)."""
+    m = make("two_stream", None)
+    assert m.page_size == 4 and m.max_patch_pages == 19 and m.max_num_pages == 40
+    g = torch.Generator().manual_seed(0)
+    visible = [[18, 39], [18, 17, 39, 38], [18, 17, 16, 39, 38, 37], [18, 16, 15, 39, 38, 37],
+               [18, 15, 17, 39, 38, 37, 36], [18, 17, 16, 39, 38, 37, 36, 35]]
+    last = [3, 2, 1, 4, 3, 2]
+    for vis, ll in zip(visible, last):
+        q, k, v = frame(7, 2, g)
+        m.append_frame(0, k.cuda(), v.cuda())
+        m.evict_frames(0, 1, 2)
+        assert m.build_visible_page_table(0) == vis
+        assert m.compute_last_page_len(0) == ll
+        assert m.device_header()["error"] == 0
+    assert m.get_cache_stats() == {"frame_count": 6, "scale_pages": 1, "live_pages": 2, "free_pages": 16,
+                                   "special_tokens": 18}
+    # non-keyframe probe: append, look, roll back -> bit-identical tables
+    before = m._tables.clone()
+    m._defer_eviction = True
+    q, k, v = frame(7, 2, g)
+    m.append_frame(0, k.cuda(), v.cuda())
+    m.evict_frames(0, 1, 2)
+    assert m.build_visible_page_table(0) == [18, 17, 16, 15, 39, 38, 37, 36, 35, 34]
+    assert m.compute_last_page_len(0) == 1
+    m.rollback_last_frame(0)
+    m._defer_eviction = False
+    hdr_plan = slice(11, 13)
+    a, b = m._tables.clone(), before
+    a[..., hdr_plan] = 0; b[..., hdr_plan] = 0
+    n_free = m.device_header()["n_free_patch"]
+    assert torch.equal(a[0, 0, :16 + n_free], b[0, 0, :16 + n_free])
+    assert m.build_visible_page_table(0) == visible[-1]
+    m.reset()
+    assert m.frame_count == [0, 0] and m.device_header()["frame_count"] == 0
+
+
+def test_reference_sanity_check_figures_on_device():
+    # lingbot_map/layers/flashinfer_cache.py:577-656, run the reference's way: block by block
+    m = make("two_stream", None, T=262, n_sp=6, scale=8, window=64, max_total=200, H=16, per_block_tables=True)
+    g = torch.Generator().manual_seed(0)
+    for block in range(2):
+        for t in range(100):
+            _, k, v = frame(262, 16, g)
+            m.append_frame(block, k.cuda(), v.cuda())
+            m.evict_frames(block, scale_frames=8, sliding_window=64)
+        st = m.get_cache_stats(block)
+        assert st["scale_pages"] == 8 and st["live_pages"] == 64 and st["special_tokens"] == 600
+        vis = m.build_visible_page_table(block)
+        assert len(vis) == 8 + 64 + 3
+        assert all(p < m.max_patch_pages for p in vis[:72]) and all(p >= m.max_patch_pages for p in vis[72:])
+        assert m.compute_last_page_len(block) == 88
+        assert m.device_header(block)["error"] == 0
+    q0, q1 = frame(262, 16, g)[0].cuda(), frame(262, 16, g)[0].cuda()
+    assert m.compute_attention(0, q0).shape == (262, 16, 64)
+    assert m.compute_attention(1, q1).shape == (262, 16, 64)
+    m.reset()
+    assert m.frame_count[0] == 0
+
+
+def test_error_conventions():
+    m = make("two_stream", None)
+    q = torch.zeros(7, 2, 64, dtype=torch.bfloat16, device="cuda")
+    assert torch.equal(m.compute_attention(0, q), torch.zeros_like(q))   # nothing cached -> zeros
+    with pytest.raises(AssertionError, match="cannot rollback"):
+        m.rollback_last_frame(0)
+    m._defer_eviction = True
+    for _ in range(19):
+        m.append_frame(0, q, q)
+    with pytest.raises(AssertionError, match="patch page pool exhausted"):
+        m.append_frame(0, q, q)
+    assert m.device_header()["error"] == 0     # the host refused before the device saw it
+    with pytest.raises(AssertionError):
+        m.append_frame(0, q[:5], q[:5])
+
+
+@pytest.mark.parametrize("layout,page_size", [("two_stream", None), ("two_stream", 16), ("frame_pages", 16)])
+@pytest.mark.parametrize("interval,native_tail", [(1, False), (3, False), (3, True)])
+def test_stream_against_oracle(layout, page_size, interval, native_tail):
+    """40 frames, 3 blocks sharing one table set: ids, pool and outputs against the oracle."""
+    from oracle.page_policy import PagePolicy, is_keyframe
+    from oracle.sdpa_cache import PagedStreamOracle
+    T, n_sp, scale, window, H, blocks = 53, 5, 2, 3, 4, 3
+    m = make(layout, page_size, T=T, n_sp=n_sp, scale=scale, window=window, max_total=64, H=H, blocks=blocks)
+    pol = [PagePolicy(T, n_sp, page_size, scale, window, 64, layout=layout) for _ in range(blocks)]
+    orc = [PagedStreamOracle(p, H, 64, torch.bfloat16) for p in pol]
+    g = torch.Generator().manual_seed(11)
+    for f in range(40):
+        kf = is_keyframe(f, scale, interval)
+        for b in range(blocks):
+            q, k, v = frame(T, H, g)
+            ref = orc[b].step(q, k, v, keyframe=kf)
+            qd, kd, vd = q.cuda(), k.cuda(), v.cuda()
+            if kf:
+                m.append_frame(b, kd, vd)
+                m.evict_frames(b, scale, window)
+                out = m.compute_attention(b, qd)
+            elif native_tail:
+                out = m.compute_attention(b, qd, kd, vd)
+            else:   # the reference block's non-keyframe sequence (block.py:257-263)
+                prev = m._defer_eviction
+                m._defer_eviction = True
+                m.append_frame(b, kd, vd)
+                out = m.compute_attention(b, qd)
+                m.rollback_last_frame(b)
+                m._defer_eviction = prev
+            err = (out.float().cpu() - ref.float()).abs()
+            assert err.max().item() <= BF16_MAX_ABS and err.mean().item() <= BF16_MEAN_ABS, (f, b, err.max().item())
+        assert m.build_visible_page_table(0) == pol[0].build_visible_page_table(), f"frame {f}"
+        assert m.build_visible_page_lens(0) == pol[0].build_visible_page_lens()
+        assert m.device_header()["error"] == 0
+        st = m.get_cache_stats(0)
+        assert st == pol[0].get_cache_stats()
+    # every live page holds exactly what the oracle's pool holds
+    for b in range(blocks):
+        ids, lens = pol[b].build_visible_page_table(), pol[b].build_visible_page_lens()
+        dev_pool = m.kv_caches[b].cpu()
+        for p, n in zip(ids, lens):
+            assert torch.equal(dev_pool[p, :, :n], orc[b].pool[p, :, :n])
+
+
+def test_fused_step_matches_method_by_method():
+    from oracle.page_policy import is_keyframe
+    T, n_sp, scale, window, H = 53, 5, 1, 4, 4
+    a = make("frame_pages", 16, T=T, n_sp=n_sp, scale=scale, window=window, max_total=64, H=H, blocks=2)
+    b = make("frame_pages", 16, T=T, n_sp=n_sp, scale=scale, window=window, max_total=64, H=H, blocks=2)
+    g = torch.Generator().manual_seed(21)
+    for f in range(30):
+        kf = is_keyframe(f, scale, 4)
+        for blk in range(2):
+            q, k, v = (x.cuda() for x in frame(T, H, g))
+            if kf:
+                a.append_frame(blk, k, v); a.evict_frames(blk, scale, window); ref = a.compute_attention(blk, q)
+            else:
+                ref = a.compute_attention(blk, q, k, v)
+            out = b.step(blk, q, k, v, keyframe=[kf])
+            assert torch.equal(out, ref)
+        assert torch.equal(a._tables[..., :11], b._tables[..., :11])
+        assert a.build_visible_page_table(0) == b.build_visible_page_table(0)
+    assert torch.equal(a.kv_caches[1], b.kv_caches[1])
