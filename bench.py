@@ -1,0 +1,172 @@
+"""Benchmark of the streaming paged-KV attention hot path on one MI355X.
+
+A step is one streamed frame at 518x378 through the hot path of all global blocks: one
+index-kernel launch (allocate, evict, visible rows) and, per block, the paged K/V append
+and the paged attention of the frame's 1004 query tokens over 1 anchor + 16 window frames
+(17,068 KV tokens, 16-token pages, 16 heads, head_dim 64, bf16).  Inputs are synthetic
+N(0,1) tensors already resident in HBM.  Prints one JSON line.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--blocks 24]
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+for _p in (ROOT, os.path.join(ROOT, "lingbot-map_amd")):
+    if _p not in sys.path:
+        sys.path.insert(0, _p)
+
+T, N_SPECIAL, H, D, PAGE = 1004, 5, 16, 64, 16
+ANCHOR, WINDOW = 1, 16
+PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA
+PEAK_HBM_GBPS = 8000.0
+METRIC = "frames/sec streaming @518x378 (1 GPU); attention TFLOPS & % bf16 MFMA peak"
+
+
+def event_time_ms(fn, iters: int, torch) -> float:
+    """Average duration of fn() in ms from one HIP event pair on the launch stream."""
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    start.record()
+    for _ in range(iters):
+        fn()
+    stop.record()
+    stop.synchronize()
+    return start.elapsed_time(stop) / iters
+
+
+def cpu_baseline(torch, kv_tokens: int, blocks: int) -> dict:
+    """The reference SDPA arithmetic (dense gather of the visible pages, then
+    F.scaled_dot_product_attention) as restated by the oracle, on the host cores."""
+    from oracle.sdpa_cache import gather_paged, sdpa_nhd
+    g = torch.Generator().manual_seed(1)
+    frames = ANCHOR + WINDOW
+    ppf = -(-T // PAGE)
+    pool = torch.randn(frames * ppf, 2, PAGE, H, D, generator=g).to(torch.bfloat16)
+    ids = list(range(frames * ppf))
+    lens = ([PAGE] * (ppf - 1) + [T - (ppf - 1) * PAGE]) * frames
+    q = torch.randn(T, H, D, generator=g).to(torch.bfloat16)
+    assert sum(lens) == kv_tokens
+
+    def one():
+        k, v = gather_paged(pool, ids, lens)
+        return sdpa_nhd(q, k, v)
+
+    for _ in range(2):
+        one()
+    times = []
+    for _ in range(5):
+        t0 = time.perf_counter()
+        one()
+        times.append(time.perf_counter() - t0)
+    t = sorted(times)[len(times) // 2]
+    flops = 4.0 * T * kv_tokens * H * D
+    return {
+        "value": 1.0 / (t * blocks), "unit": "frames/s", "cores": torch.get_num_threads(), "kind": "port",
+        "sample": f"2 warm-up + 5 timed layer-steps of gather + SDPA (q {T} x kv {kv_tokens}, {H} heads, "
+                  f"bf16 storage, fp32 math), median {t * 1e3:.1f} ms = {flops / t * 1e-9:.0f} GFLOP/s; "
+                  f"frames/s = 1 / ({blocks} x median)",
+    }
+
+
+def main() -> None:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--blocks", type=int, default=24)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--mode", choices=["full", "attention", "append", "tables"], default="full",
+                    help="full = the benchmark line; the others launch one kernel --steps times "
+                         "on the steady-state cache (for rocprofv3 runs)")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        sys.exit("bench.py: this path is built and measured on ONE GPU; --gpus N with N > 1 is not supported "
+                 "(streams shard across GPUs without communication; see DESIGN.md)")
+
+    import torch
+    from lingbot_map_amd import HipPagedKVCacheManager
+
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    blocks = args.blocks
+    m = HipPagedKVCacheManager(blocks, ANCHOR + WINDOW + 16, T, H, D, torch.bfloat16, dev,
+                               num_special_tokens=N_SPECIAL, scale_frames=ANCHOR, sliding_window=WINDOW,
+                               max_total_frames=256, page_size=PAGE, layout="frame_pages")
+    g = torch.Generator(device=dev).manual_seed(1)
+    n_sets = 4
+    qs, ks, vs = ([torch.randn(T, H, D, generator=g, device=dev, dtype=torch.float32).to(torch.bfloat16)
+                   for _ in range(n_sets)] for _ in range(3))
+
+    def frame(i: int) -> None:
+        for b in range(blocks):
+            j = (i + b) % n_sets
+            # evicted frames leave no trajectory memory here, so the KV set stays at 17,068 tokens
+            m.step(b, qs[j], ks[j], vs[j], keyframe=[True], cross_frame_special=False)
+
+    for i in range(ANCHOR + WINDOW):       # fill the anchor and the window
+        frame(i)
+    kv_tokens = (ANCHOR + WINDOW) * T
+    assert m._plan_tokens[0][0] == kv_tokens == 17068
+    if args.mode != "full":
+        ops = m._ops([{"ops": 16, "expect_kv_tokens": kv_tokens}])
+        fn = {"attention": lambda: m._attend_planned(1, qs[0], None, None),
+              "append": lambda: m._scatter(1, 0, ks[0], vs[0]),
+              "tables": lambda: m._tables_step(0, ops, kv_rows=True)}[args.mode]
+        for _ in range(args.warmup):
+            fn()
+        ms = event_time_ms(fn, args.steps, torch)
+        print(json.dumps({"mode": args.mode, "launches": args.steps, "avg_launch_us": ms * 1e3}))
+        return
+    for i in range(args.warmup):
+        frame(i)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        frame(i)
+    torch.cuda.synchronize()
+    total = time.perf_counter() - t0
+    assert m.device_header()["error"] == 0
+    ms_per_step = total / args.steps * 1e3
+    fps = args.steps / total
+
+    # ---- per-kernel timings with HIP events on the launch stream
+    flops = 4.0 * T * kv_tokens * H * D
+    attn_ms = event_time_ms(lambda: m._attend_planned(1, qs[0], None, None), 200, torch)
+    append_ms = event_time_ms(lambda: m._scatter(1, 0, ks[0], vs[0]), 200, torch)
+    ops = m._ops([{"ops": 16, "expect_kv_tokens": kv_tokens}])
+    tables_ms = event_time_ms(lambda: m._tables_step(0, ops, kv_rows=True), 200, torch)
+    attn_tflops = flops / (attn_ms * 1e-3) * 1e-12
+    append_bytes = 2 * 2 * T * H * D * 2
+    append_gbps = append_bytes / (append_ms * 1e-3) * 1e-9
+
+    line = {
+        "metric": METRIC, "value": fps, "unit": "frames/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": f"config 2: 518x378 streaming, {T} tokens/frame, page {PAGE}, {ANCHOR} anchor + "
+                               f"{WINDOW} window frames = {kv_tokens} KV tokens, {H} heads x {D}, {blocks} global "
+                               f"blocks per frame (tables step + per block paged append + paged attention)",
+                   "blocks": blocks, "kv_tokens": kv_tokens, "q_tokens": T, "page_size": PAGE},
+        "roofline": {"bound": "mfma", "achieved": attn_tflops, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
+                     "frac": attn_tflops / PEAK_BF16_TFLOPS, "traffic": None,
+                     "kernel": "lbm_attn_bf16_d64_kernel + lbm_attn_combine_bf16_kernel (one lbm_attn_run)",
+                     "flop_per_launch": flops, "avg_launch_us": attn_ms * 1e3},
+        "attention_tflops": attn_tflops,
+        "append": {"bound": "hbm", "achieved": append_gbps, "peak": PEAK_HBM_GBPS, "unit": "GB/s",
+                   "frac": append_gbps / PEAK_HBM_GBPS, "bytes_per_launch": append_bytes,
+                   "avg_launch_us": append_ms * 1e3},
+        "tables_step_us": tables_ms * 1e3,
+    }
+    if not args.no_cpu_baseline:
+        line["cpu_baseline"] = cpu_baseline(torch, kv_tokens, blocks)
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

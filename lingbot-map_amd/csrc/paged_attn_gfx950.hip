@@ -2,9 +2,9 @@
 // rows a row table names (pool pages in any order, partially filled pages already squeezed
 // out by the table, optional read-only tail from the caller's own K/V).
 //
-// bf16 kernel, head_dim 64.  One workgroup = 4 wavefronts x 64 query rows of one head over
+// bf16 kernel, head_dim 64.  One workgroup = 8 wavefronts x 64 query rows of one head over
 // one contiguous run of 64-token KV tiles (split-KV; partial results are merged by
-// lbm_attn_combine_kernel).  Per tile a wavefront computes
+// lbm_attn_combine_bf16_kernel).  Per tile a wavefront computes
 //     S^T = K Q^T      v_mfma_f32_32x32x16_bf16, A = K rows from LDS, B = Q in registers
 //     P   = exp2(S*c - m)   one query row per lane column, so row max/sum stay in-lane
 //                           except one half-swap (v_permlane32_swap)
@@ -13,28 +13,64 @@
 // The running maximum is only raised when a tile exceeds it by more than kTau (in log2
 // units): the rescale of the 64 output registers is skipped on almost every tile and the
 // result is mathematically unchanged because the same stale maximum divides out.
+//
+// Schedule.  A SIMD cannot overlap the matrix pipe with the vector ALU when its two waves
+// run the same phase at the same time (measured: MFMA-busy + VALU-busy = kernel time).  The
+// eight waves therefore form two groups of four (one wave of each group per SIMD) that are
+// kept one phase apart by the workgroup barrier: while one group issues the 32 MFMAs of a
+// tile (PV of the previous tile, QK of the next), the other runs the softmax VALU work of
+// its tile.  K/V tiles are shared by all eight waves through a three-stage LDS ring.
 #include <hip/hip_runtime.h>
+#include <climits>
 #include "lbm_internal.h"
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
+typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
 typedef __attribute__((ext_vector_type(16))) float f32x16;
 typedef __attribute__((ext_vector_type(8))) float f32x8;
-typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
 typedef __attribute__((ext_vector_type(4))) float f32x4;
 typedef __attribute__((ext_vector_type(4))) unsigned int u32x4;
-typedef __attribute__((ext_vector_type(2))) unsigned int u32x2;
 typedef __attribute__((ext_vector_type(4))) short s16x4;
 typedef __attribute__((ext_vector_type(8))) short s16x8;
+
+#ifndef LBM_PRIO_MODE
+#define LBM_PRIO_MODE 1
+#endif
+#if LBM_PRIO_MODE == 1   // matrix phase runs at raised priority
+#define LBM_PRIO_MATRIX_BEGIN __builtin_amdgcn_s_setprio(1)
+#define LBM_PRIO_MATRIX_END __builtin_amdgcn_s_setprio(0)
+#elif LBM_PRIO_MODE == 2  // vector phase runs at raised priority
+#define LBM_PRIO_MATRIX_BEGIN __builtin_amdgcn_s_setprio(0)
+#define LBM_PRIO_MATRIX_END __builtin_amdgcn_s_setprio(1)
+#else                    // equal priority; sched_barrier keeps the phase boundaries
+#define LBM_PRIO_MATRIX_BEGIN __builtin_amdgcn_sched_barrier(0)
+#define LBM_PRIO_MATRIX_END __builtin_amdgcn_sched_barrier(0)
+#endif
+
+#ifdef LBM_TRACE
+__device__ long long g_lbm_trace[2 * 64 * 8];
+#define LBM_TRACE_POINT(slot) do { if (blockIdx.x == 0 && (wave == 0 || wave == 4) && lane == 0 && trace_i < 64) \
+    g_lbm_trace[((wave >> 2) * 64 + trace_i) * 8 + (slot)] = __builtin_readcyclecounter(); } while (0)
+extern "C" int lbm_debug_trace_read(long long* dst) {
+  return (int)hipMemcpyFromSymbol(dst, HIP_SYMBOL(g_lbm_trace), sizeof(g_lbm_trace));
+}
+#else
+#define LBM_TRACE_POINT(slot) do { } while (0)
+#endif
 
 namespace {
 
 constexpr int kKvTile = 64;             // KV tokens per tile
 constexpr int kQPerWave = 64;           // query rows per wavefront (two 32-row MFMA blocks)
-constexpr int kWaves = 4;
+constexpr int kWaves = 8;
+constexpr int kThreads = kWaves * 64;
 constexpr int kQTile = kQPerWave * kWaves;
+constexpr int kStages = 3;              // LDS ring depth
 constexpr int kKStride = 72;            // bf16 per LDS row of K: 144 B, b128 reads hit 64 distinct banks
 constexpr int kVStride = 96;            // bf16 per LDS row of V: 192 B, 4-row transpose reads conflict-free
 constexpr float kTau = 8.0f;            // lazy-rescale threshold, log2 units
+constexpr int kTargetWgs = 256;         // one 8-wave workgroup per CU
 
 struct AttnArgs {
   const unsigned short* q;
@@ -62,6 +98,13 @@ __device__ __forceinline__ void swap_halves(float x, float& lo, float& hi) {
   lo = a;
   hi = b;
 }
+// Forces a value to exist in registers at this point of the program: the compiler otherwise
+// sinks the softmax arithmetic below the workgroup barrier into the next phase, where it
+// would run on the vector ALU at the same time as the other group's softmax.
+__device__ __forceinline__ void pin(bf16x8& x) { asm volatile("" : "+v"(x)); }
+__device__ __forceinline__ void pin(f32x16& x) { asm volatile("" : "+v"(x)); }
+__device__ __forceinline__ void pin(float& x) { asm volatile("" : "+v"(x)); }
+
 __device__ __forceinline__ float swap_max(float x) {
   float lo, hi;
   swap_halves(x, lo, hi);
@@ -75,12 +118,13 @@ __device__ __forceinline__ float swap_sum(float x) {
 
 }  // namespace
 
-__global__ __launch_bounds__(256, 2) void lbm_attn_bf16_d64_kernel(AttnArgs a) {
-  __shared__ __attribute__((aligned(16))) unsigned short lds_k[2][kKvTile * kKStride];
-  __shared__ __attribute__((aligned(16))) unsigned short lds_v[2][kKvTile * kVStride];
+__global__ __launch_bounds__(kThreads, 1) void lbm_attn_bf16_d64_kernel(AttnArgs a) {
+  __shared__ __attribute__((aligned(16))) unsigned short lds_k[kStages][kKvTile * kKStride];
+  __shared__ __attribute__((aligned(16))) unsigned short lds_v[kStages][kKvTile * kVStride];
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int n32 = lane & 31, g = lane >> 5;
+  const int group = wave >> 2;  // waves w and w+4 share a SIMD and run opposite phases
 
   // ---- which piece of work is this workgroup
   int b = 0;
@@ -106,8 +150,8 @@ __global__ __launch_bounds__(256, 2) void lbm_attn_bf16_d64_kernel(AttnArgs a) {
   const int n_tiles = (sp.kv_tokens + kKvTile - 1) / kKvTile;
   const int t0 = split * sp.tiles_per_split;
   const int t1 = min(t0 + sp.tiles_per_split, n_tiles);
+  const int n = t1 - t0;
   const size_t row_elems = (size_t)H * 64;
-  const size_t v_off = (size_t)a.page_size * row_elems;
 
   // ---- Q fragments (B operand of S^T = K Q^T): lane holds q row n32, d = ks*16 + g*8 .. +8
   bf16x8 qf[2][4];
@@ -134,69 +178,80 @@ __global__ __launch_bounds__(256, 2) void lbm_attn_bf16_d64_kernel(AttnArgs a) {
   float m_run[2] = {-INFINITY, -INFINITY};
   float l_run[2] = {0.f, 0.f};
 
-  // ---- tile staging: each thread moves two 16-byte pieces of K and of V per tile
+  // ---- tile staging: each thread moves one 16-byte piece of a K row and of a V row per tile
   const int ld_r = tid >> 3, ld_c = (tid & 7) * 8;
-  u32x4 kreg[2], vreg[2];
-  auto fetch = [&](int t) {
-#pragma unroll
-    for (int i = 0; i < 2; ++i) {
-      const int kvi = t * kKvTile + ld_r + 32 * i;
-      u32x4 kk = {0u, 0u, 0u, 0u}, vv = {0u, 0u, 0u, 0u};
-      if (kvi < sp.kv_tokens) {
-        const int e = a.kv_rows[sp.kv_row_begin + kvi];
-        const unsigned short *kp, *vp;
-        if (e >= 0) {
-          kp = a.pool + ((size_t)e * H + head) * 64 + ld_c;
-          vp = kp + v_off;
-        } else {
-          const size_t off = ((size_t)(-1 - e) * H + head) * 64 + ld_c;
-          kp = a.self_k + off;
-          vp = a.self_v + off;
-        }
-        kk = *(const u32x4*)kp;
-        vv = *(const u32x4*)vp;
-      }
-      kreg[i] = kk;
-      vreg[i] = vv;
-    }
+  const unsigned short* pool_k = a.pool + (size_t)head * 64 + ld_c;
+  const unsigned short* pool_v = pool_k + (size_t)a.page_size * row_elems;
+  const unsigned short* own_k = a.self_k + (size_t)head * 64 + ld_c;
+  const unsigned short* own_v = a.self_v + (size_t)head * 64 + ld_c;
+  const int32_t* rows = a.kv_rows + sp.kv_row_begin;
+  // Row-table entry of this thread's row in tile t; INT_MIN marks "no token" (zero fill).
+  auto row_entry = [&](int t) -> int {
+    const int kvi = t * kKvTile + ld_r;
+    return (t < t1 && kvi < sp.kv_tokens) ? rows[kvi] : INT_MIN;
   };
-  auto stage = [&](int buf) {
-#pragma unroll
-    for (int i = 0; i < 2; ++i) {
-      const int r = ld_r + 32 * i;
-      *(u32x4*)&lds_k[buf][r * kKStride + ld_c] = kreg[i];
-      *(u32x4*)&lds_v[buf][r * kVStride + ld_c] = vreg[i];
+  auto fetch = [&](int e, const unsigned short* pool_base, const unsigned short* own_base) -> u32x4 {
+    u32x4 v = {0u, 0u, 0u, 0u};
+    if (e != INT_MIN) {
+      const bool own = e < 0;
+      const unsigned short* base = own ? own_base : pool_base;
+      const size_t r = own ? (size_t)(-1 - e) : (size_t)e;
+      v = *(const u32x4*)(base + r * row_elems);
     }
+    return v;
   };
+  auto put_k = [&](int stage, u32x4 v) { *(u32x4*)&lds_k[stage][ld_r * kKStride + ld_c] = v; };
+  auto put_v = [&](int stage, u32x4 v) { *(u32x4*)&lds_v[stage][ld_r * kVStride + ld_c] = v; };
 
-  fetch(t0);
-  stage(0);
-  __syncthreads();
+  f32x16 s[2][2];   // s[kvb][qb][i]: kv = kvb*32 + 8*(i/4) + 4*g + i%4, q = qb*32 + n32
+  bf16x8 pb[2][4];  // softmax numerators as the B operand of O^T += V^T P^T
 
-  for (int t = t0; t < t1; ++t) {
-    const int buf = (t - t0) & 1;
-    if (t + 1 < t1) fetch(t + 1);
-
-    // ---- S^T = K Q^T : s[kvb][qb][i] is kv = kvb*32 + 8*(i/4) + 4*g + i%4, q = qb*32 + n32
-    f32x16 s[2][2];
-#pragma unroll
-    for (int kvb = 0; kvb < 2; ++kvb)
-#pragma unroll
-      for (int qb = 0; qb < 2; ++qb)
-#pragma unroll
-        for (int i = 0; i < 16; ++i) s[kvb][qb][i] = 0.f;
+  // S^T = K Q^T for the tile in K stage `st`
+  auto qk = [&](int st) {
 #pragma unroll
     for (int kvb = 0; kvb < 2; ++kvb) {
 #pragma unroll
       for (int ks = 0; ks < 4; ++ks) {
         const bf16x8 ka = __builtin_bit_cast(
-            bf16x8, *(const u32x4*)&lds_k[buf][(kvb * 32 + n32) * kKStride + ks * 16 + g * 8]);
+            bf16x8, *(const u32x4*)&lds_k[st][(kvb * 32 + n32) * kKStride + ks * 16 + g * 8]);
 #pragma unroll
-        for (int qb = 0; qb < 2; ++qb)
-          s[kvb][qb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka, qf[qb][ks], s[kvb][qb], 0, 0, 0);
+        for (int qb = 0; qb < 2; ++qb) {
+          if (ks == 0) {
+            f32x16 z;
+#pragma unroll
+            for (int i = 0; i < 16; ++i) z[i] = 0.f;
+            s[kvb][qb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka, qf[qb][ks], z, 0, 0, 0);
+          } else {
+            s[kvb][qb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka, qf[qb][ks], s[kvb][qb], 0, 0, 0);
+          }
+        }
       }
     }
-
+  };
+  // O^T += V^T P^T : o[qb][db][i] is d = db*32 + 8*(i/4) + 4*g + i%4, q = qb*32 + n32
+  auto pv = [&](int st) {
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) {
+#pragma unroll
+      for (int db = 0; db < 2; ++db) {
+        const int row = ks * 16 + 4 * g + ((lane & 15) >> 2);
+        const int col = db * 32 + ((lane >> 4) & 1) * 16 + (lane & 3) * 4;
+        const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+            (s16x4 __attribute__((address_space(3)))*)&lds_v[st][row * kVStride + col]);
+        const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+            (s16x4 __attribute__((address_space(3)))*)&lds_v[st][(row + 8) * kVStride + col]);
+        s16x8 both;
+        both[0] = lo[0]; both[1] = lo[1]; both[2] = lo[2]; both[3] = lo[3];
+        both[4] = hi[0]; both[5] = hi[1]; both[6] = hi[2]; both[7] = hi[3];
+        const bf16x8 va = __builtin_bit_cast(bf16x8, both);
+#pragma unroll
+        for (int qb = 0; qb < 2; ++qb)
+          o[qb][db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va, pb[qb][ks], o[qb][db], 0, 0, 0);
+      }
+    }
+  };
+  // softmax numerators of tile t from s into pb; maintains m_run, l_run, rescales o lazily
+  auto softmax = [&](int t) {
     const int n_valid = sp.kv_tokens - t * kKvTile;
     if (n_valid < kKvTile) {
 #pragma unroll
@@ -210,9 +265,7 @@ __global__ __launch_bounds__(256, 2) void lbm_attn_bf16_d64_kernel(AttnArgs a) {
           }
         }
     }
-
-    // ---- softmax numerators, packed to bf16 as the B operand of O^T += V^T P^T
-    bf16x8 pb[2][4];
+    const bf16x2 ones = {(__bf16)1.0f, (__bf16)1.0f};
 #pragma unroll
     for (int qb = 0; qb < 2; ++qb) {
       float mx = s[0][qb][0];
@@ -234,47 +287,103 @@ __global__ __launch_bounds__(256, 2) void lbm_attn_bf16_d64_kernel(AttnArgs a) {
           for (int i = 0; i < 16; ++i) o[qb][db][i] *= alpha;
       }
       const float mr = m_run[qb];
-      float lsum = 0.f;
+      float lsum = l_run[qb];
 #pragma unroll
       for (int kvb = 0; kvb < 2; ++kvb) {
 #pragma unroll
         for (int hh = 0; hh < 2; ++hh) {
           f32x8 p;
 #pragma unroll
-          for (int j = 0; j < 8; ++j) {
+          for (int j = 0; j < 8; ++j)
             p[j] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[kvb][qb][hh * 8 + j], a.scale_log2, -mr));
-            lsum += p[j];
+          const bf16x8 pk = __builtin_convertvector(p, bf16x8);
+          pb[qb][kvb * 2 + hh] = pk;
+          // the denominator sums the bf16-rounded numerators the PV product actually uses
+#pragma unroll
+          for (int j = 0; j < 8; j += 2) {
+            const bf16x2 pr = {pk[j], pk[j + 1]};
+            lsum = __builtin_amdgcn_fdot2_f32_bf16(pr, ones, lsum, false);
           }
-          pb[qb][kvb * 2 + hh] = __builtin_convertvector(p, bf16x8);
         }
       }
-      l_run[qb] += lsum;
+      l_run[qb] = lsum;
     }
+  };
 
-    // ---- O^T += V^T P^T : o[qb][db][i] is d = db*32 + 8*(i/4) + 4*g + i%4, q = qb*32 + n32
+  // ---- prologue: K(0), K(1), V(0) into the ring
+  put_k(0, fetch(row_entry(t0), pool_k, own_k));
+  put_k(1, fetch(row_entry(t0 + 1), pool_k, own_k));
+  put_v(0, fetch(row_entry(t0), pool_v, own_v));
+  int ek = row_entry(t0 + 2), ev = row_entry(t0 + 1);   // entries of the next pieces to fetch
+  __syncthreads();
+  if (group == 1) __syncthreads();  // puts the second group one phase behind the first
+
+  // matrix phase 0
+  u32x4 kreg = fetch(ek, pool_k, own_k), vreg = fetch(ev, pool_v, own_v);
+  LBM_PRIO_MATRIX_BEGIN;
+  qk(0);
+  LBM_PRIO_MATRIX_END;
 #pragma unroll
-    for (int ks = 0; ks < 4; ++ks) {
+  for (int kvb = 0; kvb < 2; ++kvb)
 #pragma unroll
-      for (int db = 0; db < 2; ++db) {
-        const int row = ks * 16 + 4 * g + ((lane & 15) >> 2);
-        const int col = db * 32 + ((lane >> 4) & 1) * 16 + (lane & 3) * 4;
-        const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-            (s16x4 __attribute__((address_space(3)))*)&lds_v[buf][row * kVStride + col]);
-        const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-            (s16x4 __attribute__((address_space(3)))*)&lds_v[buf][(row + 8) * kVStride + col]);
-        s16x8 both;
-        both[0] = lo[0]; both[1] = lo[1]; both[2] = lo[2]; both[3] = lo[3];
-        both[4] = hi[0]; both[5] = hi[1]; both[6] = hi[2]; both[7] = hi[3];
-        const bf16x8 va = __builtin_bit_cast(bf16x8, both);
+    for (int qb = 0; qb < 2; ++qb) pin(s[kvb][qb]);
+  __syncthreads();
+
+  int st_k = 0, st_v = 0;  // stage of K(i) and of V(i)
+  for (int i = 0; i < n; ++i) {
+    const int t = t0 + i;
+    const int trace_i = i; (void)trace_i;
+    LBM_TRACE_POINT(0);
+    // ---- vector phase i: softmax of tile i; land K(i+2), V(i+1) in the ring
+    ek = row_entry(t + 3);
+    ev = row_entry(t + 2);
+#ifndef LBM_SKIP_VECTOR
+    softmax(t);
+#endif
+    int st_k2 = st_k + 2; if (st_k2 >= kStages) st_k2 -= kStages;
+    int st_v1 = st_v + 1; if (st_v1 >= kStages) st_v1 -= kStages;
+    if (i + 2 < n) put_k(st_k2, kreg);
+    if (i + 1 < n) put_v(st_v1, vreg);
 #pragma unroll
-        for (int qb = 0; qb < 2; ++qb)
-          o[qb][db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va, pb[qb][ks], o[qb][db], 0, 0, 0);
-      }
+    for (int qb = 0; qb < 2; ++qb) {
+#pragma unroll
+      for (int ks = 0; ks < 4; ++ks) pin(pb[qb][ks]);
+      pin(l_run[qb]);
     }
-
-    if (t + 1 < t1) stage(buf ^ 1);
+    LBM_TRACE_POINT(1);
     __syncthreads();
+    LBM_TRACE_POINT(2);
+    // ---- matrix phase i+1: PV of tile i, QK of tile i+1; start fetching K(i+3), V(i+2)
+    kreg = fetch(ek, pool_k, own_k);
+    vreg = fetch(ev, pool_v, own_v);
+    int st_k1 = st_k + 1; if (st_k1 >= kStages) st_k1 -= kStages;
+    LBM_PRIO_MATRIX_BEGIN;
+#ifndef LBM_SKIP_MATRIX
+    pv(st_v);
+    qk(st_k1);  // on the last tile this reads a stale stage and its result is never used
+    // LDS fragment reads run three steps (of two MFMAs) ahead of the MFMAs that use them:
+    // 8 PV steps with two transpose reads each, then 8 QK steps with one 128-bit read each.
+    __builtin_amdgcn_sched_group_barrier(0x100, 6, 0);
+#pragma unroll
+    for (int step = 0; step < 16; ++step) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
+      const int ahead = step + 3;
+      if (ahead < 8) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+      else if (ahead < 16) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+    }
+#endif
+    LBM_PRIO_MATRIX_END;
+#pragma unroll
+    for (int kvb = 0; kvb < 2; ++kvb)
+#pragma unroll
+      for (int qb = 0; qb < 2; ++qb) pin(s[kvb][qb]);
+    LBM_TRACE_POINT(3);
+    __syncthreads();
+    LBM_TRACE_POINT(4);
+    st_k = st_k1;
+    st_v = st_v1;
   }
+  if (group == 0) __syncthreads();  // both groups pass the same number of barriers
 
   // ---- epilogue
 #pragma unroll
@@ -346,8 +455,8 @@ __global__ __launch_bounds__(256) void lbm_attn_combine_bf16_kernel(AttnArgs a) 
 // ---------------------------------------------------------------------------- schedule
 void lbm_attn_schedule(const lbm_attn_stream* streams, int n_streams, int num_heads,
                        LbmAttnSchedule* out) {
-  // Aim at two workgroups on each of the 256 CUs, all with about the same number of tiles.
-  const long long target_wgs = 512;
+  // Aim at one 8-wave workgroup on each of the 256 CUs, all with about the same number of tiles.
+  const long long target_wgs = kTargetWgs;
   LbmAttnSchedule& sch = *out;
   sch = LbmAttnSchedule{};
   sch.n_streams = n_streams;
@@ -409,7 +518,7 @@ int lbm_launch_attention(const void* q, const void* pool, void* out, const void*
   a.scale_log2 = sm_scale * 1.4426950408889634f;
   a.sch = sch;
   if (sch.total_wgs == 0) return LBM_OK;
-  hipLaunchKernelGGL(lbm_attn_bf16_d64_kernel, dim3(sch.total_wgs), dim3(256), 0, stream, a);
+  hipLaunchKernelGGL(lbm_attn_bf16_d64_kernel, dim3(sch.total_wgs), dim3(kThreads), 0, stream, a);
   int rc = lbm_check_launch("lbm_attn_bf16_d64_kernel");
   if (rc != LBM_OK) return rc;
   if (sch.part_rows > 0) {
