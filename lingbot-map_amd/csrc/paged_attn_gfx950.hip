@@ -14,12 +14,17 @@
 // units): the rescale of the 64 output registers is skipped on almost every tile and the
 // result is mathematically unchanged because the same stale maximum divides out.
 //
-// Schedule.  A SIMD cannot overlap the matrix pipe with the vector ALU when its two waves
-// run the same phase at the same time (measured: MFMA-busy + VALU-busy = kernel time).  The
-// eight waves therefore form two groups of four (one wave of each group per SIMD) that are
-// kept one phase apart by the workgroup barrier: while one group issues the 32 MFMAs of a
-// tile (PV of the previous tile, QK of the next), the other runs the softmax VALU work of
-// its tile.  K/V tiles are shared by all eight waves through a three-stage LDS ring.
+// Schedule.  Measured on MI355X: one wavefront alone issues a vector-ALU instruction only
+// every ~8 cycles, two wavefronts of a SIMD together reach the full rate of one per 4, and
+// the matrix pipe overlaps with the vector ALU only when MFMAs and vector instructions
+// alternate in program order.  Each wavefront therefore runs a software pipeline over
+// 32-token half tiles: while the vector ALU turns the scores of one half into softmax
+// numerators, the MFMAs of the next half's QK^T and of the previous half's PV are issued in
+// between (sched_group_barrier fixes the interleaving), and the two wavefronts of a SIMD
+// fill each other's issue gaps.  The running reference maximum and the softmax scale are
+// folded into the QK^T contraction, so the vector ALU only does max, exp2, bf16 packing and
+// the row sum.  K/V tiles are shared by all eight waves through a three-stage LDS ring with
+// one workgroup barrier per tile.
 #include <hip/hip_runtime.h>
 #include <climits>
 #include "lbm_internal.h"
@@ -33,31 +38,6 @@ typedef __attribute__((ext_vector_type(4))) float f32x4;
 typedef __attribute__((ext_vector_type(4))) unsigned int u32x4;
 typedef __attribute__((ext_vector_type(4))) short s16x4;
 typedef __attribute__((ext_vector_type(8))) short s16x8;
-
-#ifndef LBM_PRIO_MODE
-#define LBM_PRIO_MODE 1
-#endif
-#if LBM_PRIO_MODE == 1   // matrix phase runs at raised priority
-#define LBM_PRIO_MATRIX_BEGIN __builtin_amdgcn_s_setprio(1)
-#define LBM_PRIO_MATRIX_END __builtin_amdgcn_s_setprio(0)
-#elif LBM_PRIO_MODE == 2  // vector phase runs at raised priority
-#define LBM_PRIO_MATRIX_BEGIN __builtin_amdgcn_s_setprio(0)
-#define LBM_PRIO_MATRIX_END __builtin_amdgcn_s_setprio(1)
-#else                    // equal priority; sched_barrier keeps the phase boundaries
-#define LBM_PRIO_MATRIX_BEGIN __builtin_amdgcn_sched_barrier(0)
-#define LBM_PRIO_MATRIX_END __builtin_amdgcn_sched_barrier(0)
-#endif
-
-#ifdef LBM_TRACE
-__device__ long long g_lbm_trace[2 * 64 * 8];
-#define LBM_TRACE_POINT(slot) do { if (blockIdx.x == 0 && (wave == 0 || wave == 4) && lane == 0 && trace_i < 64) \
-    g_lbm_trace[((wave >> 2) * 64 + trace_i) * 8 + (slot)] = __builtin_readcyclecounter(); } while (0)
-extern "C" int lbm_debug_trace_read(long long* dst) {
-  return (int)hipMemcpyFromSymbol(dst, HIP_SYMBOL(g_lbm_trace), sizeof(g_lbm_trace));
-}
-#else
-#define LBM_TRACE_POINT(slot) do { } while (0)
-#endif
 
 namespace {
 
@@ -79,7 +59,7 @@ struct AttnArgs {
   const unsigned short* self_k;
   const unsigned short* self_v;
   const int32_t* kv_rows;
-  float* part_o;
+  unsigned short* part_o;  // split-KV partial outputs, normalised, bf16
   float* part_lse;
   int num_heads;
   int page_size;
@@ -98,17 +78,13 @@ __device__ __forceinline__ void swap_halves(float x, float& lo, float& hi) {
   lo = a;
   hi = b;
 }
-// Forces a value to exist in registers at this point of the program: the compiler otherwise
-// sinks the softmax arithmetic below the workgroup barrier into the next phase, where it
-// would run on the vector ALU at the same time as the other group's softmax.
-__device__ __forceinline__ void pin(bf16x8& x) { asm volatile("" : "+v"(x)); }
-__device__ __forceinline__ void pin(f32x16& x) { asm volatile("" : "+v"(x)); }
-__device__ __forceinline__ void pin(float& x) { asm volatile("" : "+v"(x)); }
-
+// Built with -fno-honor-nans, fmaxf chains become v_max3_f32 without NaN-quieting moves.
+__device__ __forceinline__ float max3(float a, float b, float c) { return fmaxf(fmaxf(a, b), c); }
+__device__ __forceinline__ float max2(float a, float b) { return fmaxf(a, b); }
 __device__ __forceinline__ float swap_max(float x) {
   float lo, hi;
   swap_halves(x, lo, hi);
-  return fmaxf(lo, hi);
+  return max2(lo, hi);
 }
 __device__ __forceinline__ float swap_sum(float x) {
   float lo, hi;
@@ -124,7 +100,6 @@ __global__ __launch_bounds__(kThreads, 1) void lbm_attn_bf16_d64_kernel(AttnArgs
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int n32 = lane & 31, g = lane >> 5;
-  const int group = wave >> 2;  // waves w and w+4 share a SIMD and run opposite phases
 
   // ---- which piece of work is this workgroup
   int b = 0;
@@ -151,9 +126,11 @@ __global__ __launch_bounds__(kThreads, 1) void lbm_attn_bf16_d64_kernel(AttnArgs
   const int t0 = split * sp.tiles_per_split;
   const int t1 = min(t0 + sp.tiles_per_split, n_tiles);
   const int n = t1 - t0;
-  const size_t row_elems = (size_t)H * 64;
+  const unsigned row_bytes = (unsigned)H * 128u;
 
-  // ---- Q fragments (B operand of S^T = K Q^T): lane holds q row n32, d = ks*16 + g*8 .. +8
+  // ---- Q fragments (B operand of S^T = K Q^T): lane holds q row n32, d = ks*16 + g*8 .. +8.
+  // The softmax scale and log2(e) are folded into Q here (one extra bf16 rounding of q), so
+  // the MFMA result is already the exponent of 2.
   bf16x8 qf[2][4];
   const int q_row0 = qt * kQTile + wave * kQPerWave;
 #pragma unroll
@@ -164,9 +141,20 @@ __global__ __launch_bounds__(kThreads, 1) void lbm_attn_bf16_d64_kernel(AttnArgs
     for (int ks = 0; ks < 4; ++ks) {
       u32x4 v = {0u, 0u, 0u, 0u};
       if (r < sp.q_rows) v = *(const u32x4*)(qp + ks * 16);
-      qf[qb][ks] = __builtin_bit_cast(bf16x8, v);
+      const bf16x8 raw = __builtin_bit_cast(bf16x8, v);
+      f32x8 f = __builtin_convertvector(raw, f32x8);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) f[j] *= a.scale_log2;
+      qf[qb][ks] = __builtin_convertvector(f, bf16x8);
     }
   }
+  // One more 16-wide step of the QK contraction carries the running reference maximum:
+  // K side is the constant row (-1, -1, 0, ...), Q side is (m_hi, m_lo, 0, ...) with
+  // m_hi + m_lo = m_run exactly, so S arrives as score*scale - m_run at no vector-ALU cost.
+  u32x4 kaug_bits = {0u, 0u, 0u, 0u};
+  if (g == 0) kaug_bits[0] = 0xBF80BF80u;
+  const bf16x8 kaug = __builtin_bit_cast(bf16x8, kaug_bits);
+  u32x4 qaug_bits[2] = {{0u, 0u, 0u, 0u}, {0u, 0u, 0u, 0u}};
 
   f32x16 o[2][2];
 #pragma unroll
@@ -175,221 +163,239 @@ __global__ __launch_bounds__(kThreads, 1) void lbm_attn_bf16_d64_kernel(AttnArgs
     for (int db = 0; db < 2; ++db)
 #pragma unroll
       for (int i = 0; i < 16; ++i) o[qb][db][i] = 0.f;
-  float m_run[2] = {-INFINITY, -INFINITY};
-  float l_run[2] = {0.f, 0.f};
+  float m_run[2] = {0.f, 0.f};  // re-referenced to the first tile's maximum before first use
+  float l_run[2][4] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};  // four partial row sums per query block
 
-  // ---- tile staging: each thread moves one 16-byte piece of a K row and of a V row per tile
+  // ---- tile staging: each thread moves one 16-byte piece of a K row and of a V row per tile.
+  // Rows past the last token re-read the last token (finite data; the softmax masks them).
   const int ld_r = tid >> 3, ld_c = (tid & 7) * 8;
-  const unsigned short* pool_k = a.pool + (size_t)head * 64 + ld_c;
-  const unsigned short* pool_v = pool_k + (size_t)a.page_size * row_elems;
-  const unsigned short* own_k = a.self_k + (size_t)head * 64 + ld_c;
-  const unsigned short* own_v = a.self_v + (size_t)head * 64 + ld_c;
+  const char* pool_k = (const char*)(a.pool + (size_t)head * 64 + ld_c);
+  const char* pool_v = pool_k + (size_t)a.page_size * row_bytes;
+  const char* own_k = (const char*)(a.self_k + (size_t)head * 64 + ld_c);
+  const char* own_v = (const char*)(a.self_v + (size_t)head * 64 + ld_c);
   const int32_t* rows = a.kv_rows + sp.kv_row_begin;
-  // Row-table entry of this thread's row in tile t; INT_MIN marks "no token" (zero fill).
-  auto row_entry = [&](int t) -> int {
-    const int kvi = t * kKvTile + ld_r;
-    return (t < t1 && kvi < sp.kv_tokens) ? rows[kvi] : INT_MIN;
-  };
-  auto fetch = [&](int e, const unsigned short* pool_base, const unsigned short* own_base) -> u32x4 {
-    u32x4 v = {0u, 0u, 0u, 0u};
-    if (e != INT_MIN) {
-      const bool own = e < 0;
-      const unsigned short* base = own ? own_base : pool_base;
-      const size_t r = own ? (size_t)(-1 - e) : (size_t)e;
-      v = *(const u32x4*)(base + r * row_elems);
-    }
-    return v;
+  const int last_token = sp.kv_tokens - 1;
+  // Tiles past the end of this split re-read its last tile: the data lands in ring stages
+  // nobody reads any more, and the code stays free of branches.
+  auto row_entry = [&](int t) -> int { return rows[min(min(t, t1 - 1) * kKvTile + ld_r, last_token)]; };
+  auto fetch = [&](int e, const char* pool_base, const char* own_base) -> u32x4 {
+    // negative entries name rows of the caller's own K/V (read-only tail of a non-keyframe)
+    const char* base = e < 0 ? own_base : pool_base;
+    const unsigned r = (unsigned)(e ^ (e >> 31));
+    return *(const u32x4*)(base + (unsigned long long)r * row_bytes);
   };
   auto put_k = [&](int stage, u32x4 v) { *(u32x4*)&lds_k[stage][ld_r * kKStride + ld_c] = v; };
   auto put_v = [&](int stage, u32x4 v) { *(u32x4*)&lds_v[stage][ld_r * kVStride + ld_c] = v; };
 
-  f32x16 s[2][2];   // s[kvb][qb][i]: kv = kvb*32 + 8*(i/4) + 4*g + i%4, q = qb*32 + n32
-  bf16x8 pb[2][4];  // softmax numerators as the B operand of O^T += V^T P^T
+  // Register state of the software pipeline.  A 64-token tile is processed as two 32-token
+  // halves; while the vector ALU turns the scores of one half into softmax numerators, the
+  // matrix pipe computes the scores of the next half and folds the numerators of the
+  // previous half into O.  The two halves alternate between the A and B register sets.
+  f32x16 sA[2], sB[2];        // s[qb][i]: kv = 32*half + 8*(i/4) + 4*g + i%4, q = qb*32 + n32
+  bf16x8 pA[2][2], pB[2][2];  // numerators [qb][k-step] as the B operand of O^T += V^T P^T
+  bf16x8 vnext[2];            // V^T fragments of the next PV's first k-step, read early
 
-  // S^T = K Q^T for the tile in K stage `st`
-  auto qk = [&](int st) {
-#pragma unroll
-    for (int kvb = 0; kvb < 2; ++kvb) {
-#pragma unroll
-      for (int ks = 0; ks < 4; ++ks) {
-        const bf16x8 ka = __builtin_bit_cast(
-            bf16x8, *(const u32x4*)&lds_k[st][(kvb * 32 + n32) * kKStride + ks * 16 + g * 8]);
-#pragma unroll
-        for (int qb = 0; qb < 2; ++qb) {
-          if (ks == 0) {
-            f32x16 z;
-#pragma unroll
-            for (int i = 0; i < 16; ++i) z[i] = 0.f;
-            s[kvb][qb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka, qf[qb][ks], z, 0, 0, 0);
-          } else {
-            s[kvb][qb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka, qf[qb][ks], s[kvb][qb], 0, 0, 0);
-          }
-        }
-      }
-    }
+  // V^T fragment (A operand): lane holds d = db*32 + n32 and the kv rows
+  // ks*16 + {4g..4g+3, 8+4g..8+4g+3} of the V tile in stage st
+  auto v_frag = [&](int st, int ks, int db) -> bf16x8 {
+    const int row = ks * 16 + 4 * g + ((lane & 15) >> 2);
+    const int col = db * 32 + ((lane >> 4) & 1) * 16 + (lane & 3) * 4;
+    const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+        (s16x4 __attribute__((address_space(3)))*)&lds_v[st][row * kVStride + col]);
+    const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+        (s16x4 __attribute__((address_space(3)))*)&lds_v[st][(row + 8) * kVStride + col]);
+    s16x8 both;
+    both[0] = lo[0]; both[1] = lo[1]; both[2] = lo[2]; both[3] = lo[3];
+    both[4] = hi[0]; both[5] = hi[1]; both[6] = hi[2]; both[7] = hi[3];
+    return __builtin_bit_cast(bf16x8, both);
   };
-  // O^T += V^T P^T : o[qb][db][i] is d = db*32 + 8*(i/4) + 4*g + i%4, q = qb*32 + n32
-  auto pv = [&](int st) {
+  // One k-step (16 kv rows) of O^T += V^T P^T; o[qb][db][i] is d = db*32 + 8*(i/4) + 4*g + i%4
+  auto pv_step = [&](const bf16x8 (&va)[2], const bf16x8 (&p)[2][2], int kk) {
+#pragma unroll
+    for (int db = 0; db < 2; ++db)
+#pragma unroll
+      for (int qb = 0; qb < 2; ++qb)
+        o[qb][db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va[db], p[qb][kk], o[qb][db], 0, 0, 0);
+  };
+  // S^T = K Q^T - m_run for the 32 kv rows of half h of the K tile in stage st
+  auto qk_half = [&](int st, int h, f32x16 (&sd)[2]) {
+    f32x16 z;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) z[i] = 0.f;
+#pragma unroll
+    for (int qb = 0; qb < 2; ++qb)
+      sd[qb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kaug, __builtin_bit_cast(bf16x8, qaug_bits[qb]), z, 0, 0, 0);
 #pragma unroll
     for (int ks = 0; ks < 4; ++ks) {
+      const bf16x8 ka = __builtin_bit_cast(
+          bf16x8, *(const u32x4*)&lds_k[st][(h * 32 + n32) * kKStride + ks * 16 + g * 8]);
 #pragma unroll
-      for (int db = 0; db < 2; ++db) {
-        const int row = ks * 16 + 4 * g + ((lane & 15) >> 2);
-        const int col = db * 32 + ((lane >> 4) & 1) * 16 + (lane & 3) * 4;
-        const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-            (s16x4 __attribute__((address_space(3)))*)&lds_v[st][row * kVStride + col]);
-        const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-            (s16x4 __attribute__((address_space(3)))*)&lds_v[st][(row + 8) * kVStride + col]);
-        s16x8 both;
-        both[0] = lo[0]; both[1] = lo[1]; both[2] = lo[2]; both[3] = lo[3];
-        both[4] = hi[0]; both[5] = hi[1]; both[6] = hi[2]; both[7] = hi[3];
-        const bf16x8 va = __builtin_bit_cast(bf16x8, both);
-#pragma unroll
-        for (int qb = 0; qb < 2; ++qb)
-          o[qb][db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va, pb[qb][ks], o[qb][db], 0, 0, 0);
-      }
+      for (int qb = 0; qb < 2; ++qb)
+        sd[qb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka, qf[qb][ks], sd[qb], 0, 0, 0);
     }
   };
-  // softmax numerators of tile t from s into pb; maintains m_run, l_run, rescales o lazily
-  auto softmax = [&](int t) {
-    const int n_valid = sp.kv_tokens - t * kKvTile;
-    if (n_valid < kKvTile) {
+  // First part of the softmax of one half: mask, row maxima, and - on the first half of the
+  // split or when a score exceeds the reference by more than kTau - move the reference.
+  auto soft_check = [&](f32x16 (&sc)[2], int n_valid, bool first) {
+    if (n_valid < 32) {
 #pragma unroll
-      for (int kvb = 0; kvb < 2; ++kvb)
-#pragma unroll
-        for (int i = 0; i < 16; ++i) {
-          const int kv = kvb * 32 + 8 * (i >> 2) + 4 * g + (i & 3);
-          if (kv >= n_valid) {
-            s[kvb][0][i] = -INFINITY;
-            s[kvb][1][i] = -INFINITY;
-          }
+      for (int i = 0; i < 16; ++i) {
+        const int kv = 8 * (i >> 2) + 4 * g + (i & 3);
+        if (kv >= n_valid) {
+          sc[0][i] = -INFINITY;
+          sc[1][i] = -INFINITY;
         }
+      }
     }
-    const bf16x2 ones = {(__bf16)1.0f, (__bf16)1.0f};
+    float mx[2];
 #pragma unroll
     for (int qb = 0; qb < 2; ++qb) {
-      float mx = s[0][qb][0];
+      float m0 = max3(sc[qb][0], sc[qb][1], sc[qb][2]), m1 = max3(sc[qb][3], sc[qb][4], sc[qb][5]);
+      m0 = max3(m0, sc[qb][6], sc[qb][7]);
+      m1 = max3(m1, sc[qb][8], sc[qb][9]);
+      m0 = max3(m0, sc[qb][10], sc[qb][11]);
+      m1 = max3(m1, sc[qb][12], sc[qb][13]);
+      m0 = max3(m0, sc[qb][14], sc[qb][15]);
+      mx[qb] = swap_max(max2(m0, m1));
+    }
+    if (__builtin_amdgcn_ballot_w64(first || mx[0] > kTau || mx[1] > kTau)) {
 #pragma unroll
-      for (int i = 1; i < 16; ++i) mx = fmaxf(mx, s[0][qb][i]);
-#pragma unroll
-      for (int i = 0; i < 16; ++i) mx = fmaxf(mx, s[1][qb][i]);
-      mx = swap_max(mx);
-      const float ms = mx * a.scale_log2;
-      const bool raise = ms > m_run[qb] + kTau;
-      if (__builtin_amdgcn_ballot_w64(raise)) {
-        const float m_new = raise ? ms : m_run[qb];
-        const float alpha = __builtin_amdgcn_exp2f(m_run[qb] - m_new);
+      for (int qb = 0; qb < 2; ++qb) {
+        const bool move = first || mx[qb] > kTau;
+        // new reference, rounded so that two bf16 values carry it exactly
+        const float want = move ? m_run[qb] + mx[qb] : m_run[qb];
+        const float hi = (float)(__bf16)want;
+        const float lo = (float)(__bf16)(want - hi);
+        const float m_new = hi + lo;
+        const float d = m_new - m_run[qb];
+        const float alpha = __builtin_amdgcn_exp2f(-d);
         m_run[qb] = m_new;
-        l_run[qb] *= alpha;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) l_run[qb][j] *= alpha;
+        const bf16x2 pair = {(__bf16)hi, (__bf16)lo};
+        qaug_bits[qb][0] = g == 0 ? __builtin_bit_cast(unsigned, pair) : 0u;
 #pragma unroll
         for (int db = 0; db < 2; ++db)
 #pragma unroll
           for (int i = 0; i < 16; ++i) o[qb][db][i] *= alpha;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) sc[qb][i] -= d;
       }
-      const float mr = m_run[qb];
-      float lsum = l_run[qb];
-#pragma unroll
-      for (int kvb = 0; kvb < 2; ++kvb) {
-#pragma unroll
-        for (int hh = 0; hh < 2; ++hh) {
-          f32x8 p;
-#pragma unroll
-          for (int j = 0; j < 8; ++j)
-            p[j] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[kvb][qb][hh * 8 + j], a.scale_log2, -mr));
-          const bf16x8 pk = __builtin_convertvector(p, bf16x8);
-          pb[qb][kvb * 2 + hh] = pk;
-          // the denominator sums the bf16-rounded numerators the PV product actually uses
-#pragma unroll
-          for (int j = 0; j < 8; j += 2) {
-            const bf16x2 pr = {pk[j], pk[j + 1]};
-            lsum = __builtin_amdgcn_fdot2_f32_bf16(pr, ones, lsum, false);
-          }
-        }
-      }
-      l_run[qb] = lsum;
     }
   };
-
-  // ---- prologue: K(0), K(1), V(0) into the ring
-  put_k(0, fetch(row_entry(t0), pool_k, own_k));
-  put_k(1, fetch(row_entry(t0 + 1), pool_k, own_k));
-  put_v(0, fetch(row_entry(t0), pool_v, own_v));
-  int ek = row_entry(t0 + 2), ev = row_entry(t0 + 1);   // entries of the next pieces to fetch
-  __syncthreads();
-  if (group == 1) __syncthreads();  // puts the second group one phase behind the first
-
-  // matrix phase 0
-  u32x4 kreg = fetch(ek, pool_k, own_k), vreg = fetch(ev, pool_v, own_v);
-  LBM_PRIO_MATRIX_BEGIN;
-  qk(0);
-  LBM_PRIO_MATRIX_END;
-#pragma unroll
-  for (int kvb = 0; kvb < 2; ++kvb)
-#pragma unroll
-    for (int qb = 0; qb < 2; ++qb) pin(s[kvb][qb]);
-  __syncthreads();
-
-  int st_k = 0, st_v = 0;  // stage of K(i) and of V(i)
-  for (int i = 0; i < n; ++i) {
-    const int t = t0 + i;
-    const int trace_i = i; (void)trace_i;
-    LBM_TRACE_POINT(0);
-    // ---- vector phase i: softmax of tile i; land K(i+2), V(i+1) in the ring
-    ek = row_entry(t + 3);
-    ev = row_entry(t + 2);
-#ifndef LBM_SKIP_VECTOR
-    softmax(t);
-#endif
-    int st_k2 = st_k + 2; if (st_k2 >= kStages) st_k2 -= kStages;
-    int st_v1 = st_v + 1; if (st_v1 >= kStages) st_v1 -= kStages;
-    if (i + 2 < n) put_k(st_k2, kreg);
-    if (i + 1 < n) put_v(st_v1, vreg);
+  // Second part: numerators 2^s, packed to bf16; the denominator sums the rounded values.
+  auto soft_exp = [&](const f32x16 (&sc)[2], bf16x8 (&pd)[2][2]) {
+    const bf16x2 ones = {(__bf16)1.0f, (__bf16)1.0f};
 #pragma unroll
     for (int qb = 0; qb < 2; ++qb) {
 #pragma unroll
-      for (int ks = 0; ks < 4; ++ks) pin(pb[qb][ks]);
-      pin(l_run[qb]);
+      for (int kk = 0; kk < 2; ++kk) {
+        f32x8 e;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) e[j] = __builtin_amdgcn_exp2f(sc[qb][kk * 8 + j]);
+        const bf16x8 pk = __builtin_convertvector(e, bf16x8);
+        pd[qb][kk] = pk;
+#pragma unroll
+        for (int j = 0; j < 8; j += 2) {
+          const bf16x2 pr = {pk[j], pk[j + 1]};
+          l_run[qb][j >> 1] = __builtin_amdgcn_fdot2_f32_bf16(pr, ones, l_run[qb][j >> 1], false);
+        }
+      }
     }
-    LBM_TRACE_POINT(1);
-    __syncthreads();
-    LBM_TRACE_POINT(2);
-    // ---- matrix phase i+1: PV of tile i, QK of tile i+1; start fetching K(i+3), V(i+2)
-    kreg = fetch(ek, pool_k, own_k);
-    vreg = fetch(ev, pool_v, own_v);
+  };
+// Scheduling hints for the two regions of a half-step: one MFMA, then `v` vector-ALU
+// instructions, then `d` LDS reads, so that the matrix pipe never waits for the softmax.
+#define LBM_SLOT(v, d)                                               \
+  __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                 \
+  if (v) __builtin_amdgcn_sched_group_barrier(0x002, v, 0);          \
+  if (d) __builtin_amdgcn_sched_group_barrier(0x100, d, 0)
+
+  // ---- prologue: K(0), K(1), V(0) into the ring; the V stage the first PV reads is zeroed
+  put_k(0, fetch(row_entry(t0), pool_k, own_k));
+  put_k(1, fetch(row_entry(t0 + 1), pool_k, own_k));
+  put_v(0, fetch(row_entry(t0), pool_v, own_v));
+  {
+    const u32x4 zero = {0u, 0u, 0u, 0u};
+    put_v(2, zero);
+  }
+#pragma unroll
+  for (int qb = 0; qb < 2; ++qb)
+#pragma unroll
+    for (int kk = 0; kk < 2; ++kk) pB[qb][kk] = __builtin_bit_cast(bf16x8, u32x4{0u, 0u, 0u, 0u});
+  int ek = row_entry(t0 + 2), ev = row_entry(t0 + 1);
+  __syncthreads();
+  qk_half(0, 0, sA);
+  vnext[0] = v_frag(2, 2, 0);
+  vnext[1] = v_frag(2, 2, 1);
+
+  int st_k = 0, st_v = 0, st_vm1 = 2;  // stages of K(i), V(i), V(i-1)
+  for (int i = 0; i < n; ++i) {
+    const int t = t0 + i;
     int st_k1 = st_k + 1; if (st_k1 >= kStages) st_k1 -= kStages;
-    LBM_PRIO_MATRIX_BEGIN;
-#ifndef LBM_SKIP_MATRIX
-    pv(st_v);
-    qk(st_k1);  // on the last tile this reads a stale stage and its result is never used
-    // LDS fragment reads run three steps (of two MFMAs) ahead of the MFMAs that use them:
-    // 8 PV steps with two transpose reads each, then 8 QK steps with one 128-bit read each.
-    __builtin_amdgcn_sched_group_barrier(0x100, 6, 0);
-#pragma unroll
-    for (int step = 0; step < 16; ++step) {
-      __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
-      const int ahead = step + 3;
-      if (ahead < 8) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
-      else if (ahead < 16) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+    int st_k2 = st_k1 + 1; if (st_k2 >= kStages) st_k2 -= kStages;
+    int st_v1 = st_v + 1; if (st_v1 >= kStages) st_v1 -= kStages;
+    const int n_valid = sp.kv_tokens - t * kKvTile;
+
+    // ======== half 0 of tile i: softmax(sA) -> pA | PV(tile i-1, half 1) with pB, QK(tile i, half 1) -> sB
+    // global fetches of K(i+2), V(i+1) start here and land in the ring at the end of the step
+    const u32x4 kreg = fetch(ek, pool_k, own_k);
+    const u32x4 vreg = fetch(ev, pool_v, own_v);
+    ek = row_entry(t + 3);
+    ev = row_entry(t + 2);
+    pv_step(vnext, pB, 0);
+    soft_check(sA, n_valid, i == 0);
+    {
+      bf16x8 va[2] = {v_frag(st_vm1, 3, 0), v_frag(st_vm1, 3, 1)};
+      pv_step(va, pB, 1);
+      qk_half(st_k, 1, sB);
+      soft_exp(sA, pA);
+      vnext[0] = v_frag(st_v, 0, 0);
+      vnext[1] = v_frag(st_v, 0, 1);
+      __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
+      LBM_SLOT(8, 1); LBM_SLOT(8, 1); LBM_SLOT(8, 1); LBM_SLOT(8, 1);   // PV k-step 1
+      LBM_SLOT(8, 1); LBM_SLOT(8, 1);                                   // reference step
+      LBM_SLOT(8, 1); LBM_SLOT(8, 1); LBM_SLOT(8, 0); LBM_SLOT(8, 0);   // K steps 0-1
+      LBM_SLOT(8, 0); LBM_SLOT(8, 0); LBM_SLOT(8, 0); LBM_SLOT(8, 0);   // K steps 2-3
     }
-#endif
-    LBM_PRIO_MATRIX_END;
-#pragma unroll
-    for (int kvb = 0; kvb < 2; ++kvb)
-#pragma unroll
-      for (int qb = 0; qb < 2; ++qb) pin(s[kvb][qb]);
-    LBM_TRACE_POINT(3);
+
+    // ======== half 1 of tile i: softmax(sB) -> pB | PV(tile i, half 0) with pA, QK(tile i+1, half 0) -> sA
+    pv_step(vnext, pA, 0);
+    soft_check(sB, n_valid - 32, false);
+    {
+      bf16x8 va[2] = {v_frag(st_v, 1, 0), v_frag(st_v, 1, 1)};
+      pv_step(va, pA, 1);
+      qk_half(st_k1, 0, sA);  // after the last tile this reads a stale stage; the result is unused
+      soft_exp(sB, pB);
+      vnext[0] = v_frag(st_v, 2, 0);
+      vnext[1] = v_frag(st_v, 2, 1);
+      __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
+      LBM_SLOT(8, 1); LBM_SLOT(8, 1); LBM_SLOT(8, 1); LBM_SLOT(8, 1);
+      LBM_SLOT(8, 1); LBM_SLOT(8, 1);
+      LBM_SLOT(8, 1); LBM_SLOT(8, 1); LBM_SLOT(8, 0); LBM_SLOT(8, 0);
+      LBM_SLOT(8, 0); LBM_SLOT(8, 0); LBM_SLOT(8, 0); LBM_SLOT(8, 0);
+    }
+
+    // ======== ring upkeep: K(i+2), V(i+1) (past the last tile: stages nobody reads any more)
+    put_k(st_k2, kreg);
+    put_v(st_v1, vreg);
     __syncthreads();
-    LBM_TRACE_POINT(4);
     st_k = st_k1;
+    st_vm1 = st_v;
     st_v = st_v1;
   }
-  if (group == 0) __syncthreads();  // both groups pass the same number of barriers
+  // PV of the last half: pB with half 1 of V(n-1), whose first k-step is already in vnext
+  {
+    pv_step(vnext, pB, 0);
+    bf16x8 va[2] = {v_frag(st_vm1, 3, 0), v_frag(st_vm1, 3, 1)};
+    pv_step(va, pB, 1);
+  }
+#undef LBM_SLOT
 
   // ---- epilogue
 #pragma unroll
   for (int qb = 0; qb < 2; ++qb) {
     const int r = q_row0 + qb * 32 + n32;
-    const float l_tot = swap_sum(l_run[qb]);
+    const float l_tot = swap_sum((l_run[qb][0] + l_run[qb][1]) + (l_run[qb][2] + l_run[qb][3]));
     const float inv = l_tot > 0.f ? 1.0f / l_tot : 0.f;
     if (r >= sp.q_rows) continue;
     if (sp.n_splits == 1) {
@@ -405,7 +411,7 @@ __global__ __launch_bounds__(kThreads, 1) void lbm_attn_bf16_d64_kernel(AttnArgs
         }
     } else {
       const size_t prow = ((size_t)sp.part_begin + (size_t)split * sp.q_rows + r) * H + head;
-      float* po = a.part_o + prow * 64;
+      unsigned short* po = a.part_o + prow * 64;
 #pragma unroll
       for (int db = 0; db < 2; ++db)
 #pragma unroll
@@ -413,7 +419,7 @@ __global__ __launch_bounds__(kThreads, 1) void lbm_attn_bf16_d64_kernel(AttnArgs
           f32x4 w;
 #pragma unroll
           for (int e = 0; e < 4; ++e) w[e] = o[qb][db][c4 * 4 + e] * inv;
-          *(f32x4*)(po + db * 32 + c4 * 8 + g * 4) = w;
+          *(bf16x4*)(po + db * 32 + c4 * 8 + g * 4) = __builtin_convertvector(w, bf16x4);
         }
       if (g == 0) a.part_lse[prow] = m_run[qb] + __builtin_amdgcn_logf(l_tot);
     }
@@ -421,35 +427,38 @@ __global__ __launch_bounds__(kThreads, 1) void lbm_attn_bf16_d64_kernel(AttnArgs
 }
 
 // Merge split-KV partial results: out = sum_s w_s * o_s with w_s = 2^(lse_s - max) / sum.
-// One thread per (query row, head, 4 consecutive d).
+// One thread per (query row, head, 8 consecutive d).
 __global__ __launch_bounds__(256) void lbm_attn_combine_bf16_kernel(AttnArgs a) {
   const LbmAttnStreamPlan sp = a.sch.s[blockIdx.y];
   if (sp.n_splits <= 1) return;
   const int H = a.num_heads;
   const long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x;
-  if (idx >= (long long)sp.q_rows * H * 16) return;
-  const int d4 = (int)(idx & 15);
-  const long long rh = idx >> 4;  // r * H + h
+  if (idx >= (long long)sp.q_rows * H * 8) return;
+  const int d8 = (int)(idx & 7);
+  const long long rh = idx >> 3;  // r * H + h
   const long long split_stride = (long long)sp.q_rows * H;
   const float* lse = a.part_lse + (long long)sp.part_begin * H + rh;
   float mx = -INFINITY;
   for (int s = 0; s < sp.n_splits; ++s) mx = fmaxf(mx, lse[s * split_stride]);
   float wsum = 0.f;
-  f32x4 acc = {0.f, 0.f, 0.f, 0.f};
-  const float* po = a.part_o + ((long long)sp.part_begin * H + rh) * 64 + d4 * 4;
+  f32x8 acc;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) acc[e] = 0.f;
+  const unsigned short* po = a.part_o + ((long long)sp.part_begin * H + rh) * 64 + d8 * 8;
   for (int s = 0; s < sp.n_splits; ++s) {
     const float w = __builtin_amdgcn_exp2f(lse[s * split_stride] - mx);
-    const f32x4 v = *(const f32x4*)(po + s * split_stride * 64);
+    const bf16x8 v = *(const bf16x8*)(po + s * split_stride * 64);
+    const f32x8 vf = __builtin_convertvector(v, f32x8);
     wsum += w;
 #pragma unroll
-    for (int e = 0; e < 4; ++e) acc[e] += w * v[e];
+    for (int e = 0; e < 8; ++e) acc[e] += w * vf[e];
   }
   const float inv = 1.0f / wsum;
   const long long r = rh / H, h = rh % H;
-  unsigned short* op = a.out + ((size_t)(sp.q_begin + r) * H + h) * 64 + d4 * 4;
+  unsigned short* op = a.out + ((size_t)(sp.q_begin + r) * H + h) * 64 + d8 * 8;
 #pragma unroll
-  for (int e = 0; e < 4; ++e) acc[e] *= inv;
-  *(bf16x4*)op = __builtin_convertvector(acc, bf16x4);
+  for (int e = 0; e < 8; ++e) acc[e] *= inv;
+  *(bf16x8*)op = __builtin_convertvector(acc, bf16x8);
 }
 
 // ---------------------------------------------------------------------------- schedule
@@ -495,7 +504,8 @@ void lbm_attn_schedule(const lbm_attn_stream* streams, int n_streams, int num_he
 }
 
 size_t lbm_attn_schedule_bytes(const LbmAttnSchedule& sch, int num_heads, int head_dim) {
-  return (size_t)sch.part_rows * num_heads * (head_dim + 1) * sizeof(float);
+  // bf16 partial outputs followed by one float log-sum-exp per (row, head)
+  return (size_t)sch.part_rows * num_heads * (head_dim * 2 + 4);
 }
 
 int lbm_launch_attention(const void* q, const void* pool, void* out, const void* self_k,
@@ -511,8 +521,8 @@ int lbm_launch_attention(const void* q, const void* pool, void* out, const void*
   a.self_k = (const unsigned short*)self_k;
   a.self_v = (const unsigned short*)self_v;
   a.kv_rows = kv_rows;
-  a.part_o = (float*)workspace;
-  a.part_lse = a.part_o + (size_t)sch.part_rows * num_heads * head_dim;
+  a.part_o = (unsigned short*)workspace;
+  a.part_lse = (float*)(a.part_o + (size_t)sch.part_rows * num_heads * head_dim);
   a.num_heads = num_heads;
   a.page_size = page_size;
   a.scale_log2 = sm_scale * 1.4426950408889634f;
@@ -525,7 +535,7 @@ int lbm_launch_attention(const void* q, const void* pool, void* out, const void*
     int max_rows = 0;
     for (int i = 0; i < sch.n_streams; ++i)
       if (sch.s[i].n_splits > 1 && sch.s[i].q_rows > max_rows) max_rows = sch.s[i].q_rows;
-    const long long threads = (long long)max_rows * num_heads * 16;
+    const long long threads = (long long)max_rows * num_heads * 8;
     hipLaunchKernelGGL(lbm_attn_combine_bf16_kernel, dim3((unsigned)((threads + 255) / 256), sch.n_streams),
                        dim3(256), 0, stream, a);
     rc = lbm_check_launch("lbm_attn_combine_bf16_kernel");

@@ -55,7 +55,7 @@ def test_host_side_argument_checks_need_no_gpu():
     assert N.lib.lbm_tables_words(C.byref(bad)) == 0
     s = (N.AttnStream * 1)(N.AttnStream(0, 1004, 0, 17068))
     # 4 query tiles x 16 heads x 8 splits = 512 workgroups -> 8 partial results per row
-    assert N.lib.lbm_attn_workspace_bytes(s, 1, 16, 64) == 8 * 1004 * 16 * 65 * 4
+    assert N.lib.lbm_attn_workspace_bytes(s, 1, 16, 64) == 8 * 1004 * 16 * (64 * 2 + 4)
     s1 = (N.AttnStream * 1)(N.AttnStream(0, 8, 0, 64))
     assert N.lib.lbm_attn_workspace_bytes(s1, 1, 16, 64) == 0
     rc = N.lib.lbm_attn_run(None, None, None, None, None, None, s, 1, 16, 64, 16, 0, 0.125, None, 0, None)
