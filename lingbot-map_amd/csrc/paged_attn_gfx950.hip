@@ -236,7 +236,10 @@ __global__ __launch_bounds__(kThreads, 1) void lbm_attn_bf16_d64_kernel(AttnArgs
   };
   // First part of the softmax of one half: mask, row maxima, and - on the first half of the
   // split or when a score exceeds the reference by more than kTau - move the reference.
-  auto soft_check = [&](f32x16 (&sc)[2], int n_valid, bool first) {
+  // Everything already expressed relative to the old reference is rescaled: O, the row
+  // sums, these scores, and `pend`, the numerators whose second k-step is still to be
+  // multiplied into O.
+  auto soft_check = [&](f32x16 (&sc)[2], bf16x8 (&pend)[2][2], int n_valid, bool first) {
     if (n_valid < 32) {
 #pragma unroll
       for (int i = 0; i < 16; ++i) {
@@ -280,6 +283,11 @@ __global__ __launch_bounds__(kThreads, 1) void lbm_attn_bf16_d64_kernel(AttnArgs
           for (int i = 0; i < 16; ++i) o[qb][db][i] *= alpha;
 #pragma unroll
         for (int i = 0; i < 16; ++i) sc[qb][i] -= d;
+        // the second k-step of the previous half's numerators has not been folded into O yet
+        f32x8 pf = __builtin_convertvector(pend[qb][1], f32x8);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) pf[j] *= alpha;
+        pend[qb][1] = __builtin_convertvector(pf, bf16x8);
       }
     }
   };
@@ -343,7 +351,7 @@ __global__ __launch_bounds__(kThreads, 1) void lbm_attn_bf16_d64_kernel(AttnArgs
     ek = row_entry(t + 3);
     ev = row_entry(t + 2);
     pv_step(vnext, pB, 0);
-    soft_check(sA, n_valid, i == 0);
+    soft_check(sA, pB, n_valid, i == 0);
     {
       bf16x8 va[2] = {v_frag(st_vm1, 3, 0), v_frag(st_vm1, 3, 1)};
       pv_step(va, pB, 1);
@@ -360,7 +368,7 @@ __global__ __launch_bounds__(kThreads, 1) void lbm_attn_bf16_d64_kernel(AttnArgs
 
     // ======== half 1 of tile i: softmax(sB) -> pB | PV(tile i, half 0) with pA, QK(tile i+1, half 0) -> sA
     pv_step(vnext, pA, 0);
-    soft_check(sB, n_valid - 32, false);
+    soft_check(sB, pA, n_valid - 32, false);
     {
       bf16x8 va[2] = {v_frag(st_v, 1, 0), v_frag(st_v, 1, 1)};
       pv_step(va, pA, 1);
@@ -461,6 +469,126 @@ __global__ __launch_bounds__(256) void lbm_attn_combine_bf16_kernel(AttnArgs a) 
   *(bf16x8*)op = __builtin_convertvector(acc, bf16x8);
 }
 
+// ---------------------------------------------------------------------------- fp32 path
+// Same contract as the bf16 kernel for pools kept in fp32 (the reference's force_fp32 mode,
+// lingbot_map/layers/flashinfer_cache.py:118-127,372-383).  Accuracy path, not a speed path:
+// plain fp32 FMAs, one workgroup per (64 query rows, head), four threads per query row that
+// each own 16 of the 64 head dimensions; exact running maximum, no split-KV.
+namespace {
+constexpr int kF32Rows = 64;
+constexpr int kF32Tile = 64;
+struct AttnArgsF32 {
+  const float* q;
+  const float* pool;
+  float* out;
+  const float* self_k;
+  const float* self_v;
+  const int32_t* kv_rows;
+  int num_heads;
+  int page_size;
+  float scale_log2;
+  int n_streams;
+  lbm_attn_stream s[LBM_MAX_STREAMS];
+  int wg_begin[LBM_MAX_STREAMS + 1];
+};
+}  // namespace
+
+__global__ __launch_bounds__(256) void lbm_attn_f32_d64_kernel(AttnArgsF32 a) {
+  __shared__ __attribute__((aligned(16))) float lds_k[kF32Tile][64];
+  __shared__ __attribute__((aligned(16))) float lds_v[kF32Tile][64];
+  const int tid = threadIdx.x;
+  int b = 0;
+  for (int i = 1; i < a.n_streams; ++i)
+    if ((int)blockIdx.x >= a.wg_begin[i]) b = i;
+  const lbm_attn_stream sp = a.s[b];
+  const int H = a.num_heads;
+  const int local = (int)blockIdx.x - a.wg_begin[b];
+  const int head = local % H, qt = local / H;
+  const int r = qt * kF32Rows + (tid >> 2), c = tid & 3;  // query row, quarter of the head dim
+  const size_t row_elems = (size_t)H * 64;
+  const bool row_ok = r < sp.q_rows;
+
+  float q[16], o[16];
+  {
+    const float* qp = a.q + ((size_t)(sp.q_begin + (row_ok ? r : 0)) * H + head) * 64 + c * 16;
+#pragma unroll
+    for (int d = 0; d < 16; ++d) {
+      q[d] = row_ok ? qp[d] * a.scale_log2 : 0.f;
+      o[d] = 0.f;
+    }
+  }
+  float m = -INFINITY, l = 0.f;
+
+  const int ld_r = tid >> 2, ld_c = (tid & 3) * 16;  // each thread stages 16 floats of one K and V row
+  const int n_tiles = (sp.kv_tokens + kF32Tile - 1) / kF32Tile;
+  for (int t = 0; t < n_tiles; ++t) {
+    const int kvi = t * kF32Tile + ld_r;
+    f32x4 kk[4], vv[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) kk[i] = vv[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+    if (kvi < sp.kv_tokens) {
+      const int e = a.kv_rows[sp.kv_row_begin + kvi];
+      const float *kp, *vp;
+      if (e >= 0) {
+        kp = a.pool + ((size_t)e * H + head) * 64 + ld_c;
+        vp = kp + (size_t)a.page_size * row_elems;
+      } else {
+        const size_t off = ((size_t)(-1 - e) * H + head) * 64 + ld_c;
+        kp = a.self_k + off;
+        vp = a.self_v + off;
+      }
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        kk[i] = ((const f32x4*)kp)[i];
+        vv[i] = ((const f32x4*)vp)[i];
+      }
+    }
+    __syncthreads();  // the previous tile is no longer being read
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      *(f32x4*)&lds_k[ld_r][ld_c + 4 * i] = kk[i];
+      *(f32x4*)&lds_v[ld_r][ld_c + 4 * i] = vv[i];
+    }
+    __syncthreads();
+    const int n_valid = min(kF32Tile, sp.kv_tokens - t * kF32Tile);
+    for (int j0 = 0; j0 < n_valid; j0 += 8) {
+      float sc[8];
+#pragma unroll
+      for (int jj = 0; jj < 8; ++jj) {
+        const int j = j0 + jj;
+        float acc = 0.f;
+#pragma unroll
+        for (int d = 0; d < 16; ++d) acc = __builtin_fmaf(q[d], lds_k[j][c * 16 + d], acc);
+        acc += __shfl_xor(acc, 1);
+        acc += __shfl_xor(acc, 2);
+        sc[jj] = j < n_valid ? acc : -INFINITY;
+      }
+      float mx = m;
+#pragma unroll
+      for (int jj = 0; jj < 8; ++jj) mx = fmaxf(mx, sc[jj]);
+      const float alpha = exp2f(m - mx);  // m = -inf on the first step gives 0
+      m = mx;
+      l *= alpha;
+#pragma unroll
+      for (int d = 0; d < 16; ++d) o[d] *= alpha;
+#pragma unroll
+      for (int jj = 0; jj < 8; ++jj) {
+        const float p = exp2f(sc[jj] - m);
+        l += p;
+        const int j = min(j0 + jj, kF32Tile - 1);
+#pragma unroll
+        for (int d = 0; d < 16; ++d) o[d] = __builtin_fmaf(p, lds_v[j][c * 16 + d], o[d]);
+      }
+    }
+  }
+  if (row_ok) {
+    const float inv = l > 0.f ? 1.0f / l : 0.f;
+    float* op = a.out + ((size_t)(sp.q_begin + r) * H + head) * 64 + c * 16;
+#pragma unroll
+    for (int d = 0; d < 16; ++d) op[d] = o[d] * inv;
+  }
+}
+
 // ---------------------------------------------------------------------------- schedule
 void lbm_attn_schedule(const lbm_attn_stream* streams, int n_streams, int num_heads,
                        LbmAttnSchedule* out) {
@@ -512,8 +640,35 @@ int lbm_launch_attention(const void* q, const void* pool, void* out, const void*
                          const void* self_v, const int32_t* kv_rows, const LbmAttnSchedule& sch,
                          int num_heads, int head_dim, int page_size, int dtype, float sm_scale,
                          void* workspace, hipStream_t stream) {
-  if (dtype != LBM_DTYPE_BF16 || head_dim != 64)
-    return lbm_fail(LBM_ERR_UNSUPPORTED, "attention kernel covers bf16 with head_dim 64 (got dtype %d, head_dim %d)", dtype, head_dim);
+  if (head_dim != 64)
+    return lbm_fail(LBM_ERR_UNSUPPORTED, "attention kernels cover head_dim 64 (got %d)", head_dim);
+  if (dtype == LBM_DTYPE_F32) {
+    AttnArgsF32 f;
+    f.q = (const float*)q;
+    f.pool = (const float*)pool;
+    f.out = (float*)out;
+    f.self_k = (const float*)self_k;
+    f.self_v = (const float*)self_v;
+    f.kv_rows = kv_rows;
+    f.num_heads = num_heads;
+    f.page_size = page_size;
+    f.scale_log2 = sm_scale * 1.4426950408889634f;
+    f.n_streams = sch.n_streams;
+    int wg = 0;
+    for (int i = 0; i < LBM_MAX_STREAMS; ++i) {
+      f.s[i] = lbm_attn_stream{0, 0, 0, 0};
+      f.wg_begin[i] = wg;
+      if (i < sch.n_streams) {
+        f.s[i] = lbm_attn_stream{sch.s[i].q_begin, sch.s[i].q_rows, sch.s[i].kv_row_begin, sch.s[i].kv_tokens};
+        wg += ((sch.s[i].q_rows + kF32Rows - 1) / kF32Rows) * num_heads;
+      }
+    }
+    f.wg_begin[LBM_MAX_STREAMS] = wg;
+    if (wg == 0) return LBM_OK;
+    hipLaunchKernelGGL(lbm_attn_f32_d64_kernel, dim3(wg), dim3(256), 0, stream, f);
+    return lbm_check_launch("lbm_attn_f32_d64_kernel");
+  }
+  if (dtype != LBM_DTYPE_BF16) return lbm_fail(LBM_ERR_INVALID, "unknown dtype %d", dtype);
   AttnArgs a;
   a.q = (const unsigned short*)q;
   a.pool = (const unsigned short*)pool;

@@ -94,6 +94,15 @@ class HipPagedKVCacheManager:
         assert page_size > 0
         self.page_size = page_size
         self.scale_frames = scale_frames
+        # one window for all streams, or one per stream (ragged batch)
+        if isinstance(sliding_window, (list, tuple)):
+            assert len(sliding_window) == num_streams, "one sliding_window per stream"
+            self._windows = [int(w) for w in sliding_window]
+            self._ragged_windows = True
+            sliding_window = max(self._windows)
+        else:
+            self._windows = [int(sliding_window)] * num_streams
+            self._ragged_windows = False
         self.sliding_window = sliding_window
         self.num_heads = num_heads
         self.head_dim = head_dim
@@ -199,6 +208,11 @@ class HipPagedKVCacheManager:
 
     def _visible_tokens(self, c: _StreamCounts) -> int:
         return (c.n_anchor + c.win_count) * self._tpf + c.special_tokens
+
+    def _window_of(self, stream: int, requested: int) -> int:
+        """Window of one stream: the caller's value (as in the reference), or the stream's own
+        window when the manager was built with one window per stream."""
+        return self._windows[stream] if self._ragged_windows else requested
 
     def _keep_tokens(self, cross_frame_special: bool, camera_only: bool) -> int:
         # lingbot_map/layers/attention.py:690-696
@@ -319,12 +333,13 @@ class HipPagedKVCacheManager:
         todo = False
         for b in range(self.num_streams):
             c = self._counts[ts][b]
-            if self._active[b] and c.win_count > sliding_window:
-                self._mirror_evict(c, sliding_window, keep, block_idx)
+            w = self._window_of(b, sliding_window)
+            if self._active[b] and c.win_count > w:
+                self._mirror_evict(c, w, keep, block_idx)
                 todo = True
         if not todo:
             return
-        ops = self._ops([{"ops": N.OP_EVICT if self._active[b] else 0, "sliding_window": sliding_window,
+        ops = self._ops([{"ops": N.OP_EVICT if self._active[b] else 0, "sliding_window": self._window_of(b, sliding_window),
                           "keep_tokens": keep} for b in range(self.num_streams)])
         self._tables_step(ts, ops)
         self._plan_valid[ts] = False
@@ -400,14 +415,14 @@ class HipPagedKVCacheManager:
                     self._mirror_append(c, block_idx)
                     ops = N.OP_APPEND | N.OP_PLAN
                     if not self._defer_eviction:
-                        self._mirror_evict(c, self.sliding_window, keep, block_idx)
+                        self._mirror_evict(c, self._windows[b], keep, block_idx)
                         ops |= N.OP_EVICT
                     n = self._visible_tokens(c)
                 elif tail[b]:
                     ops = N.OP_PLAN
                     n = self._visible_tokens(c) + self.tokens_per_frame
                 self._plan_tokens[ts][b] = n
-                per.append({"ops": ops, "sliding_window": self.sliding_window, "keep_tokens": keep,
+                per.append({"ops": ops, "sliding_window": self._windows[b], "keep_tokens": keep,
                             "self_tokens": self.tokens_per_frame if tail[b] else 0, "expect_kv_tokens": n})
             self._tables_step(ts, self._ops(per), append_rows=True, kv_rows=True)
             self._plan_valid[ts] = True

@@ -132,6 +132,34 @@ def test_attention_read_only_tail_and_two_streams():
     check_bf16(out[T:], ref1)
 
 
+@pytest.mark.parametrize("order", ["rising", "falling", "spikes"])
+def test_attention_moving_reference_maximum(order):
+    """Scores whose maximum keeps rising along the KV axis force the kernel to move its
+    softmax reference late and often; falling scores and isolated spikes cover the other
+    orders.  (A reference move has to rescale everything expressed in the old reference.)
+    Logits stay within +-20 so that the absolute bf16 tolerance still applies."""
+    from oracle.sdpa_cache import sdpa_nhd
+    dev = torch.device("cuda:0")
+    g = torch.Generator().manual_seed(17)
+    tq, H, D, S, n_kv = 200, 4, 64, 16, 4096
+    q = torch.randn(tq, H, D, generator=g).to(torch.bfloat16)
+    k = torch.randn(n_kv, H, D, generator=g)
+    v = torch.randn(n_kv, H, D, generator=g).to(torch.bfloat16)
+    ramp = torch.linspace(0.1, 2.5, n_kv).view(n_kv, 1, 1)
+    if order == "falling":
+        ramp = ramp.flip(0)
+    if order == "spikes":
+        ramp = torch.full((n_kv, 1, 1), 0.1)
+        ramp[torch.randperm(n_kv, generator=g)[:40]] = 2.5
+    k = (k * ramp).to(torch.bfloat16)
+    pool = torch.zeros(n_kv // S, 2, S, H, D, dtype=torch.bfloat16)
+    pool[:, 0] = k.view(n_kv // S, S, H, D)
+    pool[:, 1] = v.view(n_kv // S, S, H, D)
+    rows, n_tok = rows_from_pages(list(range(n_kv // S)), [S] * (n_kv // S), S, dev)
+    out = run_attention(q.to(dev), pool.to(dev), rows, [(0, tq, 0, n_tok)], S)
+    check_bf16(out.cpu(), sdpa_nhd(q, k, v))
+
+
 def test_attention_closed_forms():
     dev = torch.device("cuda:0")
     H, D, S = 2, 64, 16
