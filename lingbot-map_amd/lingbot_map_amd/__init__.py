@@ -6,6 +6,7 @@
 if it has not been built: there is no CPU path.
 """
 from . import _native  # noqa: F401  (loads the library, fails loudly when missing)
+from .block import HipPagedAttention, HipPagedBlock, keyframe_flags, set_skip_append
 from .manager import HipPagedKVCacheManager
 
-__all__ = ["HipPagedKVCacheManager"]
+__all__ = ["HipPagedKVCacheManager", "HipPagedAttention", "HipPagedBlock", "keyframe_flags", "set_skip_append"]

@@ -1,0 +1,224 @@
+"""Global-attention block on the HIP paged KV cache.
+
+``HipPagedAttention`` / ``HipPagedBlock`` stand next to the reference's
+``FlashInferAttention`` / ``FlashInferBlock`` and ``SDPAAttention`` / ``SDPABlock``
+(lingbot_map/layers/attention.py:352-556, lingbot_map/layers/block.py:151-310, :461-532):
+same constructor arguments, same sub-module names (``norm1``, ``attn.qkv``, ``attn.q_norm``,
+``attn.k_norm``, ``attn.proj``, ``ls1``, ``norm2``, ``mlp.fc1``, ``mlp.fc2``, ``ls2``) so a
+reference state dict loads, the same ``forward`` signature, and the ``attn_pre`` /
+``ffn_residual`` / ``attn.proj`` / ``attn.kv_cache_*`` attributes the reference's
+compile recipe reaches into (gct_profile.py:51-56).
+
+Differences, all inside the streaming branch:
+
+* a keyframe's append, eviction and visible-row table are one index-kernel launch
+  (``manager.step``) instead of three host-side list updates plus table uploads;
+* a non-keyframe attends to the cache plus its own K/V read directly from the projection
+  output; the reference appends, attends and rolls back (block.py:257-263), which writes
+  8 MB per layer that no later frame reads.
+
+Any manager with the reference call surface works: when ``kv_cache`` lacks ``step`` the
+reference's method-by-method sequence is used.
+"""
+from __future__ import annotations
+
+from typing import Callable, Optional
+
+import torch
+import torch.nn.functional as F
+from torch import Tensor, nn
+
+
+def apply_rotary_emb(x: Tensor, freqs: Tensor) -> Tensor:
+    """Rotate interleaved (even, odd) pairs of ``x`` ``[B, H, N, D]`` by the complex
+    ``freqs`` ``[1, 1, N, D/2]`` (lingbot_map/layers/rope.py:435-461)."""
+    cos, sin = freqs.real.to(x.dtype), freqs.imag.to(x.dtype)
+    x1, x2 = x[..., 0::2], x[..., 1::2]
+    return torch.stack([x1 * cos - x2 * sin, x1 * sin + x2 * cos], dim=-1).reshape(x.shape)
+
+
+class LayerScale(nn.Module):
+    """lingbot_map/layers/layer_scale.py"""
+
+    def __init__(self, dim: int, init_values: float = 1e-5) -> None:
+        super().__init__()
+        self.gamma = nn.Parameter(init_values * torch.ones(dim))
+
+    def forward(self, x: Tensor) -> Tensor:
+        return x * self.gamma
+
+
+class Mlp(nn.Module):
+    """lingbot_map/layers/mlp.py (dropout omitted: inference only)"""
+
+    def __init__(self, in_features: int, hidden_features: Optional[int] = None, act_layer=nn.GELU,
+                 drop: float = 0.0, bias: bool = True) -> None:
+        super().__init__()
+        hidden_features = hidden_features or in_features
+        self.fc1 = nn.Linear(in_features, hidden_features, bias=bias)
+        self.act = act_layer()
+        self.fc2 = nn.Linear(hidden_features, in_features, bias=bias)
+
+    def forward(self, x: Tensor) -> Tensor:
+        return self.fc2(self.act(self.fc1(x)))
+
+
+class HipPagedAttention(nn.Module):
+    def __init__(self, dim: int, num_heads: int = 8, qkv_bias: bool = True, proj_bias: bool = True,
+                 attn_drop: float = 0.0, proj_drop: float = 0.0, norm_layer: Callable[..., nn.Module] = nn.LayerNorm,
+                 qk_norm: bool = False, fused_attn: bool = True, rope=None,
+                 kv_cache_sliding_window: int = 64, kv_cache_scale_frames: int = 8,
+                 kv_cache_cross_frame_special: bool = True, kv_cache_include_scale_frames: bool = True,
+                 kv_cache_camera_only: bool = False) -> None:
+        super().__init__()
+        assert dim % num_heads == 0, "dim should be divisible by num_heads"
+        self.num_heads = num_heads
+        self.head_dim = dim // num_heads
+        self.qkv = nn.Linear(dim, dim * 3, bias=qkv_bias)
+        self.q_norm = norm_layer(self.head_dim) if qk_norm else nn.Identity()
+        self.k_norm = norm_layer(self.head_dim) if qk_norm else nn.Identity()
+        self.proj = nn.Linear(dim, dim, bias=proj_bias)
+        self.rope = rope
+        self.kv_cache_sliding_window = kv_cache_sliding_window
+        self.kv_cache_scale_frames = kv_cache_scale_frames
+        self.kv_cache_cross_frame_special = kv_cache_cross_frame_special
+        self.kv_cache_include_scale_frames = kv_cache_include_scale_frames
+        self.kv_cache_camera_only = kv_cache_camera_only
+
+    # ------------------------------------------------------------------ projections
+    def _qkv(self, x: Tensor, pos, enable_3d_rope: bool):
+        B, N, _ = x.shape
+        qkv = self.qkv(x).reshape(B, N, 3, self.num_heads, self.head_dim).permute(2, 0, 3, 1, 4)
+        q, k, v = qkv.unbind(0)  # each [B, H, N, D]
+        q, k = self.q_norm(q), self.k_norm(k)
+        if self.rope is not None and not enable_3d_rope:
+            q, k = self.rope(q, pos), self.rope(k, pos)
+        elif self.rope is not None:
+            q, k = apply_rotary_emb(q, pos), apply_rotary_emb(k, pos)
+        return q, k, v
+
+    def prepare_qkv(self, x: Tensor, pos=None, enable_3d_rope: bool = False):
+        """q, k, v of the streamed frame(s) as ``[B * tokens, H, D]``, specials first within
+        each frame (attention.py:402-426; the reference squeezes a batch of one, here the
+        batch axis carries the independent streams of a ragged batch)."""
+        q, k, v = self._qkv(x, pos, enable_3d_rope)
+        B, H, N, D = q.shape
+        nhd = lambda t: t.permute(0, 2, 1, 3).reshape(B * N, H, D).contiguous()
+        return nhd(q), nhd(k), nhd(v)
+
+    # ------------------------------------------------------------------ cache traffic
+    def _evict_kwargs(self, num_register_tokens: int) -> dict:
+        return dict(scale_frames=self.kv_cache_scale_frames, sliding_window=self.kv_cache_sliding_window,
+                    cross_frame_special=self.kv_cache_cross_frame_special,
+                    include_scale_frames=self.kv_cache_include_scale_frames,
+                    camera_only=self.kv_cache_camera_only, num_register_tokens=num_register_tokens)
+
+    def stream_attend(self, manager, global_idx: int, q: Tensor, k: Tensor, v: Tensor,
+                      num_register_tokens: int = 4) -> Tensor:
+        """One streamed frame through the cache: block.py:256-278."""
+        skip_append = getattr(manager, "_skip_append", False)
+        if hasattr(manager, "step"):
+            return manager.step(global_idx, q, k, v, keyframe=None,  # None: follows manager._skip_append
+                                cross_frame_special=self.kv_cache_cross_frame_special,
+                                camera_only=self.kv_cache_camera_only)
+        if skip_append:
+            prev = manager._defer_eviction
+            manager._defer_eviction = True
+            manager.append_frame(global_idx, k, v)
+            out = manager.compute_attention(global_idx, q)
+            manager.rollback_last_frame(global_idx)
+            manager._defer_eviction = prev
+            return out
+        manager.append_frame(global_idx, k, v)
+        manager.evict_frames(block_idx=global_idx, **self._evict_kwargs(num_register_tokens))
+        return manager.compute_attention(global_idx, q)
+
+    def forward(self, x: Tensor, pos=None, num_patches=None, num_special=None, num_frames=None,
+                enable_3d_rope=False, kv_cache=None, global_idx=0, num_frame_per_block=1,
+                num_frame_for_scale=-1, num_register_tokens=4) -> Tensor:
+        B, N, _ = x.shape
+        has_manager = kv_cache is not None and hasattr(kv_cache, "append_frame")
+        if not has_manager:
+            # batch mode (attention.py:446-465)
+            q, k, v = self._qkv(x, pos, enable_3d_rope)
+            out = F.scaled_dot_product_attention(q, k, v).transpose(1, 2).reshape(B, N, -1)
+        elif num_frames is not None and num_frames > 1:
+            # anchor pass over several frames: dense attention among them, then one append
+            # and eviction per frame (attention.py:475-511)
+            assert B == 1, "the multi-frame anchor pass handles one stream"
+            q, k, v = self._qkv(x, pos, enable_3d_rope)
+            out = F.scaled_dot_product_attention(q, k, v).transpose(1, 2).reshape(B, N, -1)
+            tpf = kv_cache.tokens_per_frame
+            k_all, v_all = k.squeeze(0).permute(1, 0, 2), v.squeeze(0).permute(1, 0, 2)
+            for f in range(num_frames):
+                s = f * tpf
+                kv_cache.append_frame(global_idx, k_all[s:s + tpf].contiguous(), v_all[s:s + tpf].contiguous())
+                kv_cache.evict_frames(block_idx=global_idx, **self._evict_kwargs(num_register_tokens))
+        else:
+            q, k, v = self.prepare_qkv(x, pos=pos, enable_3d_rope=enable_3d_rope)
+            out = self.stream_attend(kv_cache, global_idx, q, k, v, num_register_tokens)
+            out = out.reshape(B, N, self.num_heads * self.head_dim).to(x.dtype)
+        return self.proj(out)
+
+
+class HipPagedBlock(nn.Module):
+    def __init__(self, dim: int, num_heads: int, mlp_ratio: float = 4.0, qkv_bias: bool = True,
+                 proj_bias: bool = True, ffn_bias: bool = True, drop: float = 0.0, attn_drop: float = 0.0,
+                 init_values=None, drop_path: float = 0.0, act_layer: Callable[..., nn.Module] = nn.GELU,
+                 norm_layer: Callable[..., nn.Module] = nn.LayerNorm, ffn_layer: Callable[..., nn.Module] = Mlp,
+                 qk_norm: bool = False, rope=None, kv_cache_sliding_window: int = 64,
+                 kv_cache_scale_frames: int = 8, kv_cache_cross_frame_special: bool = True,
+                 kv_cache_include_scale_frames: bool = True, kv_cache_camera_only: bool = False) -> None:
+        super().__init__()
+        self.norm1 = norm_layer(dim)
+        self.attn = HipPagedAttention(
+            dim=dim, num_heads=num_heads, qk_norm=qk_norm, qkv_bias=qkv_bias, proj_bias=proj_bias,
+            attn_drop=attn_drop, proj_drop=drop, rope=rope,
+            kv_cache_sliding_window=kv_cache_sliding_window, kv_cache_scale_frames=kv_cache_scale_frames,
+            kv_cache_cross_frame_special=kv_cache_cross_frame_special,
+            kv_cache_include_scale_frames=kv_cache_include_scale_frames,
+            kv_cache_camera_only=kv_cache_camera_only)
+        self.ls1 = LayerScale(dim, init_values=init_values) if init_values else nn.Identity()
+        self.drop_path1 = nn.Identity()
+        self.norm2 = norm_layer(dim)
+        self.mlp = ffn_layer(in_features=dim, hidden_features=int(dim * mlp_ratio), act_layer=act_layer,
+                             drop=drop, bias=ffn_bias)
+        self.ls2 = LayerScale(dim, init_values=init_values) if init_values else nn.Identity()
+        self.drop_path2 = nn.Identity()
+        self.sample_drop_ratio = drop_path
+
+    def attn_pre(self, x: Tensor, pos=None, enable_3d_rope: bool = False):
+        """norm1 + projections + qk-norm + RoPE, ready for the cache (block.py:217-227)."""
+        return self.attn.prepare_qkv(self.norm1(x), pos=pos, enable_3d_rope=enable_3d_rope)
+
+    def ffn_residual(self, x: Tensor) -> Tensor:
+        return x + self.ls2(self.mlp(self.norm2(x)))
+
+    def forward(self, x: Tensor, pos=None, num_patches=None, num_special=None, num_frames=None,
+                enable_3d_rope=False, kv_cache=None, global_idx=0, num_frame_per_block=1,
+                num_frame_for_scale=-1, num_register_tokens=4) -> Tensor:
+        is_streaming = kv_cache is not None and (num_frames is None or num_frames <= 1)
+        if is_streaming:
+            q, k, v = self.attn_pre(x, pos=pos, enable_3d_rope=enable_3d_rope)
+            attn_x = self.attn.stream_attend(kv_cache, global_idx, q, k, v, num_register_tokens)
+            attn_x = attn_x.reshape(x.shape[0], x.shape[1], self.attn.num_heads * self.attn.head_dim).to(x.dtype)
+            x = x + self.ls1(self.attn.proj(attn_x))
+        else:
+            x = x + self.ls1(self.attn(
+                self.norm1(x), pos=pos, num_patches=num_patches, num_special=num_special, num_frames=num_frames,
+                enable_3d_rope=enable_3d_rope, kv_cache=kv_cache, global_idx=global_idx,
+                num_frame_per_block=num_frame_per_block, num_frame_for_scale=num_frame_for_scale,
+                num_register_tokens=num_register_tokens))
+        return self.ffn_residual(x)
+
+
+def keyframe_flags(num_frames: int, scale_frames: int, keyframe_interval: int):
+    """Which streamed frames are cached (lingbot_map/models/gct_stream.py:450): the anchor
+    frames always, afterwards every ``keyframe_interval``-th frame."""
+    return [i < scale_frames or keyframe_interval <= 1 or (i - scale_frames) % keyframe_interval == 0
+            for i in range(num_frames)]
+
+
+def set_skip_append(manager, skip: bool) -> None:
+    """The driver's non-keyframe switch (lingbot_map/models/gct_stream.py:300-318)."""
+    manager._skip_append = bool(skip)

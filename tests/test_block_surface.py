@@ -1,0 +1,64 @@
+"""Call surface of the block that stands in for the reference's FlashInferBlock (CPU only):
+parameter names a reference state dict carries, the attributes the reference's compile
+recipe reaches into, batch mode without a cache, and the driver's keyframe rule."""
+import torch
+
+
+def make_block(**kw):
+    from lingbot_map_amd import HipPagedBlock
+    args = dict(dim=128, num_heads=2, mlp_ratio=4.0, qkv_bias=True, proj_bias=True, ffn_bias=True, init_values=0.01,
+                qk_norm=True, rope=None, kv_cache_sliding_window=16, kv_cache_scale_frames=1,
+                kv_cache_cross_frame_special=True, kv_cache_include_scale_frames=True, kv_cache_camera_only=False)
+    args.update(kw)
+    return HipPagedBlock(**args)
+
+
+def test_state_dict_keys_match_reference_block():
+    # names from lingbot_map/layers/block.py:183-213 and attention.py:61-67
+    expect = {"norm1.weight", "norm1.bias", "attn.qkv.weight", "attn.qkv.bias", "attn.q_norm.weight",
+              "attn.q_norm.bias", "attn.k_norm.weight", "attn.k_norm.bias", "attn.proj.weight", "attn.proj.bias",
+              "ls1.gamma", "norm2.weight", "norm2.bias", "mlp.fc1.weight", "mlp.fc1.bias", "mlp.fc2.weight",
+              "mlp.fc2.bias", "ls2.gamma"}
+    assert set(make_block().state_dict().keys()) == expect
+
+
+def test_attributes_the_compile_recipe_uses():
+    b = make_block()
+    for name in ("attn_pre", "ffn_residual"):
+        assert callable(getattr(b, name))
+    assert isinstance(b.attn.proj, torch.nn.Linear)
+    assert (b.attn.kv_cache_sliding_window, b.attn.kv_cache_scale_frames) == (16, 1)
+    assert b.attn.kv_cache_cross_frame_special and b.attn.kv_cache_include_scale_frames and not b.attn.kv_cache_camera_only
+
+
+def test_batch_mode_without_cache_is_dense_attention():
+    torch.manual_seed(0)
+    b = make_block().eval()
+    x = torch.randn(2, 11, 128)
+    y = b(x)
+    # the same arithmetic written out
+    h = b.norm1(x)
+    q, k, v = b.attn._qkv(h, None, False)
+    a = torch.softmax(q @ k.transpose(-1, -2) / 8.0, -1) @ v
+    a = b.attn.proj(a.transpose(1, 2).reshape(2, 11, 128))
+    ref = b.ffn_residual(x + b.ls1(a))
+    assert torch.allclose(y, ref, atol=1e-5)
+    q2, k2, v2 = b.attn_pre(x)
+    assert q2.shape == (22, 2, 64) and torch.allclose(q2[11:], q[1].permute(1, 0, 2), atol=1e-6)
+
+
+def test_rotary_matches_complex_multiplication():
+    from lingbot_map_amd.block import apply_rotary_emb
+    x = torch.randn(1, 2, 5, 8)
+    ang = torch.randn(1, 1, 5, 4)
+    freqs = torch.polar(torch.ones_like(ang), ang)
+    ref = torch.view_as_real(torch.view_as_complex(x.reshape(1, 2, 5, 4, 2)) * freqs).reshape(1, 2, 5, 8)
+    assert torch.allclose(apply_rotary_emb(x, freqs), ref, atol=1e-6)
+
+
+def test_keyframe_flags_follow_driver_rule():
+    from lingbot_map_amd import keyframe_flags
+    # lingbot_map/models/gct_stream.py:450 with 1 anchor frame and interval 4
+    assert keyframe_flags(10, 1, 4) == [True, True, False, False, False, True, False, False, False, True]
+    assert sum(keyframe_flags(320, 1, 4)) == 81
+    assert all(keyframe_flags(20, 8, 1))

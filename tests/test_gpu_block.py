@@ -1,0 +1,76 @@
+"""The streaming branch of the block on the GPU: outputs against the same block evaluated
+with a dense dict cache (the reference SDPA path's semantics) and torch SDPA in fp32."""
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+
+class ReferenceSurfaceOnly:
+    """Hides everything but the reference manager's call surface
+    (lingbot_map/layers/flashinfer_cache.py:202-560)."""
+
+    def __init__(self, m):
+        object.__setattr__(self, "_m", m)
+
+    def __getattr__(self, name):
+        if name in ("step", "set_active_streams"):
+            raise AttributeError(name)
+        return getattr(self._m, name)
+
+    def __setattr__(self, name, value):
+        setattr(self._m, name, value)
+
+
+@pytest.mark.parametrize("reference_calls", [False, True])
+def test_block_stream_matches_dense_cache(reference_calls):
+    from lingbot_map_amd import HipPagedBlock, HipPagedKVCacheManager, keyframe_flags, set_skip_append
+    from oracle.sdpa_cache import DictCacheOracle
+    torch.manual_seed(5)
+    dev = torch.device("cuda:0")
+    dim, H, T, n_sp, scale, window, blocks = 256, 4, 53, 5, 1, 3, 2
+    mods = [HipPagedBlock(dim, H, init_values=0.1, qk_norm=True, kv_cache_sliding_window=window,
+                          kv_cache_scale_frames=scale).to(dev, torch.bfloat16).eval() for _ in range(blocks)]
+    m = HipPagedKVCacheManager(blocks, scale + window + 16, T, H, 64, torch.bfloat16, dev, num_special_tokens=n_sp,
+                               scale_frames=scale, sliding_window=window, max_total_frames=64, page_size=16,
+                               layout="frame_pages")
+    cache = ReferenceSurfaceOnly(m) if reference_calls else m
+    dense = [DictCacheOracle(scale, window, n_sp) for _ in range(blocks)]
+    flags = keyframe_flags(14, scale, 3)
+    with torch.no_grad():
+        for f, kf in enumerate(flags):
+            x = torch.randn(1, T, dim, device=dev).to(torch.bfloat16)
+            set_skip_append(cache, not kf)
+            y, y_ref = x, x
+            for b, mod in enumerate(mods):
+                y = mod(y, kv_cache=cache, global_idx=b, num_frames=1)
+                q, k, v = mod.attn_pre(y_ref)
+                kk, vv = dense[b].visible(k, v, keyframe=kf)
+                a = torch.nn.functional.scaled_dot_product_attention(
+                    q.float().permute(1, 0, 2)[None], kk.float().permute(1, 0, 2)[None], vv.float().permute(1, 0, 2)[None])
+                a = a[0].permute(1, 0, 2).reshape(1, T, dim).to(torch.bfloat16)
+                y_ref = mod.ffn_residual(y_ref + mod.ls1(mod.attn.proj(a)))
+            set_skip_append(cache, False)
+            err = (y.float() - y_ref.float()).abs()
+            assert err.max().item() <= 3e-2 and err.mean().item() <= 2e-3, (f, err.max().item(), err.mean().item())
+    assert m.frame_count == [sum(flags)] * blocks and m.device_header()["error"] == 0
+
+
+def test_two_streams_through_one_block():
+    from lingbot_map_amd import HipPagedBlock, HipPagedKVCacheManager
+    torch.manual_seed(6)
+    dev = torch.device("cuda:0")
+    dim, H, T = 256, 4, 53
+    mod = HipPagedBlock(dim, H, qk_norm=True, kv_cache_sliding_window=2, kv_cache_scale_frames=1).to(dev, torch.bfloat16).eval()
+    both = HipPagedKVCacheManager(1, 19, T, H, 64, torch.bfloat16, dev, num_special_tokens=5, scale_frames=1,
+                                  sliding_window=2, max_total_frames=32, page_size=16, layout="frame_pages", num_streams=2)
+    single = [HipPagedKVCacheManager(1, 19, T, H, 64, torch.bfloat16, dev, num_special_tokens=5, scale_frames=1,
+                                     sliding_window=2, max_total_frames=32, page_size=16, layout="frame_pages")
+              for _ in range(2)]
+    with torch.no_grad():
+        for f in range(6):
+            x = torch.randn(2, T, dim, device=dev).to(torch.bfloat16)
+            y = mod(x, kv_cache=both, global_idx=0, num_frames=1)
+            for s in range(2):
+                ys = mod(x[s:s + 1], kv_cache=single[s], global_idx=0, num_frames=1)
+                assert (y[s:s + 1].float() - ys.float()).abs().max().item() <= 1e-2
