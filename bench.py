@@ -25,7 +25,35 @@ T, N_SPECIAL, H, D, PAGE = 1004, 5, 16, 64, 16
 ANCHOR, WINDOW = 1, 16
 PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA
 PEAK_HBM_GBPS = 8000.0
+# HBM bytes of one lbm_attn_bf16_d64_kernel launch at this workload, from rocprofv3 --pmc
+# FETCH_SIZE (x2.0, the factor a 256 MiB plain copy gives) and WRITE_SIZE (x1.0), in KiB:
+# 35,492 * 2 + 20,082 KiB  (profiles/attention_config2_hbm_traffic.md)
+ATTN_TRAFFIC_BYTES = (35492.0 * 2.0 + 20082.0) * 1024.0
 METRIC = "frames/sec streaming @518x378 (1 GPU); attention TFLOPS & % bf16 MFMA peak"
+
+
+def kernel_time_ms(fn, iters: int, torch) -> float:
+    """Average GPU time of one fn() launch in ms for kernels shorter than the host's launch
+    overhead: `iters` launches are captured into one HIP graph, the graph is replayed and
+    timed with a HIP event pair on the launch stream, so the launches run back to back."""
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        fn()  # warm up outside capture
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=side):
+            for _ in range(iters):
+                fn()
+        start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        graph.replay()
+        side.synchronize()
+        start.record(side)
+        for _ in range(4):
+            graph.replay()
+        stop.record(side)
+        stop.synchronize()
+    torch.cuda.current_stream().wait_stream(side)
+    return start.elapsed_time(stop) / (4 * iters)
 
 
 def event_time_ms(fn, iters: int, torch) -> float:
@@ -81,9 +109,10 @@ def main() -> None:
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--blocks", type=int, default=24)
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--mode", choices=["full", "attention", "append", "tables"], default="full",
-                    help="full = the benchmark line; the others launch one kernel --steps times "
-                         "on the steady-state cache (for rocprofv3 runs)")
+    ap.add_argument("--mode", choices=["full", "attention", "append", "tables", "copy"], default="full",
+                    help="full = the benchmark line; attention/append/tables launch one kernel --steps "
+                         "times on the steady-state cache (for rocprofv3 runs); copy = a plain 256 MiB "
+                         "device copy, the known-size kernel the HBM counters are calibrated on")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         sys.exit("bench.py: this path is built and measured on ONE GPU; --gpus N with N > 1 is not supported "
@@ -94,6 +123,15 @@ def main() -> None:
 
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+    if args.mode == "copy":
+        src = torch.full((256 << 20,), 3, dtype=torch.uint8, device=dev)
+        dst = torch.empty_like(src)
+        for _ in range(args.warmup):
+            dst.copy_(src)
+        ms = event_time_ms(lambda: dst.copy_(src), args.steps, torch)
+        print(json.dumps({"mode": "copy", "bytes_read": src.numel(), "bytes_written": dst.numel(),
+                          "launches": args.steps, "avg_launch_us": ms * 1e3}))
+        return
     blocks = args.blocks
     m = HipPagedKVCacheManager(blocks, ANCHOR + WINDOW + 16, T, H, D, torch.bfloat16, dev,
                                num_special_tokens=N_SPECIAL, scale_frames=ANCHOR, sliding_window=WINDOW,
@@ -145,10 +183,10 @@ def main() -> None:
 
     # ---- per-kernel timings with HIP events on the launch stream
     flops = 4.0 * T * kv_tokens * H * D
-    attn_ms = event_time_ms(lambda: m._attend_planned(1, qs[0], None, None), 200, torch)
-    append_ms = event_time_ms(lambda: m._scatter(1, 0, ks[0], vs[0]), 200, torch)
+    attn_ms = event_time_ms(lambda: m._attend_planned(1, qs[0], None, None), 500, torch)
+    append_ms = kernel_time_ms(lambda: m._scatter(1, 0, ks[0], vs[0]), 100, torch)
     ops = m._ops([{"ops": 16, "expect_kv_tokens": kv_tokens}])
-    tables_ms = event_time_ms(lambda: m._tables_step(0, ops, kv_rows=True), 200, torch)
+    tables_ms = kernel_time_ms(lambda: m._tables_step(0, ops, kv_rows=True), 100, torch)
     attn_tflops = flops / (attn_ms * 1e-3) * 1e-12
     append_bytes = 2 * 2 * T * H * D * 2
     append_gbps = append_bytes / (append_ms * 1e-3) * 1e-9
@@ -162,7 +200,7 @@ def main() -> None:
                                f"blocks per frame (tables step + per block paged append + paged attention)",
                    "blocks": blocks, "kv_tokens": kv_tokens, "q_tokens": T, "page_size": PAGE},
         "roofline": {"bound": "mfma", "achieved": attn_tflops, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-                     "frac": attn_tflops / PEAK_BF16_TFLOPS, "traffic": None,
+                     "frac": attn_tflops / PEAK_BF16_TFLOPS, "traffic": ATTN_TRAFFIC_BYTES,
                      "kernel": "lbm_attn_bf16_d64_kernel + lbm_attn_combine_bf16_kernel (one lbm_attn_run)",
                      "flop_per_launch": flops, "avg_launch_us": attn_ms * 1e3},
         "attention_tflops": attn_tflops,
