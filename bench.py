@@ -116,7 +116,7 @@ def main() -> None:
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         sys.exit("bench.py: this path is built and measured on ONE GPU; --gpus N with N > 1 is not supported "
-                 "(streams shard across GPUs without communication; see DESIGN.md)")
+                 "(independent streams would shard across GPUs without communication)")
 
     import torch
     from lingbot_map_amd import HipPagedKVCacheManager
