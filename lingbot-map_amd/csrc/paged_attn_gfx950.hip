@@ -151,10 +151,12 @@ __global__ __launch_bounds__(kThreads, 1) void lbm_attn_bf16_d64_kernel(AttnArgs
   // One more 16-wide step of the QK contraction carries the running reference maximum:
   // K side is the constant row (-1, -1, 0, ...), Q side is (m_hi, m_lo, 0, ...) with
   // m_hi + m_lo = m_run exactly, so S arrives as score*scale - m_run at no vector-ALU cost.
+  // A third element masks the rows past the last token: K side -1 on such rows (0 elsewhere),
+  // Q side 2^100, so their scores arrive as about -2^100 and their numerators are exactly 0.
   u32x4 kaug_bits = {0u, 0u, 0u, 0u};
   if (g == 0) kaug_bits[0] = 0xBF80BF80u;
-  const bf16x8 kaug = __builtin_bit_cast(bf16x8, kaug_bits);
   u32x4 qaug_bits[2] = {{0u, 0u, 0u, 0u}, {0u, 0u, 0u, 0u}};
+  if (g == 0) qaug_bits[0][1] = qaug_bits[1][1] = 0x7180u;  // bf16 2^100
 
   f32x16 o[2][2];
 #pragma unroll
@@ -218,10 +220,13 @@ __global__ __launch_bounds__(kThreads, 1) void lbm_attn_bf16_d64_kernel(AttnArgs
         o[qb][db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va[db], p[qb][kk], o[qb][db], 0, 0, 0);
   };
   // S^T = K Q^T - m_run for the 32 kv rows of half h of the K tile in stage st
-  auto qk_half = [&](int st, int h, f32x16 (&sd)[2]) {
+  auto qk_half = [&](int st, int h, int n_valid, f32x16 (&sd)[2]) {
     f32x16 z;
 #pragma unroll
     for (int i = 0; i < 16; ++i) z[i] = 0.f;
+    u32x4 kb = kaug_bits;
+    kb[1] = (g == 0 && h * 32 + n32 >= n_valid) ? 0xBF80u : 0u;
+    const bf16x8 kaug = __builtin_bit_cast(bf16x8, kb);
 #pragma unroll
     for (int qb = 0; qb < 2; ++qb)
       sd[qb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kaug, __builtin_bit_cast(bf16x8, qaug_bits[qb]), z, 0, 0, 0);
@@ -234,22 +239,12 @@ __global__ __launch_bounds__(kThreads, 1) void lbm_attn_bf16_d64_kernel(AttnArgs
         sd[qb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka, qf[qb][ks], sd[qb], 0, 0, 0);
     }
   };
-  // First part of the softmax of one half: mask, row maxima, and - on the first half of the
+  // First part of the softmax of one half: row maxima, and - on the first half of the
   // split or when a score exceeds the reference by more than kTau - move the reference.
   // Everything already expressed relative to the old reference is rescaled: O, the row
   // sums, these scores, and `pend`, the numerators whose second k-step is still to be
   // multiplied into O.
-  auto soft_check = [&](f32x16 (&sc)[2], bf16x8 (&pend)[2][2], int n_valid, bool first) {
-    if (n_valid < 32) {
-#pragma unroll
-      for (int i = 0; i < 16; ++i) {
-        const int kv = 8 * (i >> 2) + 4 * g + (i & 3);
-        if (kv >= n_valid) {
-          sc[0][i] = -INFINITY;
-          sc[1][i] = -INFINITY;
-        }
-      }
-    }
+  auto soft_check = [&](f32x16 (&sc)[2], bf16x8 (&pend)[2][2], bool first) {
     float mx[2];
 #pragma unroll
     for (int qb = 0; qb < 2; ++qb) {
@@ -311,12 +306,22 @@ __global__ __launch_bounds__(kThreads, 1) void lbm_attn_bf16_d64_kernel(AttnArgs
       }
     }
   };
-// Scheduling hints for the two regions of a half-step: one MFMA, then `v` vector-ALU
-// instructions, then `d` LDS reads, so that the matrix pipe never waits for the softmax.
-#define LBM_SLOT(v, d)                                               \
+// Scheduling hints for a half-step: one MFMA, then `t` transcendental and `v` other
+// vector-ALU instructions, then `d` LDS reads, so that the matrix pipe never waits for the
+// softmax.  A half-step is one basic block: PV k-step 1, the reference step and K steps of
+// the next half's scores, PV k-step 0 of the next half, then the row maxima and the test
+// whether the reference has to move.
+#define LBM_SLOT(t, v, d)                                            \
   __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                 \
+  if (t) __builtin_amdgcn_sched_group_barrier(0x400, t, 0);          \
   if (v) __builtin_amdgcn_sched_group_barrier(0x002, v, 0);          \
   if (d) __builtin_amdgcn_sched_group_barrier(0x100, d, 0)
+#define LBM_HALF_SCHEDULE                                                                   \
+  __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);                                        \
+  LBM_SLOT(3, 2, 1); LBM_SLOT(3, 2, 1); LBM_SLOT(3, 2, 1); LBM_SLOT(3, 2, 1); /* PV 1 */    \
+  LBM_SLOT(2, 2, 1); LBM_SLOT(2, 2, 1);                                 /* reference */    \
+  LBM_SLOT(2, 2, 1); LBM_SLOT(2, 2, 1); LBM_SLOT(2, 2, 0); LBM_SLOT(2, 2, 0); /* K 0-1 */   \
+  LBM_SLOT(2, 2, 0); LBM_SLOT(2, 2, 0); LBM_SLOT(2, 2, 0); LBM_SLOT(2, 2, 0)  /* K 2-3 */
 
   // ---- prologue: K(0), K(1), V(0) into the ring; the V stage the first PV reads is zeroed
   put_k(0, fetch(row_entry(t0), pool_k, own_k));
@@ -332,7 +337,7 @@ __global__ __launch_bounds__(kThreads, 1) void lbm_attn_bf16_d64_kernel(AttnArgs
     for (int kk = 0; kk < 2; ++kk) pB[qb][kk] = __builtin_bit_cast(bf16x8, u32x4{0u, 0u, 0u, 0u});
   int ek = row_entry(t0 + 2), ev = row_entry(t0 + 1);
   __syncthreads();
-  qk_half(0, 0, sA);
+  qk_half(0, 0, sp.kv_tokens - t0 * kKvTile, sA);
   vnext[0] = v_frag(2, 2, 0);
   vnext[1] = v_frag(2, 2, 1);
 
@@ -351,36 +356,28 @@ __global__ __launch_bounds__(kThreads, 1) void lbm_attn_bf16_d64_kernel(AttnArgs
     ek = row_entry(t + 3);
     ev = row_entry(t + 2);
     pv_step(vnext, pB, 0);
-    soft_check(sA, pB, n_valid, i == 0);
+    soft_check(sA, pB, i == 0);
     {
       bf16x8 va[2] = {v_frag(st_vm1, 3, 0), v_frag(st_vm1, 3, 1)};
       pv_step(va, pB, 1);
-      qk_half(st_k, 1, sB);
+      qk_half(st_k, 1, n_valid, sB);
       soft_exp(sA, pA);
       vnext[0] = v_frag(st_v, 0, 0);
       vnext[1] = v_frag(st_v, 0, 1);
-      __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
-      LBM_SLOT(8, 1); LBM_SLOT(8, 1); LBM_SLOT(8, 1); LBM_SLOT(8, 1);   // PV k-step 1
-      LBM_SLOT(8, 1); LBM_SLOT(8, 1);                                   // reference step
-      LBM_SLOT(8, 1); LBM_SLOT(8, 1); LBM_SLOT(8, 0); LBM_SLOT(8, 0);   // K steps 0-1
-      LBM_SLOT(8, 0); LBM_SLOT(8, 0); LBM_SLOT(8, 0); LBM_SLOT(8, 0);   // K steps 2-3
+      LBM_HALF_SCHEDULE;
     }
 
     // ======== half 1 of tile i: softmax(sB) -> pB | PV(tile i, half 0) with pA, QK(tile i+1, half 0) -> sA
     pv_step(vnext, pA, 0);
-    soft_check(sB, pA, n_valid - 32, false);
+    soft_check(sB, pA, false);
     {
       bf16x8 va[2] = {v_frag(st_v, 1, 0), v_frag(st_v, 1, 1)};
       pv_step(va, pA, 1);
-      qk_half(st_k1, 0, sA);  // after the last tile this reads a stale stage; the result is unused
+      qk_half(st_k1, 0, n_valid - kKvTile, sA);  // after the last tile this reads a stale stage; the result is unused
       soft_exp(sB, pB);
       vnext[0] = v_frag(st_v, 2, 0);
       vnext[1] = v_frag(st_v, 2, 1);
-      __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
-      LBM_SLOT(8, 1); LBM_SLOT(8, 1); LBM_SLOT(8, 1); LBM_SLOT(8, 1);
-      LBM_SLOT(8, 1); LBM_SLOT(8, 1);
-      LBM_SLOT(8, 1); LBM_SLOT(8, 1); LBM_SLOT(8, 0); LBM_SLOT(8, 0);
-      LBM_SLOT(8, 0); LBM_SLOT(8, 0); LBM_SLOT(8, 0); LBM_SLOT(8, 0);
+      LBM_HALF_SCHEDULE;
     }
 
     // ======== ring upkeep: K(i+2), V(i+1) (past the last tile: stages nobody reads any more)
@@ -397,40 +394,41 @@ __global__ __launch_bounds__(kThreads, 1) void lbm_attn_bf16_d64_kernel(AttnArgs
     bf16x8 va[2] = {v_frag(st_vm1, 3, 0), v_frag(st_vm1, 3, 1)};
     pv_step(va, pB, 1);
   }
+#undef LBM_HALF_SCHEDULE
 #undef LBM_SLOT
 
-  // ---- epilogue
+  // ---- epilogue.  The accumulators hold O^T (a lane owns 4-element runs of 32 different
+  // rows); written straight out that is 32 scattered 8-byte stores per instruction.  Each
+  // wavefront instead transposes its rows through LDS (the ring is dead by now) and stores
+  // whole 128-byte rows, eight lanes per row.
+  __syncthreads();  // every wave has finished reading the ring
+  unsigned short* stage = &lds_v[0][0] + wave * (32 * kKStride);
+  const bool direct = sp.n_splits == 1;
+  unsigned short* dst = direct ? a.out : a.part_o;
+  const size_t dst_row0 = direct ? (size_t)sp.q_begin : (size_t)sp.part_begin + (size_t)split * sp.q_rows;
 #pragma unroll
   for (int qb = 0; qb < 2; ++qb) {
-    const int r = q_row0 + qb * 32 + n32;
     const float l_tot = swap_sum((l_run[qb][0] + l_run[qb][1]) + (l_run[qb][2] + l_run[qb][3]));
     const float inv = l_tot > 0.f ? 1.0f / l_tot : 0.f;
-    if (r >= sp.q_rows) continue;
-    if (sp.n_splits == 1) {
-      unsigned short* op = a.out + ((size_t)(sp.q_begin + r) * H + head) * 64;
 #pragma unroll
-      for (int db = 0; db < 2; ++db)
+    for (int db = 0; db < 2; ++db)
 #pragma unroll
-        for (int c4 = 0; c4 < 4; ++c4) {
-          f32x4 w;
+      for (int c4 = 0; c4 < 4; ++c4) {
+        f32x4 w;
 #pragma unroll
-          for (int e = 0; e < 4; ++e) w[e] = o[qb][db][c4 * 4 + e] * inv;
-          *(bf16x4*)(op + db * 32 + c4 * 8 + g * 4) = __builtin_convertvector(w, bf16x4);
-        }
-    } else {
-      const size_t prow = ((size_t)sp.part_begin + (size_t)split * sp.q_rows + r) * H + head;
-      unsigned short* po = a.part_o + prow * 64;
+        for (int e = 0; e < 4; ++e) w[e] = o[qb][db][c4 * 4 + e] * inv;
+        *(bf16x4*)&stage[n32 * kKStride + db * 32 + c4 * 8 + g * 4] = __builtin_convertvector(w, bf16x4);
+      }
 #pragma unroll
-      for (int db = 0; db < 2; ++db)
-#pragma unroll
-        for (int c4 = 0; c4 < 4; ++c4) {
-          f32x4 w;
-#pragma unroll
-          for (int e = 0; e < 4; ++e) w[e] = o[qb][db][c4 * 4 + e] * inv;
-          *(bf16x4*)(po + db * 32 + c4 * 8 + g * 4) = __builtin_convertvector(w, bf16x4);
-        }
-      if (g == 0) a.part_lse[prow] = m_run[qb] + __builtin_amdgcn_logf(l_tot);
+    for (int k = 0; k < 4; ++k) {
+      const int row = k * 8 + (lane >> 3);
+      const u32x4 v = *(const u32x4*)&stage[row * kKStride + (lane & 7) * 8];
+      const int r = q_row0 + qb * 32 + row;
+      if (r < sp.q_rows) *(u32x4*)(dst + ((dst_row0 + r) * H + head) * 64 + (lane & 7) * 8) = v;
     }
+    const int r = q_row0 + qb * 32 + n32;
+    if (!direct && g == 0 && r < sp.q_rows)
+      a.part_lse[(dst_row0 + r) * H + head] = m_run[qb] + __builtin_amdgcn_logf(l_tot);
   }
 }
 
@@ -446,20 +444,39 @@ __global__ __launch_bounds__(256) void lbm_attn_combine_bf16_kernel(AttnArgs a) 
   const long long rh = idx >> 3;  // r * H + h
   const long long split_stride = (long long)sp.q_rows * H;
   const float* lse = a.part_lse + (long long)sp.part_begin * H + rh;
+  const int n = sp.n_splits;
+  // loads are issued in batches (the split count is a run-time value, a plain loop would
+  // wait for each load in turn)
   float mx = -INFINITY;
-  for (int s = 0; s < sp.n_splits; ++s) mx = fmaxf(mx, lse[s * split_stride]);
+  for (int s0 = 0; s0 < n; s0 += 8) {
+    float t[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) t[j] = lse[min(s0 + j, n - 1) * split_stride];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) mx = fmaxf(mx, t[j]);
+  }
   float wsum = 0.f;
   f32x8 acc;
 #pragma unroll
   for (int e = 0; e < 8; ++e) acc[e] = 0.f;
   const unsigned short* po = a.part_o + ((long long)sp.part_begin * H + rh) * 64 + d8 * 8;
-  for (int s = 0; s < sp.n_splits; ++s) {
-    const float w = __builtin_amdgcn_exp2f(lse[s * split_stride] - mx);
-    const bf16x8 v = *(const bf16x8*)(po + s * split_stride * 64);
-    const f32x8 vf = __builtin_convertvector(v, f32x8);
-    wsum += w;
+  for (int s0 = 0; s0 < n; s0 += 4) {
+    float t[4];
+    bf16x8 v[4];
 #pragma unroll
-    for (int e = 0; e < 8; ++e) acc[e] += w * vf[e];
+    for (int j = 0; j < 4; ++j) {
+      const long long s = min(s0 + j, n - 1);
+      t[j] = lse[s * split_stride];
+      v[j] = *(const bf16x8*)(po + s * split_stride * 64);
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const float w = s0 + j < n ? __builtin_amdgcn_exp2f(t[j] - mx) : 0.f;
+      const f32x8 vf = __builtin_convertvector(v[j], f32x8);
+      wsum += w;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) acc[e] += w * vf[e];
+    }
   }
   const float inv = 1.0f / wsum;
   const long long r = rh / H, h = rh % H;
