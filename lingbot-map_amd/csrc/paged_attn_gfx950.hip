@@ -5,26 +5,36 @@
 // bf16 kernel, head_dim 64.  One workgroup = 8 wavefronts x 64 query rows of one head over
 // one contiguous run of 64-token KV tiles (split-KV; partial results are merged by
 // lbm_attn_combine_bf16_kernel).  Per tile a wavefront computes
-//     S^T = K Q^T      v_mfma_f32_32x32x16_bf16, A = K rows from LDS, B = Q in registers
-//     P   = exp2(S*c - m)   one query row per lane column, so row max/sum stay in-lane
-//                           except one half-swap (v_permlane32_swap)
+//     S^T = K Q^T - m  v_mfma_f32_32x32x16_bf16, A = K rows from LDS, B = Q in registers; the
+//                      softmax scale (in log2 units) is folded into Q and the reference m
+//                      into one more k-step, so S arrives ready for exp2
+//     P   = exp2(S)    one query row per lane column; v_exp_f32 + v_cvt_pk_bf16_f32
 //     O^T += V^T P^T   A = V^T read with ds_read_b64_tr_b16 from the row-major V tile,
-//                      B = P^T straight from the accumulator registers of S^T
-// The running maximum is only raised when a tile exceeds it by more than kTau (in log2
-// units): the rescale of the 64 output registers is skipped on almost every tile and the
-// result is mathematically unchanged because the same stale maximum divides out.
+//                      B = P^T straight from the registers the packing wrote
+//     l   += 1^T P^T   row sums on the matrix pipe too (16x16x32 with a 0/1 selector)
+// The reference m of a row is not its running maximum but a value kHeadroom above the
+// maximum seen when it was last set, and it is only raised when a numerator reaches 2, i.e.
+// when a score exceeds it; the same reference divides out of O / l, so the result is
+// mathematically unchanged, no row maximum is computed on the common path, and O is rescaled
+// only on the rare path.  The test costs a few OR instructions per half tile: a bf16 numerator
+// is >= 2 (or infinite) exactly when the top bit of its exponent field is set.
 //
-// Schedule.  Measured on MI355X: one wavefront alone issues a vector-ALU instruction only
-// every ~8 cycles, two wavefronts of a SIMD together reach the full rate of one per 4, and
-// the matrix pipe overlaps with the vector ALU only when MFMAs and vector instructions
-// alternate in program order.  Each wavefront therefore runs a software pipeline over
-// 32-token half tiles: while the vector ALU turns the scores of one half into softmax
-// numerators, the MFMAs of the next half's QK^T and of the previous half's PV are issued in
-// between (sched_group_barrier fixes the interleaving), and the two wavefronts of a SIMD
-// fill each other's issue gaps.  The running reference maximum and the softmax scale are
-// folded into the QK^T contraction, so the vector ALU only does max, exp2, bf16 packing and
-// the row sum.  K/V tiles are shared by all eight waves through a three-stage LDS ring with
-// one workgroup barrier per tile.
+// Why it is built this way.  Measured on MI355X with two wavefronts per SIMD: v_exp_f32 issues
+// every ~4.6 ns per SIMD, v_cvt_pk_bf16_f32 / v_max3_f32 / v_dot2c_f32_bf16 every ~2.7 ns, plain
+// fp32 adds and multiplies every ~1.4 ns, and a 32x32x16 MFMA occupies the matrix pipe for
+// 13.8 ns.  With head_dim 64 every score needs one exp2 and half a packing instruction, so the
+// vector ALU, not the matrix pipe, bounds the loop; everything that can run as an MFMA (scale,
+// reference subtraction, masking of the ragged tail, row sums) does, and the vector ALU is
+// left with exp2, packing and the overflow test.
+//
+// Schedule.  Each wavefront runs a software pipeline over 32-token half tiles: while the
+// vector ALU turns the scores of one half into numerators, the MFMAs of the next half's QK^T
+// and of the previous half's PV and row sums are issued in between.  A half-step is one basic
+// block written as 22 slices (one MFMA plus its share of the vector work and LDS reads each)
+// fenced with sched_barrier, and the two wavefronts of a SIMD fill each other's issue gaps.
+// The numerators of a half are computed before the test on them, so the test's branch is the
+// only one in the loop and its condition is ready long before it is taken.  K/V tiles are
+// shared by all eight waves through a three-stage LDS ring with one workgroup barrier per tile.
 #include <hip/hip_runtime.h>
 #include <climits>
 #include "lbm_internal.h"
@@ -49,7 +59,7 @@ constexpr int kQTile = kQPerWave * kWaves;
 constexpr int kStages = 3;              // LDS ring depth
 constexpr int kKStride = 72;            // bf16 per LDS row of K: 144 B, b128 reads hit 64 distinct banks
 constexpr int kVStride = 96;            // bf16 per LDS row of V: 192 B, 4-row transpose reads conflict-free
-constexpr float kTau = 8.0f;            // lazy-rescale threshold, log2 units
+constexpr float kHeadroom = 11.0f;      // the softmax reference is set this far above the row maxima (log2 units)
 constexpr int kTargetWgs = 256;         // one 8-wave workgroup per CU
 
 struct AttnArgs {
@@ -86,11 +96,6 @@ __device__ __forceinline__ float swap_max(float x) {
   swap_halves(x, lo, hi);
   return max2(lo, hi);
 }
-__device__ __forceinline__ float swap_sum(float x) {
-  float lo, hi;
-  swap_halves(x, lo, hi);
-  return lo + hi;
-}
 
 }  // namespace
 
@@ -122,6 +127,15 @@ __global__ __launch_bounds__(kThreads, 1) void lbm_attn_bf16_d64_kernel(AttnArgs
   }
   if (local >= sp.n_qtiles * n_hs) return;  // padding between streams
   const int head = hs % H, split = hs / H;
+  if (sp.kv_tokens <= 0) {
+    // nothing visible: the reference returns zeros (lingbot_map/layers/flashinfer_cache.py:368-370)
+    for (int k = 0; k < kQPerWave / 8; ++k) {
+      const int r = qt * kQTile + wave * kQPerWave + k * 8 + (lane >> 3);
+      if (r < sp.q_rows)
+        *(u32x4*)(a.out + ((size_t)(sp.q_begin + r) * H + head) * 64 + (lane & 7) * 8) = u32x4{0u, 0u, 0u, 0u};
+    }
+    return;
+  }
   const int n_tiles = (sp.kv_tokens + kKvTile - 1) / kKvTile;
   const int t0 = split * sp.tiles_per_split;
   const int t1 = min(t0 + sp.tiles_per_split, n_tiles);
@@ -165,8 +179,16 @@ __global__ __launch_bounds__(kThreads, 1) void lbm_attn_bf16_d64_kernel(AttnArgs
     for (int db = 0; db < 2; ++db)
 #pragma unroll
       for (int i = 0; i < 16; ++i) o[qb][db][i] = 0.f;
-  float m_run[2] = {0.f, 0.f};  // re-referenced to the first tile's maximum before first use
-  float l_run[2][4] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};  // four partial row sums per query block
+  float m_run[2] = {0.f, 0.f};  // moved to the first half's maxima before the loop
+  // Row sums (softmax denominators) are accumulated by the matrix pipe as well: a 16x16x32 MFMA
+  // with a 0/1 selector as A and the numerators, exactly as they sit in the registers for PV,
+  // as B.  Read as a 32x16 B operand the numerator registers hold, for column n, query n in
+  // k rows 0-7 and 16-23 and query n+16 in k rows 8-15 and 24-31; selector row 0 picks the
+  // former and row 1 the latter, so lane n < 16 ends up with the sums of query n (element 0)
+  // and of query n+16 (element 1) of the block, and every other element stays 0.
+  f32x4 lacc[2] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
+  const unsigned sel_word = (lane == 0 || lane == 32 || lane == 17 || lane == 49) ? 0x3F803F80u : 0u;
+  const bf16x8 lsel = __builtin_bit_cast(bf16x8, u32x4{sel_word, sel_word, sel_word, sel_word});
 
   // ---- tile staging: each thread moves one 16-byte piece of a K row and of a V row per tile.
   // Rows past the last token re-read the last token (finite data; the softmax masks them).
@@ -239,13 +261,9 @@ __global__ __launch_bounds__(kThreads, 1) void lbm_attn_bf16_d64_kernel(AttnArgs
         sd[qb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka, qf[qb][ks], sd[qb], 0, 0, 0);
     }
   };
-  // First part of the softmax of one half: row maxima, and - on the first half of the
-  // split or when a score exceeds the reference by more than kTau - move the reference.
-  // Everything already expressed relative to the old reference is rescaled: O, the row
-  // sums, these scores, and `pend`, the numerators whose second k-step is still to be
-  // multiplied into O.
-  auto soft_check = [&](f32x16 (&sc)[2], bf16x8 (&pend)[2][2], bool first) {
-    float mx[2];
+  // Row maxima of one half, per query block (the lane's own 16 scores, then the other
+  // half-wave's through one swap).
+  auto row_max = [&](const f32x16 (&sc)[2], float (&mx)[2]) {
 #pragma unroll
     for (int qb = 0; qb < 2; ++qb) {
       float m0 = max3(sc[qb][0], sc[qb][1], sc[qb][2]), m1 = max3(sc[qb][3], sc[qb][4], sc[qb][5]);
@@ -256,72 +274,143 @@ __global__ __launch_bounds__(kThreads, 1) void lbm_attn_bf16_d64_kernel(AttnArgs
       m0 = max3(m0, sc[qb][14], sc[qb][15]);
       mx[qb] = swap_max(max2(m0, m1));
     }
-    if (__builtin_amdgcn_ballot_w64(first || mx[0] > kTau || mx[1] > kTau)) {
-#pragma unroll
-      for (int qb = 0; qb < 2; ++qb) {
-        const bool move = first || mx[qb] > kTau;
-        // new reference, rounded so that two bf16 values carry it exactly
-        const float want = move ? m_run[qb] + mx[qb] : m_run[qb];
-        const float hi = (float)(__bf16)want;
-        const float lo = (float)(__bf16)(want - hi);
-        const float m_new = hi + lo;
-        const float d = m_new - m_run[qb];
-        const float alpha = __builtin_amdgcn_exp2f(-d);
-        m_run[qb] = m_new;
-#pragma unroll
-        for (int j = 0; j < 4; ++j) l_run[qb][j] *= alpha;
-        const bf16x2 pair = {(__bf16)hi, (__bf16)lo};
-        qaug_bits[qb][0] = g == 0 ? __builtin_bit_cast(unsigned, pair) : 0u;
-#pragma unroll
-        for (int db = 0; db < 2; ++db)
-#pragma unroll
-          for (int i = 0; i < 16; ++i) o[qb][db][i] *= alpha;
-#pragma unroll
-        for (int i = 0; i < 16; ++i) sc[qb][i] -= d;
-        // the second k-step of the previous half's numerators has not been folded into O yet
-        f32x8 pf = __builtin_convertvector(pend[qb][1], f32x8);
-#pragma unroll
-        for (int j = 0; j < 8; ++j) pf[j] *= alpha;
-        pend[qb][1] = __builtin_convertvector(pf, bf16x8);
-      }
-    }
   };
-  // Second part: numerators 2^s, packed to bf16; the denominator sums the rounded values.
-  auto soft_exp = [&](const f32x16 (&sc)[2], bf16x8 (&pd)[2][2]) {
-    const bf16x2 ones = {(__bf16)1.0f, (__bf16)1.0f};
+  // Numerators 2^s packed to bf16.
+  auto numerators = [&](const f32x16 (&sc)[2], bf16x8 (&pd)[2][2]) {
 #pragma unroll
-    for (int qb = 0; qb < 2; ++qb) {
+    for (int qb = 0; qb < 2; ++qb)
 #pragma unroll
       for (int kk = 0; kk < 2; ++kk) {
         f32x8 e;
 #pragma unroll
         for (int j = 0; j < 8; ++j) e[j] = __builtin_amdgcn_exp2f(sc[qb][kk * 8 + j]);
-        const bf16x8 pk = __builtin_convertvector(e, bf16x8);
-        pd[qb][kk] = pk;
+        pd[qb][kk] = __builtin_convertvector(e, bf16x8);
+      }
+  };
+  // Move the reference of query block qb to m_run + rise (rounded so that two bf16 values
+  // carry it exactly) and return how far it moved.
+  auto move_reference = [&](int qb, float rise) -> float {
+    const float want = m_run[qb] + rise;
+    const float hi = (float)(__bf16)want;
+    const float lo = (float)(__bf16)(want - hi);
+    const float d = (hi + lo) - m_run[qb];
+    m_run[qb] = hi + lo;
+    const bf16x2 pair = {(__bf16)hi, (__bf16)lo};
+    qaug_bits[qb][0] = g == 0 ? __builtin_bit_cast(unsigned, pair) : 0u;
+    return d;
+  };
+  // Rare path of a half-step: a numerator of `cur` came out as 2 or more, i.e. a score
+  // exceeded the reference by at least 1 (in log2 units; an overflow to infinity included).
+  // Nothing has consumed these numerators yet.  Raise the reference to the row maxima, rescale
+  // what is already expressed in the old one (O, the row sums, and the scores of `cur` and of
+  // `next`, which the MFMAs of this half-step produced with the old reference) and recompute
+  // the numerators, which are then at most 1.
+  auto raise_reference = [&](f32x16 (&cur)[2], bf16x8 (&pd)[2][2], f32x16 (&next)[2]) {
+    float mx[2];
+    row_max(cur, mx);
 #pragma unroll
-        for (int j = 0; j < 8; j += 2) {
-          const bf16x2 pr = {pk[j], pk[j + 1]};
-          l_run[qb][j >> 1] = __builtin_amdgcn_fdot2_f32_bf16(pr, ones, l_run[qb][j >> 1], false);
-        }
+    for (int qb = 0; qb < 2; ++qb) {
+      const float d = move_reference(qb, max2(mx[qb] + kHeadroom, 0.f));
+      const float alpha = __builtin_amdgcn_exp2f(-d);
+      // row sums: lane n < 16 holds query n in element 0 and query n + 16 in element 1
+      const float alpha_hi = __builtin_bit_cast(
+          float, __builtin_amdgcn_ds_bpermute(4 * ((lane & 15) + 16), __builtin_bit_cast(int, alpha)));
+      lacc[qb][0] *= alpha;
+      lacc[qb][1] *= alpha_hi;
+#pragma unroll
+      for (int db = 0; db < 2; ++db)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) o[qb][db][i] *= alpha;
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        cur[qb][i] -= d;
+        next[qb][i] -= d;
       }
     }
+    numerators(cur, pd);
   };
-// Scheduling hints for a half-step: one MFMA, then `t` transcendental and `v` other
-// vector-ALU instructions, then `d` LDS reads, so that the matrix pipe never waits for the
-// softmax.  A half-step is one basic block: PV k-step 1, the reference step and K steps of
-// the next half's scores, PV k-step 0 of the next half, then the row maxima and the test
-// whether the reference has to move.
-#define LBM_SLOT(t, v, d)                                            \
-  __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                 \
-  if (t) __builtin_amdgcn_sched_group_barrier(0x400, t, 0);          \
-  if (v) __builtin_amdgcn_sched_group_barrier(0x002, v, 0);          \
-  if (d) __builtin_amdgcn_sched_group_barrier(0x100, d, 0)
-#define LBM_HALF_SCHEDULE                                                                   \
-  __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);                                        \
-  LBM_SLOT(3, 2, 1); LBM_SLOT(3, 2, 1); LBM_SLOT(3, 2, 1); LBM_SLOT(3, 2, 1); /* PV 1 */    \
-  LBM_SLOT(2, 2, 1); LBM_SLOT(2, 2, 1);                                 /* reference */    \
-  LBM_SLOT(2, 2, 1); LBM_SLOT(2, 2, 1); LBM_SLOT(2, 2, 0); LBM_SLOT(2, 2, 0); /* K 0-1 */   \
-  LBM_SLOT(2, 2, 0); LBM_SLOT(2, 2, 0); LBM_SLOT(2, 2, 0); LBM_SLOT(2, 2, 0)  /* K 2-3 */
+// One half-step is one basic block of 22 MFMAs, written as 22 slices fenced by
+// sched_barrier so that the interleaving is the one spelled out here.  Slice j issues MFMA j
+//    0-3   O += V^T P^T, k-step 0 of `prev`        4-7   the same, k-step 1
+//    8-11  row sums of `prev` (16x16x32)           12-13 reference step of the next scores
+//   14-21  their four K steps
+// then its share of the vector work on `cur` (two exp2 each in slices 0-15, the bf16 packing
+// one slice later, then the OR of the packed words whose exponent bits tell whether any
+// numerator reached 2) and the LDS reads of operands a few slices ahead of their MFMA.
+//   cur/pd    scores of this half and where its numerators go
+//   prev      numerators of the previous half; their V rows: k-step 0 already in vnext,
+//             k-step 1 = k-step ks_pv of the V tile in stage st_pv
+//   next      scores of the next half: K tile in stage st_qk, half h_qk, nv_qk valid tokens left
+//   st_vn, ks_vn   V tile / k-step whose V^T goes to vnext for the following half-step
+#define LBM_SLICE(j, cur, pd, prev, next, st_pv, ks_pv, st_qk, h_qk, st_vn, ks_vn)                 \
+  {                                                                                              \
+    /* ---- the MFMA of this slice */                                                            \
+    if ((j) < 4)                                                                                 \
+      o[(j) & 1][(j) >> 1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(                            \
+          vnext[(j) >> 1], prev[(j) & 1][0], o[(j) & 1][(j) >> 1], 0, 0, 0);                     \
+    else if ((j) < 8)                                                                            \
+      o[(j) & 1][((j) - 4) >> 1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(                      \
+          va[((j) - 4) >> 1], prev[(j) & 1][1], o[(j) & 1][((j) - 4) >> 1], 0, 0, 0);            \
+    else if ((j) < 12)                                                                           \
+      lacc[(j) & 1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(                                   \
+          lsel, prev[(j) & 1][((j) - 8) >> 1], lacc[(j) & 1], 0, 0, 0);                          \
+    else if ((j) < 14)                                                                           \
+      next[(j) & 1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(                                   \
+          kaug, __builtin_bit_cast(bf16x8, qaug_bits[(j) & 1]), zero16, 0, 0, 0);                \
+    else                                                                                         \
+      next[(j) & 1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(                                   \
+          ka[((j) - 14) >> 1], qf[(j) & 1][((j) - 14) >> 1], next[(j) & 1], 0, 0, 0);            \
+    /* ---- numerators of cur: exp2 of scores 2j, 2j+1; packing of the pair of slice j-1 */      \
+    if ((j) < 16) {                                                                              \
+      e[2 * (j)] = __builtin_amdgcn_exp2f(cur[(j) >> 3][(2 * (j)) & 15]);                        \
+      e[2 * (j) + 1] = __builtin_amdgcn_exp2f(cur[(j) >> 3][(2 * (j) + 1) & 15]);                \
+    }                                                                                            \
+    if ((j) >= 1 && (j) <= 16) {                                                                 \
+      constexpr int c = (j) - 1, ci = (2 * c) & 15;                                              \
+      pd[c >> 3][ci >> 3][ci & 7] = (__bf16)e[2 * c];                                            \
+      pd[c >> 3][ci >> 3][(ci & 7) + 1] = (__bf16)e[2 * c + 1];                                  \
+    }                                                                                            \
+    /* ---- OR of the packed numerators, one 4-word group per two slices once it is complete */  \
+    if ((j) >= 5 && (j) <= 18 && (((j) - 5) & 3) < 2) {                                          \
+      constexpr int grp = ((j) - 5) >> 2, w = (((j) - 5) & 3) * 2;                               \
+      const u32x4 words = __builtin_bit_cast(u32x4, pd[grp >> 1][grp & 1]);                      \
+      chk = ((j) == 5 ? 0u : chk) | words[w] | words[w + 1];                                     \
+    }                                                                                            \
+    /* ---- LDS reads */                                                                         \
+    if ((j) == 0) va[0] = v_frag(st_pv, ks_pv, 0);                                               \
+    if ((j) == 1) va[1] = v_frag(st_pv, ks_pv, 1);                                               \
+    if ((j) == 10 || (j) == 12 || (j) == 14 || (j) == 16)                                        \
+      ka[((j) - 10) >> 1] = __builtin_bit_cast(                                                  \
+          bf16x8, *(const u32x4*)&lds_k[st_qk][((h_qk) * 32 + n32) * kKStride + (((j) - 10) >> 1) * 16 + g * 8]); \
+    if ((j) == 17) vnext[0] = v_frag(st_vn, ks_vn, 0);                                           \
+    if ((j) == 18) vnext[1] = v_frag(st_vn, ks_vn, 1);                                           \
+    __builtin_amdgcn_sched_barrier(0);                                                           \
+  }
+#define LBM_S4(j, ...) LBM_SLICE(j, __VA_ARGS__) LBM_SLICE(j + 1, __VA_ARGS__) LBM_SLICE(j + 2, __VA_ARGS__) LBM_SLICE(j + 3, __VA_ARGS__)
+// `hot` tells whether a numerator of `cur` reached 2 (bf16 exponent field >= 128)
+#define LBM_HALF_STEP(cur, pd, prev, next, st_pv, ks_pv, st_qk, h_qk, nv_qk, st_vn, ks_vn, hot)   \
+  {                                                                                              \
+    u32x4 kb = kaug_bits;                                                                        \
+    kb[1] = (g == 0 && (h_qk) * 32 + n32 >= (nv_qk)) ? 0xBF80u : 0u;                             \
+    const bf16x8 kaug = __builtin_bit_cast(bf16x8, kb);                                          \
+    bf16x8 va[2], ka[4];                                                                         \
+    float e[32];                                                                                 \
+    unsigned chk;                                                                                \
+    __builtin_amdgcn_sched_barrier(0);                                                           \
+    LBM_S4(0, cur, pd, prev, next, st_pv, ks_pv, st_qk, h_qk, st_vn, ks_vn)                       \
+    LBM_S4(4, cur, pd, prev, next, st_pv, ks_pv, st_qk, h_qk, st_vn, ks_vn)                       \
+    LBM_S4(8, cur, pd, prev, next, st_pv, ks_pv, st_qk, h_qk, st_vn, ks_vn)                       \
+    LBM_S4(12, cur, pd, prev, next, st_pv, ks_pv, st_qk, h_qk, st_vn, ks_vn)                      \
+    LBM_S4(16, cur, pd, prev, next, st_pv, ks_pv, st_qk, h_qk, st_vn, ks_vn)                      \
+    LBM_SLICE(20, cur, pd, prev, next, st_pv, ks_pv, st_qk, h_qk, st_vn, ks_vn)                   \
+    LBM_SLICE(21, cur, pd, prev, next, st_pv, ks_pv, st_qk, h_qk, st_vn, ks_vn)                   \
+    /* the numerators exist before the test that follows, not only on its common branch */       \
+    asm volatile("" : "+v"(pd[0][0]), "+v"(pd[0][1]), "+v"(pd[1][0]), "+v"(pd[1][1]));             \
+    hot = (chk & 0x40004000u) != 0u;                                                             \
+  }
+  f32x16 zero16;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) zero16[i] = 0.f;
 
   // ---- prologue: K(0), K(1), V(0) into the ring; the V stage the first PV reads is zeroed
   put_k(0, fetch(row_entry(t0), pool_k, own_k));
@@ -338,6 +427,17 @@ __global__ __launch_bounds__(kThreads, 1) void lbm_attn_bf16_d64_kernel(AttnArgs
   int ek = row_entry(t0 + 2), ev = row_entry(t0 + 1);
   __syncthreads();
   qk_half(0, 0, sp.kv_tokens - t0 * kKvTile, sA);
+  {
+    // the reference starts at the maxima of the first half
+    float mx[2];
+    row_max(sA, mx);
+#pragma unroll
+    for (int qb = 0; qb < 2; ++qb) {
+      const float d = move_reference(qb, mx[qb] + kHeadroom);
+#pragma unroll
+      for (int i = 0; i < 16; ++i) sA[qb][i] -= d;
+    }
+  }
   vnext[0] = v_frag(2, 2, 0);
   vnext[1] = v_frag(2, 2, 1);
 
@@ -348,39 +448,24 @@ __global__ __launch_bounds__(kThreads, 1) void lbm_attn_bf16_d64_kernel(AttnArgs
     int st_k2 = st_k1 + 1; if (st_k2 >= kStages) st_k2 -= kStages;
     int st_v1 = st_v + 1; if (st_v1 >= kStages) st_v1 -= kStages;
     const int n_valid = sp.kv_tokens - t * kKvTile;
+    bool hot;
 
-    // ======== half 0 of tile i: softmax(sA) -> pA | PV(tile i-1, half 1) with pB, QK(tile i, half 1) -> sB
     // global fetches of K(i+2), V(i+1) start here and land in the ring at the end of the step
     const u32x4 kreg = fetch(ek, pool_k, own_k);
     const u32x4 vreg = fetch(ev, pool_v, own_v);
     ek = row_entry(t + 3);
     ev = row_entry(t + 2);
-    pv_step(vnext, pB, 0);
-    soft_check(sA, pB, i == 0);
-    {
-      bf16x8 va[2] = {v_frag(st_vm1, 3, 0), v_frag(st_vm1, 3, 1)};
-      pv_step(va, pB, 1);
-      qk_half(st_k, 1, n_valid, sB);
-      soft_exp(sA, pA);
-      vnext[0] = v_frag(st_v, 0, 0);
-      vnext[1] = v_frag(st_v, 0, 1);
-      LBM_HALF_SCHEDULE;
-    }
 
-    // ======== half 1 of tile i: softmax(sB) -> pB | PV(tile i, half 0) with pA, QK(tile i+1, half 0) -> sA
-    pv_step(vnext, pA, 0);
-    soft_check(sB, pA, false);
-    {
-      bf16x8 va[2] = {v_frag(st_v, 1, 0), v_frag(st_v, 1, 1)};
-      pv_step(va, pA, 1);
-      qk_half(st_k1, 0, n_valid - kKvTile, sA);  // after the last tile this reads a stale stage; the result is unused
-      soft_exp(sB, pB);
-      vnext[0] = v_frag(st_v, 2, 0);
-      vnext[1] = v_frag(st_v, 2, 1);
-      LBM_HALF_SCHEDULE;
-    }
+    // half 0 of tile i: softmax(sA) -> pA | PV(tile i-1, half 1) with pB | QK(tile i, half 1) -> sB
+    LBM_HALF_STEP(sA, pA, pB, sB, st_vm1, 3, st_k, 1, n_valid, st_v, 0, hot);
+    if (__builtin_amdgcn_ballot_w64(hot)) raise_reference(sA, pA, sB);
 
-    // ======== ring upkeep: K(i+2), V(i+1) (past the last tile: stages nobody reads any more)
+    // half 1 of tile i: softmax(sB) -> pB | PV(tile i, half 0) with pA | QK(tile i+1, half 0) -> sA
+    // (after the last tile that QK reads a stale stage; its result is unused)
+    LBM_HALF_STEP(sB, pB, pA, sA, st_v, 1, st_k1, 0, n_valid - kKvTile, st_v, 2, hot);
+    if (__builtin_amdgcn_ballot_w64(hot)) raise_reference(sB, pB, sA);
+
+    // ring upkeep: K(i+2), V(i+1) (past the last tile: stages nobody reads any more)
     put_k(st_k2, kreg);
     put_v(st_v1, vreg);
     __syncthreads();
@@ -388,14 +473,20 @@ __global__ __launch_bounds__(kThreads, 1) void lbm_attn_bf16_d64_kernel(AttnArgs
     st_vm1 = st_v;
     st_v = st_v1;
   }
-  // PV of the last half: pB with half 1 of V(n-1), whose first k-step is already in vnext
+  // PV and row sums of the last half: pB with half 1 of V(n-1), first k-step already in vnext
   {
     pv_step(vnext, pB, 0);
     bf16x8 va[2] = {v_frag(st_vm1, 3, 0), v_frag(st_vm1, 3, 1)};
     pv_step(va, pB, 1);
+#pragma unroll
+    for (int qb = 0; qb < 2; ++qb)
+#pragma unroll
+      for (int kk = 0; kk < 2; ++kk)
+        lacc[qb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(lsel, pB[qb][kk], lacc[qb], 0, 0, 0);
   }
-#undef LBM_HALF_SCHEDULE
-#undef LBM_SLOT
+#undef LBM_HALF_STEP
+#undef LBM_S4
+#undef LBM_SLICE
 
   // ---- epilogue.  The accumulators hold O^T (a lane owns 4-element runs of 32 different
   // rows); written straight out that is 32 scattered 8-byte stores per instruction.  Each
@@ -408,7 +499,14 @@ __global__ __launch_bounds__(kThreads, 1) void lbm_attn_bf16_d64_kernel(AttnArgs
   const size_t dst_row0 = direct ? (size_t)sp.q_begin : (size_t)sp.part_begin + (size_t)split * sp.q_rows;
 #pragma unroll
   for (int qb = 0; qb < 2; ++qb) {
-    const float l_tot = swap_sum((l_run[qb][0] + l_run[qb][1]) + (l_run[qb][2] + l_run[qb][3]));
+    // the row sum of query n32 of this block sits in lane n32 % 16, element n32 / 16
+    // (the two elements go through an opaque asm: fed two elements of one vector, the compiler
+    // folds the select below into the permute's data operand, which picks by the wrong lane)
+    float sum_lo = lacc[qb][0], sum_hi = lacc[qb][1];
+    asm volatile("" : "+v"(sum_lo), "+v"(sum_hi));
+    const float l_lo = __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute(4 * (lane & 15), __builtin_bit_cast(int, sum_lo)));
+    const float l_hi = __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute(4 * (lane & 15), __builtin_bit_cast(int, sum_hi)));
+    const float l_tot = (n32 & 16) ? l_hi : l_lo;
     const float inv = l_tot > 0.f ? 1.0f / l_tot : 0.f;
 #pragma unroll
     for (int db = 0; db < 2; ++db)

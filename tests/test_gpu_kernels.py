@@ -160,6 +160,32 @@ def test_attention_moving_reference_maximum(order):
     check_bf16(out.cpu(), sdpa_nhd(q, k, v))
 
 
+def test_attention_late_dominant_tokens():
+    """Tokens whose score towers over everything before them (by 30+ in log2 units) arrive
+    late, in either half of a tile, three times in a row for the same query row: the kernel has
+    to raise its softmax reference after the numerators of that half were already computed
+    against the old one, and redo them.  The row's output is then that token's V row."""
+    from oracle.sdpa_cache import sdpa_nhd
+    dev = torch.device("cuda:0")
+    g = torch.Generator().manual_seed(23)
+    tq, H, D, S, n_kv = 200, 4, 64, 16, 4096
+    q = torch.randn(tq, H, D, generator=g).to(torch.bfloat16)
+    k = (0.1 * torch.randn(n_kv, H, D, generator=g))
+    v = torch.randn(n_kv, H, D, generator=g).to(torch.bfloat16)
+    spikes = [(5, 100, 2.0), (5, 1000, 3.0), (5, 4000, 4.0), (70, 1337, 3.0), (150, 63, 2.5), (199, 4095, 3.0)]
+    for r, t, c in spikes:
+        k[t] = c * q[r].float()
+    k = k.to(torch.bfloat16)
+    pool = torch.zeros(n_kv // S, 2, S, H, D, dtype=torch.bfloat16)
+    pool[:, 0] = k.view(n_kv // S, S, H, D)
+    pool[:, 1] = v.view(n_kv // S, S, H, D)
+    rows, n_tok = rows_from_pages(list(range(n_kv // S)), [S] * (n_kv // S), S, dev)
+    out = run_attention(q.to(dev), pool.to(dev), rows, [(0, tq, 0, n_tok)], S).cpu()
+    check_bf16(out, sdpa_nhd(q, k, v))
+    for r, t in [(5, 4000), (70, 1337), (150, 63), (199, 4095)]:
+        assert (out[r].float() - v[t].float()).abs().max().item() <= 1e-2
+
+
 def test_attention_closed_forms():
     dev = torch.device("cuda:0")
     H, D, S = 2, 64, 16
