@@ -102,6 +102,52 @@ def cpu_baseline(torch, kv_tokens: int, blocks: int) -> dict:
     }
 
 
+def aggregator_step(torch, blocks: int, steps: int, warmup: int) -> dict:
+    """One streamed frame through `blocks` groups of (frame block, global block) at ViT-L size
+    (dim 1024, 16 heads, MLP 4096, LayerNorm, qk-norm, rotary embedding, LayerScale), random
+    init, bf16: the aggregator's alternating-attention trunk (lingbot_map/aggregator/stream.py:
+    415-529).  The global blocks run the HIP cache path; linears, norms, GELU and the frame
+    blocks' dense attention are PyTorch-ROCm library calls.  Patch embedding, the image encoder
+    and the prediction heads are not part of the step."""
+    from lingbot_map_amd import HipPagedBlock, HipPagedKVCacheManager
+    dev = torch.device("cuda:0")
+    dim = H * D
+    torch.manual_seed(4)
+    kw = dict(dim=dim, num_heads=H, mlp_ratio=4.0, qk_norm=True, init_values=0.01, rope=True,
+              kv_cache_sliding_window=WINDOW, kv_cache_scale_frames=ANCHOR)
+    frame_blocks = [HipPagedBlock(**kw).to(dev, torch.bfloat16).eval() for _ in range(blocks)]
+    global_blocks = [HipPagedBlock(**kw).to(dev, torch.bfloat16).eval() for _ in range(blocks)]
+    m = HipPagedKVCacheManager(blocks, ANCHOR + WINDOW + 16, T, H, D, torch.bfloat16, dev,
+                               num_special_tokens=N_SPECIAL, scale_frames=ANCHOR, sliding_window=WINDOW,
+                               max_total_frames=256, page_size=PAGE, layout="frame_pages")
+    g = torch.Generator(device=dev).manual_seed(4)
+    ang = torch.rand(1, 1, T, D // 2, generator=g, device=dev) * 6.283185
+    freqs = torch.polar(torch.ones_like(ang), ang)
+    xs = [torch.randn(1, T, dim, generator=g, device=dev, dtype=torch.float32).to(torch.bfloat16) for _ in range(4)]
+
+    @torch.no_grad()
+    def frame(i: int):
+        x = xs[i % len(xs)]
+        for b in range(blocks):
+            x = frame_blocks[b](x, pos=freqs, enable_3d_rope=True)
+            x = global_blocks[b](x, pos=freqs, enable_3d_rope=True, kv_cache=m, global_idx=b)
+        return x
+
+    for i in range(ANCHOR + WINDOW + warmup):
+        frame(i)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(steps):
+        out = frame(i)
+    torch.cuda.synchronize()
+    dt = (time.perf_counter() - t0) / steps
+    assert torch.isfinite(out.float()).all() and m.device_header()["error"] == 0
+    return {"value": 1.0 / dt, "unit": "frames/s", "ms_per_step": dt * 1e3, "steps": steps,
+            "what": f"{blocks} x (frame block + global block), dim {dim}, {H} heads, MLP {4 * dim}, 1 stream, "
+                    f"{T} tokens/frame, steady-state cache of {(ANCHOR + WINDOW) * T} KV tokens; eager PyTorch-ROCm "
+                    f"for linears/norms/GELU/frame attention, HIP kernels for the cache path"}
+
+
 def main() -> None:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -109,6 +155,8 @@ def main() -> None:
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--blocks", type=int, default=24)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-aggregator", action="store_true",
+                    help="skip the full aggregator-trunk step (frame + global blocks) timed after the hot path")
     ap.add_argument("--mode", choices=["full", "attention", "append", "tables", "copy"], default="full",
                     help="full = the benchmark line; attention/append/tables launch one kernel --steps "
                          "times on the steady-state cache (for rocprofv3 runs); copy = a plain 256 MiB "
@@ -209,6 +257,9 @@ def main() -> None:
                    "avg_launch_us": append_ms * 1e3},
         "tables_step_us": tables_ms * 1e3,
     }
+    if not args.no_aggregator:
+        del m
+        line["aggregator_step"] = aggregator_step(torch, blocks, 20, 3)
     if not args.no_cpu_baseline:
         line["cpu_baseline"] = cpu_baseline(torch, kv_tokens, blocks)
     print(json.dumps(line))
