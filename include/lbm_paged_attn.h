@@ -148,6 +148,28 @@ int lbm_kv_append(const void* k, const void* v, int32_t src_dtype, void* pool,
                   int32_t pool_dtype, const int32_t* append_rows, int32_t n_tokens,
                   int32_t num_heads, int32_t head_dim, int32_t page_size, void* stream);
 
+/* Fused pre-attention producer: per-head LayerNorm of q and k, rotary embedding of q and k
+ * (interleaved pairs), [token][head][dim] layout and the keyframe-gated paged append of k and
+ * v, in one pass over the output of the qkv projection.  Replaces q_norm / k_norm,
+ * apply_rotary_emb and the three permute + contiguous copies of
+ * FlashInferAttention.prepare_qkv (attention.py:402-426, rope.py:438-461) together with the
+ * writes of append_frame (flashinfer_cache.py:215-218, :504-505, :548-549).  Roundings follow
+ * the reference's bf16 sequence when src_dtype is bf16 (LayerNorm output, cos, sin, each
+ * product and each sum rounded to bf16) and plain fp32 arithmetic when it is fp32.
+ *   qkv          [n_tokens][3][num_heads][head_dim], dtype src_dtype
+ *   q_norm_w/_b, k_norm_w/_b   [head_dim] float32 LayerNorm affine; all four NULL = no qk-norm
+ *   rope_cs      [n_tokens][head_dim / 2][2] float32 (cos, sin), i.e. torch.view_as_real of
+ *                the reference's complex freqs; NULL = no rotary embedding
+ *   q_out        [n_tokens][num_heads][head_dim], dtype dst_dtype (the cache dtype)
+ *   k_out, v_out same shape; may be NULL when only the pool copy is wanted (keyframes)
+ *   pool, append_rows, page_size   as lbm_kv_append; append_rows NULL = no pool write
+ * head_dim must be 64. */
+int lbm_qkv_prepare(const void* qkv, int32_t src_dtype, const float* q_norm_w,
+                    const float* q_norm_b, const float* k_norm_w, const float* k_norm_b,
+                    float norm_eps, const float* rope_cs, void* q_out, void* k_out, void* v_out,
+                    int32_t dst_dtype, void* pool, const int32_t* append_rows, int32_t n_tokens,
+                    int32_t num_heads, int32_t head_dim, int32_t page_size, void* stream);
+
 /* Bytes of workspace lbm_attn_run needs for this batch (split-KV partial results). */
 size_t lbm_attn_workspace_bytes(const lbm_attn_stream* streams, int32_t n_streams,
                                 int32_t num_heads, int32_t head_dim);

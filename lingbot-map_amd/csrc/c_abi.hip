@@ -88,6 +88,27 @@ int lbm_kv_append(const void* k, const void* v, int32_t src_dtype, void* pool, i
                            head_dim, page_size, (hipStream_t)stream);
 }
 
+int lbm_qkv_prepare(const void* qkv, int32_t src_dtype, const float* q_norm_w, const float* q_norm_b,
+                    const float* k_norm_w, const float* k_norm_b, float norm_eps, const float* rope_cs,
+                    void* q_out, void* k_out, void* v_out, int32_t dst_dtype, void* pool,
+                    const int32_t* append_rows, int32_t n_tokens, int32_t num_heads, int32_t head_dim,
+                    int32_t page_size, void* stream) {
+  if (!qkv || !q_out) return lbm_fail(LBM_ERR_INVALID, "lbm_qkv_prepare: null qkv or q_out");
+  if (n_tokens < 0 || num_heads <= 0 || page_size <= 0)
+    return lbm_fail(LBM_ERR_INVALID, "lbm_qkv_prepare: bad sizes (tokens %d, heads %d, page %d)", n_tokens, num_heads, page_size);
+  if (head_dim != 64) return lbm_fail(LBM_ERR_UNSUPPORTED, "lbm_qkv_prepare covers head_dim 64 (got %d)", head_dim);
+  if ((src_dtype != LBM_DTYPE_BF16 && src_dtype != LBM_DTYPE_F32) || (dst_dtype != LBM_DTYPE_BF16 && dst_dtype != LBM_DTYPE_F32))
+    return lbm_fail(LBM_ERR_INVALID, "lbm_qkv_prepare: unknown dtype");
+  const int n_norm = (q_norm_w != nullptr) + (q_norm_b != nullptr) + (k_norm_w != nullptr) + (k_norm_b != nullptr);
+  if (n_norm != 0 && n_norm != 4)
+    return lbm_fail(LBM_ERR_INVALID, "lbm_qkv_prepare: the four LayerNorm arrays go together");
+  if ((k_out == nullptr) != (v_out == nullptr)) return lbm_fail(LBM_ERR_INVALID, "lbm_qkv_prepare: k_out and v_out go together");
+  if (append_rows && !pool) return lbm_fail(LBM_ERR_INVALID, "lbm_qkv_prepare: append_rows without a pool");
+  return lbm_launch_qkv_prepare(qkv, src_dtype, q_norm_w, q_norm_b, k_norm_w, k_norm_b, norm_eps, rope_cs, q_out,
+                                k_out, v_out, dst_dtype, pool, append_rows, n_tokens, num_heads, page_size,
+                                (hipStream_t)stream);
+}
+
 static int lbm_check_attn_streams(const lbm_attn_stream* s, int n, const char* who) {
   if (!s) return lbm_fail(LBM_ERR_INVALID, "%s: null streams", who);
   if (n < 1 || n > LBM_MAX_STREAMS) return lbm_fail(LBM_ERR_INVALID, "%s: n_streams %d outside [1, %d]", who, n, LBM_MAX_STREAMS);

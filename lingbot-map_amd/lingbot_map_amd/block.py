@@ -133,6 +133,46 @@ class HipPagedAttention(nn.Module):
         manager.evict_frames(block_idx=global_idx, **self._evict_kwargs(num_register_tokens))
         return manager.compute_attention(global_idx, q)
 
+    # ------------------------------------------------------------------ fused producer
+    def can_fuse(self, manager, pos, enable_3d_rope: bool) -> bool:
+        """Whether the manager's fused producer covers this module's pre-attention ops: plain
+        LayerNorm (or none) on q and k and either no rotary embedding or the interleaved-pair
+        one driven by a complex table (the 2-D variant of the frame blocks is not covered)."""
+        if not hasattr(manager, "step_qkv") or self.head_dim != 64:
+            return False
+        norms = (self.q_norm, self.k_norm)
+        if not (all(isinstance(m, nn.Identity) for m in norms) or
+                all(type(m) is nn.LayerNorm and m.elementwise_affine and m.bias is not None for m in norms)):
+            return False
+        if self.rope is None:
+            return True
+        return bool(enable_3d_rope) and torch.is_tensor(pos) and pos.is_complex()
+
+    def _norm_f32(self, m: nn.LayerNorm):
+        key = (m.weight._version, m.bias._version, m.weight.data_ptr(), m.weight.device)
+        cache = self.__dict__.setdefault("_norm_cache", {})
+        if cache.get(id(m), (None,))[0] != key:
+            cache[id(m)] = (key, (m.weight.detach().float().contiguous(), m.bias.detach().float().contiguous()))
+        return cache[id(m)][1]
+
+    def stream_attend_fused(self, manager, global_idx: int, x: Tensor, pos=None) -> Tensor:
+        """qkv projection, then one kernel for q/k LayerNorm + rotary embedding + layout +
+        paged append, then the paged attention (attention.py:402-426 and block.py:256-278)."""
+        B, N, _ = x.shape
+        qkv = self.qkv(x).reshape(B * N, -1)
+        has_norm = isinstance(self.q_norm, nn.LayerNorm)
+        rope_cs = None
+        if self.rope is not None:
+            rope_cs = torch.view_as_real(pos.to(torch.complex64)).reshape(-1, self.head_dim // 2, 2)
+            assert rope_cs.shape[0] == N, f"rotary table for {rope_cs.shape[0]} tokens, frame has {N}"
+            if B > 1:
+                rope_cs = rope_cs.unsqueeze(0).expand(B, -1, -1, -1).reshape(B * N, self.head_dim // 2, 2)
+        return manager.step_qkv(global_idx, qkv, self._norm_f32(self.q_norm) if has_norm else None,
+                                self._norm_f32(self.k_norm) if has_norm else None, rope_cs,
+                                norm_eps=self.q_norm.eps if has_norm else 1e-5, keyframe=None,
+                                cross_frame_special=self.kv_cache_cross_frame_special,
+                                camera_only=self.kv_cache_camera_only)
+
     def forward(self, x: Tensor, pos=None, num_patches=None, num_special=None, num_frames=None,
                 enable_3d_rope=False, kv_cache=None, global_idx=0, num_frame_per_block=1,
                 num_frame_for_scale=-1, num_register_tokens=4) -> Tensor:
@@ -155,8 +195,11 @@ class HipPagedAttention(nn.Module):
                 kv_cache.append_frame(global_idx, k_all[s:s + tpf].contiguous(), v_all[s:s + tpf].contiguous())
                 kv_cache.evict_frames(block_idx=global_idx, **self._evict_kwargs(num_register_tokens))
         else:
-            q, k, v = self.prepare_qkv(x, pos=pos, enable_3d_rope=enable_3d_rope)
-            out = self.stream_attend(kv_cache, global_idx, q, k, v, num_register_tokens)
+            if self.can_fuse(kv_cache, pos, enable_3d_rope):
+                out = self.stream_attend_fused(kv_cache, global_idx, x, pos)
+            else:
+                q, k, v = self.prepare_qkv(x, pos=pos, enable_3d_rope=enable_3d_rope)
+                out = self.stream_attend(kv_cache, global_idx, q, k, v, num_register_tokens)
             out = out.reshape(B, N, self.num_heads * self.head_dim).to(x.dtype)
         return self.proj(out)
 
@@ -199,8 +242,11 @@ class HipPagedBlock(nn.Module):
                 num_frame_for_scale=-1, num_register_tokens=4) -> Tensor:
         is_streaming = kv_cache is not None and (num_frames is None or num_frames <= 1)
         if is_streaming:
-            q, k, v = self.attn_pre(x, pos=pos, enable_3d_rope=enable_3d_rope)
-            attn_x = self.attn.stream_attend(kv_cache, global_idx, q, k, v, num_register_tokens)
+            if self.attn.can_fuse(kv_cache, pos, enable_3d_rope):
+                attn_x = self.attn.stream_attend_fused(kv_cache, global_idx, self.norm1(x), pos)
+            else:
+                q, k, v = self.attn_pre(x, pos=pos, enable_3d_rope=enable_3d_rope)
+                attn_x = self.attn.stream_attend(kv_cache, global_idx, q, k, v, num_register_tokens)
             attn_x = attn_x.reshape(x.shape[0], x.shape[1], self.attn.num_heads * self.attn.head_dim).to(x.dtype)
             x = x + self.ls1(self.attn.proj(attn_x))
         else:

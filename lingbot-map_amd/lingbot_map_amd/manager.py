@@ -397,14 +397,71 @@ class HipPagedKVCacheManager:
         """One frame of every stream through one block: keyframes append, evict and attend;
         the others attend to the cache plus their own K/V and leave it untouched.  On the
         leading block all table work (allocate, evict, visible rows) is one launch."""
+        k, v = self._check_frame("k", k), self._check_frame("v", v)
+        if v.dtype != k.dtype:
+            v = v.to(k.dtype)
+        ts, keyframe, tail = self._step_tables(block_idx, keyframe, cross_frame_special, camera_only)
+        if any(keyframe):
+            self._scatter(block_idx, ts, k, v)
+            self.frame_count[block_idx] += 1
+        return self._attend_planned(block_idx, q, k if any(tail) else None, v if any(tail) else None)
+
+    def step_qkv(self, block_idx: int, qkv: Tensor, q_norm=None, k_norm=None, rope_cs: Optional[Tensor] = None,
+                 norm_eps: float = 1e-5, keyframe: Optional[Sequence[bool]] = None,
+                 cross_frame_special: bool = True, camera_only: bool = False) -> Tensor:
+        """`step` fed with the output of the qkv projection instead of finished q, k, v: one
+        kernel applies the per-head LayerNorm of q and k, the rotary embedding, lays q out as
+        [token, head, dim] and writes k and v straight into the page pool (attention.py:402-426
+        plus append_frame).  ``qkv``: [streams * tokens_per_frame, 3 * heads * head_dim];
+        ``q_norm`` / ``k_norm``: (weight, bias) float32 tensors of [head_dim] or None;
+        ``rope_cs``: float32 [streams * tokens_per_frame, head_dim / 2, 2] holding (cos, sin),
+        i.e. ``torch.view_as_real`` of the reference's complex ``freqs``, or None."""
+        rows, H, D = self.num_streams * self.tokens_per_frame, self.num_heads, self.head_dim
+        assert qkv.shape[0] == rows and qkv.numel() == rows * 3 * H * D, (
+            f"qkv: expected [{rows}, {3 * H * D}], got {tuple(qkv.shape)}")
+        assert (q_norm is None) == (k_norm is None), "q_norm and k_norm go together"
+        if qkv.dtype not in (torch.bfloat16, torch.float32):
+            qkv = qkv.to(self.dtype)
+        qkv = qkv.contiguous()
+        ts, keyframe, tail = self._step_tables(block_idx, keyframe, cross_frame_special, camera_only)
+        q = torch.empty(rows, H, D, dtype=self.dtype, device=self.device)
+        k = torch.empty_like(q) if any(tail) else None
+        v = torch.empty_like(q) if any(tail) else None
+        # float32 copies of the LayerNorm parameters, kept alive until the launch is queued
+        norm = [self._as_f32(t, D) for t in (tuple(q_norm) + tuple(k_norm))] if q_norm is not None else [None] * 4
+        norm_ptr = [None if t is None else C.c_void_p(t.data_ptr()) for t in norm]
+        if rope_cs is not None:
+            assert rope_cs.dtype == torch.float32 and rope_cs.numel() == rows * D, (
+                f"rope_cs: expected float32 [{rows}, {D // 2}, 2], got {rope_cs.dtype} {tuple(rope_cs.shape)}")
+            rope_cs = rope_cs.contiguous()
+        dt = lambda d: N.DTYPE_BF16 if d == torch.bfloat16 else N.DTYPE_F32
+        N.check(N.lib.lbm_qkv_prepare(
+            C.c_void_p(qkv.data_ptr()), dt(qkv.dtype),
+            norm_ptr[0], norm_ptr[1], norm_ptr[2], norm_ptr[3], float(norm_eps),
+            C.c_void_p(rope_cs.data_ptr()) if rope_cs is not None else None,
+            C.c_void_p(q.data_ptr()), C.c_void_p(k.data_ptr()) if k is not None else None,
+            C.c_void_p(v.data_ptr()) if v is not None else None, dt(self.dtype),
+            C.c_void_p(self.kv_caches[block_idx].data_ptr()),
+            C.c_void_p(self._append_rows[ts].data_ptr()) if any(keyframe) else None,
+            rows, H, D, self.page_size, self._stream_handle()))
+        if any(keyframe):
+            self.frame_count[block_idx] += 1
+        return self._attend_planned(block_idx, q, k, v)
+
+    def _as_f32(self, t: Tensor, n: int) -> Tensor:
+        assert t.numel() == n, f"expected {n} LayerNorm parameters, got {tuple(t.shape)}"
+        return t if (t.dtype == torch.float32 and t.is_contiguous() and t.device == self.device) else \
+            t.detach().to(device=self.device, dtype=torch.float32).contiguous()
+
+    def _step_tables(self, block_idx: int, keyframe: Optional[Sequence[bool]], cross_frame_special: bool,
+                     camera_only: bool):
+        """Table work of one streamed frame (allocate, evict, visible rows; one launch on the
+        leading block).  Returns the table set and the per-stream keyframe / read-only flags."""
         if keyframe is None:
             keyframe = [not self._skip_append] * self.num_streams
         keyframe = [bool(x) and self._active[b] for b, x in enumerate(keyframe)]
         tail = [self._active[b] and not keyframe[b] for b in range(self.num_streams)]
         ts = self._set(block_idx)
-        k, v = self._check_frame("k", k), self._check_frame("v", v)
-        if v.dtype != k.dtype:
-            v = v.to(k.dtype)
         if self._leads(block_idx):
             keep = self._keep_tokens(cross_frame_special, camera_only)
             per = []
@@ -426,10 +483,7 @@ class HipPagedKVCacheManager:
                             "self_tokens": self.tokens_per_frame if tail[b] else 0, "expect_kv_tokens": n})
             self._tables_step(ts, self._ops(per), append_rows=True, kv_rows=True)
             self._plan_valid[ts] = True
-        if any(keyframe):
-            self._scatter(block_idx, ts, k, v)
-            self.frame_count[block_idx] += 1
-        return self._attend_planned(block_idx, q, k if any(tail) else None, v if any(tail) else None)
+        return ts, keyframe, tail
 
     def _attend_planned(self, block_idx: int, q: Tensor, self_k: Optional[Tensor], self_v: Optional[Tensor]) -> Tensor:
         ts = self._set(block_idx)

@@ -16,7 +16,7 @@ def declared_functions():
 
 def test_header_declares_the_expected_entry_points():
     names = declared_functions()
-    for n in ("lbm_tables_step", "lbm_rows_from_pages", "lbm_kv_append", "lbm_attn_run",
+    for n in ("lbm_tables_step", "lbm_rows_from_pages", "lbm_kv_append", "lbm_qkv_prepare", "lbm_attn_run",
               "lbm_attn_workspace_bytes", "lbm_tables_words", "lbm_abi_version", "lbm_last_error"):
         assert n in names
 

@@ -14,7 +14,7 @@ class ReferenceSurfaceOnly:
         object.__setattr__(self, "_m", m)
 
     def __getattr__(self, name):
-        if name in ("step", "set_active_streams"):
+        if name in ("step", "step_qkv", "set_active_streams"):
             raise AttributeError(name)
         return getattr(self._m, name)
 
@@ -22,15 +22,22 @@ class ReferenceSurfaceOnly:
         setattr(self._m, name, value)
 
 
-@pytest.mark.parametrize("reference_calls", [False, True])
-def test_block_stream_matches_dense_cache(reference_calls):
+@pytest.mark.parametrize("reference_calls,rope", [(False, False), (True, False), (False, True), (True, True)])
+def test_block_stream_matches_dense_cache(reference_calls, rope):
+    """reference_calls=False takes the fused producer + `step_qkv`; True the reference's own
+    method sequence.  rope=True adds the interleaved-pair rotary embedding of the global blocks."""
     from lingbot_map_amd import HipPagedBlock, HipPagedKVCacheManager, keyframe_flags, set_skip_append
     from oracle.sdpa_cache import DictCacheOracle
     torch.manual_seed(5)
     dev = torch.device("cuda:0")
     dim, H, T, n_sp, scale, window, blocks = 256, 4, 53, 5, 1, 3, 2
-    mods = [HipPagedBlock(dim, H, init_values=0.1, qk_norm=True, kv_cache_sliding_window=window,
+    mods = [HipPagedBlock(dim, H, init_values=0.1, qk_norm=True, rope=True if rope else None,
+                          kv_cache_sliding_window=window,
                           kv_cache_scale_frames=scale).to(dev, torch.bfloat16).eval() for _ in range(blocks)]
+    for mod in mods:   # non-trivial LayerNorm parameters
+        for ln in (mod.attn.q_norm, mod.attn.k_norm):
+            ln.weight.data.uniform_(0.5, 1.5)
+            ln.bias.data.uniform_(-0.2, 0.2)
     m = HipPagedKVCacheManager(blocks, scale + window + 16, T, H, 64, torch.bfloat16, dev, num_special_tokens=n_sp,
                                scale_frames=scale, sliding_window=window, max_total_frames=64, page_size=16,
                                layout="frame_pages")
@@ -40,11 +47,15 @@ def test_block_stream_matches_dense_cache(reference_calls):
     with torch.no_grad():
         for f, kf in enumerate(flags):
             x = torch.randn(1, T, dim, device=dev).to(torch.bfloat16)
+            pos = None
+            if rope:
+                ang = torch.rand(1, 1, T, 32, device=dev) * 6.283185
+                pos = torch.polar(torch.ones_like(ang), ang)
             set_skip_append(cache, not kf)
             y, y_ref = x, x
             for b, mod in enumerate(mods):
-                y = mod(y, kv_cache=cache, global_idx=b, num_frames=1)
-                q, k, v = mod.attn_pre(y_ref)
+                y = mod(y, pos=pos, enable_3d_rope=rope, kv_cache=cache, global_idx=b, num_frames=1)
+                q, k, v = mod.attn_pre(y_ref, pos=pos, enable_3d_rope=rope)
                 kk, vv = dense[b].visible(k, v, keyframe=kf)
                 a = torch.nn.functional.scaled_dot_product_attention(
                     q.float().permute(1, 0, 2)[None], kk.float().permute(1, 0, 2)[None], vv.float().permute(1, 0, 2)[None])

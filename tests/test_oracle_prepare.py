@@ -1,0 +1,79 @@
+"""Pins of oracle/prepare_qkv.py by what the mathematics fixes (no GPU)."""
+import math
+
+import torch
+
+from oracle.prepare_qkv import apply_rotary_emb, prepare_qkv
+
+
+def _freqs(n, d, seed=0, angle=None):
+    g = torch.Generator().manual_seed(seed)
+    ang = torch.rand(1, 1, n, d // 2, generator=g) * 2 * math.pi if angle is None else torch.full((1, 1, n, d // 2), angle)
+    return torch.polar(torch.ones_like(ang), ang)
+
+
+def test_rotation_by_zero_and_by_a_quarter_turn():
+    g = torch.Generator().manual_seed(1)
+    x = torch.randn(1, 2, 5, 64, generator=g)
+    assert torch.equal(apply_rotary_emb(x, _freqs(5, 64, angle=0.0)), x)
+    quarter = torch.complex(torch.zeros(1, 1, 5, 32), torch.ones(1, 1, 5, 32))   # cos 0, sin 1 exactly
+    y = apply_rotary_emb(x, quarter)
+    assert torch.equal(y[..., 0::2], -x[..., 1::2]) and torch.equal(y[..., 1::2], x[..., 0::2])
+
+
+def test_rotation_equals_the_complex_product_and_keeps_pair_norms():
+    g = torch.Generator().manual_seed(2)
+    x = torch.randn(1, 3, 7, 64, generator=g, dtype=torch.float64)
+    ang = torch.rand(1, 1, 7, 32, generator=g, dtype=torch.float64) * 2 * math.pi
+    fr = torch.polar(torch.ones_like(ang), ang)
+    y = apply_rotary_emb(x, fr)
+    z = torch.view_as_real(torch.view_as_complex(x.reshape(1, 3, 7, 32, 2).contiguous()) * fr).reshape(x.shape)
+    assert (y - z).abs().max().item() < 1e-14
+    n_in = x.reshape(1, 3, 7, 32, 2).norm(dim=-1)
+    n_out = y.reshape(1, 3, 7, 32, 2).norm(dim=-1)
+    assert (n_in - n_out).abs().max().item() < 1e-13
+
+
+def test_layernorm_closed_forms_and_float64_restatement():
+    H, D, n = 2, 64, 6
+    g = torch.Generator().manual_seed(4)
+    w, b = torch.randn(D, generator=g), torch.randn(D, generator=g)
+    const = torch.full((n, 3 * H * D), 1.75)
+    q, k, v = prepare_qkv(const, H, D, (w, b), (w, b), None, eps=1e-5)
+    assert torch.allclose(q, b.expand(n, H, D), atol=1e-6) and torch.allclose(k, b.expand(n, H, D), atol=1e-6)
+    assert torch.equal(v, torch.full((n, H, D), 1.75))
+    x = torch.randn(n, 3 * H * D, generator=g)
+    q, k, v = prepare_qkv(x, H, D, (w, b), (2 * w, -b), None, eps=1e-5)
+    x5 = x.double().reshape(n, 3, H, D)
+    for which, got, ww, bb in ((0, q, w, b), (1, k, 2 * w, -b)):
+        z = x5[:, which]
+        mean = z.mean(-1, keepdim=True)
+        var = ((z - mean) ** 2).mean(-1, keepdim=True)          # biased, as LayerNorm defines it
+        want = (z - mean) / torch.sqrt(var + 1e-5) * ww.double() + bb.double()
+        assert (got.double() - want).abs().max().item() < 1e-5
+    assert torch.equal(v, x.reshape(n, 3, H, D)[:, 2])
+
+
+def test_layout_is_token_head_dim_of_the_projection_output():
+    H, D, n = 3, 64, 4
+    x = torch.arange(n * 3 * H * D, dtype=torch.float32).reshape(n, 3 * H * D)
+    q, k, v = prepare_qkv(x, H, D)
+    x5 = x.reshape(n, 3, H, D)
+    assert torch.equal(q, x5[:, 0]) and torch.equal(k, x5[:, 1]) and torch.equal(v, x5[:, 2])
+    assert q.is_contiguous() and q.shape == (n, H, D)
+
+
+def test_bf16_rounds_where_the_reference_rounds():
+    """bf16 activations: cos and sin are rounded to bf16 and every product and sum is rounded,
+    so the result differs from the fp32 computation rounded once - by a few bf16 ulps at most."""
+    g = torch.Generator().manual_seed(5)
+    H, D, n = 2, 64, 9
+    x = torch.randn(n, 3 * H * D, generator=g)
+    w, b = torch.randn(D, generator=g), 0.1 * torch.randn(D, generator=g)
+    fr = _freqs(n, D, seed=6)
+    q32, k32, _ = prepare_qkv(x.to(torch.bfloat16).float(), H, D, (w.bfloat16().float(), b.bfloat16().float()),
+                              (w.bfloat16().float(), b.bfloat16().float()), fr)
+    q16, k16, _ = prepare_qkv(x.to(torch.bfloat16), H, D, (w.bfloat16(), b.bfloat16()), (w.bfloat16(), b.bfloat16()), fr)
+    assert q16.dtype == torch.bfloat16
+    err = (q16.float() - q32).abs() / q32.abs().clamp_min(1.0)
+    assert 0 < err.max().item() < 4 * 2 ** -8
