@@ -157,8 +157,8 @@ def main() -> None:
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-aggregator", action="store_true",
                     help="skip the full aggregator-trunk step (frame + global blocks) timed after the hot path")
-    ap.add_argument("--mode", choices=["full", "attention", "append", "tables", "copy"], default="full",
-                    help="full = the benchmark line; attention/append/tables launch one kernel --steps "
+    ap.add_argument("--mode", choices=["full", "attention", "append", "prepare", "tables", "copy"], default="full",
+                    help="full = the benchmark line; attention/append/prepare/tables launch one kernel --steps "
                          "times on the steady-state cache (for rocprofv3 runs); copy = a plain 256 MiB "
                          "device copy, the known-size kernel the HBM counters are calibrated on")
     args = ap.parse_args()
@@ -189,6 +189,21 @@ def main() -> None:
     qs, ks, vs = ([torch.randn(T, H, D, generator=g, device=dev, dtype=torch.float32).to(torch.bfloat16)
                    for _ in range(n_sets)] for _ in range(3))
 
+    # inputs of the fused producer: qkv projection output, LayerNorm parameters, rotary table
+    qkv_in = torch.randn(T, 3 * H * D, generator=g, device=dev, dtype=torch.float32).to(torch.bfloat16)
+    ln = [torch.rand(D, generator=g, device=dev) + 0.5 for _ in range(4)]
+    ang = torch.rand(T, D // 2, generator=g, device=dev) * 6.283185
+    rope_cs = torch.stack([ang.cos(), ang.sin()], dim=-1).contiguous()
+    q_tmp = torch.empty(T, H, D, dtype=torch.bfloat16, device=dev)
+
+    def prepare(block: int) -> None:
+        from lingbot_map_amd import _native as N
+        import ctypes as C
+        vp = lambda t: C.c_void_p(t.data_ptr())
+        N.check(N.lib.lbm_qkv_prepare(vp(qkv_in), N.DTYPE_BF16, vp(ln[0]), vp(ln[1]), vp(ln[2]), vp(ln[3]), 1e-5,
+                                      vp(rope_cs), vp(q_tmp), None, None, N.DTYPE_BF16, vp(m.kv_caches[block]),
+                                      vp(m._append_rows[0]), T, H, D, PAGE, m._stream_handle()))
+
     def frame(i: int) -> None:
         for b in range(blocks):
             j = (i + b) % n_sets
@@ -208,6 +223,7 @@ def main() -> None:
         ops = m._ops([{"ops": 16, "expect_kv_tokens": kv_tokens}])
         fn = {"attention": lambda: m._attend_planned(1, qs[0], None, None),
               "append": lambda: m._scatter(1, 0, ks[0], vs[0]),
+              "prepare": lambda: prepare(1),
               "tables": lambda: m._tables_step(0, ops, kv_rows=True)}[args.mode]
         for _ in range(args.warmup):
             fn()
@@ -238,6 +254,9 @@ def main() -> None:
     attn_tflops = flops / (attn_ms * 1e-3) * 1e-12
     append_bytes = 2 * 2 * T * H * D * 2
     append_gbps = append_bytes / (append_ms * 1e-3) * 1e-9
+    prepare_ms = kernel_time_ms(lambda: prepare(1), 100, torch)
+    prepare_bytes = (3 + 3) * T * H * D * 2 + rope_cs.numel() * 4   # read qkv, write q and the K/V rows, read the table
+    prepare_gbps = prepare_bytes / (prepare_ms * 1e-3) * 1e-9
 
     line = {
         "metric": METRIC, "value": fps, "unit": "frames/s", "n_gpus": 1, "steps": args.steps,
@@ -255,6 +274,11 @@ def main() -> None:
         "append": {"bound": "hbm", "achieved": append_gbps, "peak": PEAK_HBM_GBPS, "unit": "GB/s",
                    "frac": append_gbps / PEAK_HBM_GBPS, "bytes_per_launch": append_bytes,
                    "avg_launch_us": append_ms * 1e3},
+        "qkv_prepare": {"bound": "hbm", "achieved": prepare_gbps, "peak": PEAK_HBM_GBPS, "unit": "GB/s",
+                        "frac": prepare_gbps / PEAK_HBM_GBPS, "bytes_per_launch": prepare_bytes,
+                        "avg_launch_us": prepare_ms * 1e3,
+                        "what": "fused q/k LayerNorm + rotary + layout + paged append (replaces the append pass "
+                                "when the block feeds the qkv projection output; not in `value`'s timed loop)"},
         "tables_step_us": tables_ms * 1e3,
     }
     if not args.no_aggregator:

@@ -21,16 +21,13 @@
 
 typedef __attribute__((ext_vector_type(4))) unsigned int u32x4;
 typedef __attribute__((ext_vector_type(4))) float f32x4;
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 
 namespace {
 
-// round-to-nearest-even to bf16 and back, NaN kept quiet (torch's .to(bfloat16))
-__device__ __forceinline__ unsigned int bf16_bits(float f) {
-  unsigned int u = __builtin_bit_cast(unsigned int, f);
-  if ((u & 0x7fffffffu) > 0x7f800000u) return (u >> 16) | 0x40u;
-  return (u + 0x7fffu + ((u >> 16) & 1u)) >> 16;
-}
-__device__ __forceinline__ float round_bf16(float f) { return __builtin_bit_cast(float, bf16_bits(f) << 16); }
+// round-to-nearest-even to bf16 and back (torch's .to(bfloat16)); the hardware conversion
+// v_cvt_pk_bf16_f32 rounds the same way
+__device__ __forceinline__ float round_bf16(float f) { return (float)(__bf16)f; }
 
 template <int DT>  // 0 = bf16, 1 = f32
 __device__ __forceinline__ void load8(const void* base, long long elem, float (&x)[8]) {
@@ -54,10 +51,10 @@ __device__ __forceinline__ void load8(const void* base, long long elem, float (&
 template <int DT>
 __device__ __forceinline__ void store8(void* base, long long elem, const float (&x)[8]) {
   if (DT == 0) {
-    u32x4 a;
+    bf16x8 a;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) a[i] = bf16_bits(x[2 * i]) | (bf16_bits(x[2 * i + 1]) << 16);
-    *(u32x4*)((unsigned short*)base + elem) = a;
+    for (int i = 0; i < 8; ++i) a[i] = (__bf16)x[i];
+    *(bf16x8*)((unsigned short*)base + elem) = a;
   } else {
     f32x4* p = (f32x4*)((float*)base + elem);
     p[0] = f32x4{x[0], x[1], x[2], x[3]};
@@ -81,18 +78,19 @@ struct PrepareArgs {
 template <int SRC, int DST>
 __global__ __launch_bounds__(256) void lbm_qkv_prepare_d64_kernel(PrepareArgs a) {
   const int H = a.num_heads;
-  const long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x;
-  const long long rows = (long long)a.n_tokens * 3 * H;  // (token, q|k|v, head)
+  // 32 rows of (token, q|k|v, head) per workgroup; the host checks that the row count fits 32 bits
+  const unsigned rw = blockIdx.x * 32u + (threadIdx.x >> 3);
+  const unsigned rows = (unsigned)a.n_tokens * 3u * (unsigned)H;
   // whole 8-lane groups leave together, so the shuffles below see all their lanes
-  if ((idx >> 3) >= rows) return;
-  const int c = (int)(idx & 7);
-  const long long rw = idx >> 3;
-  const int h = (int)(rw % H);
-  const int which = (int)((rw / H) % 3);
-  const int t = (int)(rw / (3LL * H));
+  if (rw >= rows) return;
+  const int c = (int)(threadIdx.x & 7);
+  const unsigned th = rw / (unsigned)H;       // token * 3 + which
+  const int h = (int)(rw - th * (unsigned)H);
+  const int t = (int)(th / 3u);
+  const int which = (int)(th - (unsigned)t * 3u);
 
   float x[8];
-  load8<SRC>(a.qkv, rw * 64 + c * 8, x);
+  load8<SRC>(a.qkv, (long long)rw * 64 + c * 8, x);
 
   if (which < 2) {
     if (a.norm_w[which]) {
@@ -109,7 +107,7 @@ __global__ __launch_bounds__(256) void lbm_qkv_prepare_d64_kernel(PrepareArgs a)
       v += __shfl_xor(v, 1);
       v += __shfl_xor(v, 2);
       v += __shfl_xor(v, 4);
-      const float rstd = 1.0f / __builtin_sqrtf(v * (1.0f / 64.0f) + a.eps);
+      const float rstd = __builtin_amdgcn_rsqf(v * (1.0f / 64.0f) + a.eps);  // torch's LayerNorm uses rsqrt too
       const float* w = a.norm_w[which] + c * 8;
       const float* b = a.norm_b[which] + c * 8;
 #pragma unroll
@@ -172,9 +170,10 @@ int lbm_launch_qkv_prepare(const void* qkv, int src_dtype, const float* q_norm_w
   a.append_rows = append_rows;
   a.eps = norm_eps;
   a.n_tokens = n_tokens; a.num_heads = num_heads; a.page_size = page_size;
-  const long long threads = (long long)n_tokens * 3 * num_heads * 8;
-  if (threads == 0) return LBM_OK;
-  const dim3 grid((unsigned)((threads + 255) / 256)), block(256);
+  const long long rows = (long long)n_tokens * 3 * num_heads;
+  if (rows == 0) return LBM_OK;
+  if (rows > 0x7fffffffLL) return lbm_fail(LBM_ERR_UNSUPPORTED, "lbm_qkv_prepare: %lld rows exceed 2^31", rows);
+  const dim3 grid((unsigned)((rows + 31) / 32)), block(256);
 #define LBM_PREPARE_CASE(S, D) hipLaunchKernelGGL((lbm_qkv_prepare_d64_kernel<S, D>), grid, block, 0, stream, a)
   if (src_dtype == LBM_DTYPE_BF16 && dst_dtype == LBM_DTYPE_BF16) LBM_PREPARE_CASE(0, 0);
   else if (src_dtype == LBM_DTYPE_F32 && dst_dtype == LBM_DTYPE_F32) LBM_PREPARE_CASE(1, 1);
