@@ -109,14 +109,15 @@ def aggregator_step(torch, blocks: int, steps: int, warmup: int) -> dict:
     415-529).  The global blocks run the HIP cache path; linears, norms, GELU and the frame
     blocks' dense attention are PyTorch-ROCm library calls.  Patch embedding, the image encoder
     and the prediction heads are not part of the step."""
-    from lingbot_map_amd import HipPagedBlock, HipPagedKVCacheManager
+    from lingbot_map_amd import HipPagedBlock, HipPagedKVCacheManager, RotaryPositionEmbedding2D
     dev = torch.device("cuda:0")
     dim = H * D
     torch.manual_seed(4)
-    kw = dict(dim=dim, num_heads=H, mlp_ratio=4.0, qk_norm=True, init_values=0.01, rope=True,
+    kw = dict(dim=dim, num_heads=H, mlp_ratio=4.0, qk_norm=True, init_values=0.01,
               kv_cache_sliding_window=WINDOW, kv_cache_scale_frames=ANCHOR)
-    frame_blocks = [HipPagedBlock(**kw).to(dev, torch.bfloat16).eval() for _ in range(blocks)]
-    global_blocks = [HipPagedBlock(**kw).to(dev, torch.bfloat16).eval() for _ in range(blocks)]
+    rope2d = RotaryPositionEmbedding2D()    # frame blocks: 2-D embedding over the 27 x 37 patch grid
+    frame_blocks = [HipPagedBlock(rope=rope2d, **kw).to(dev, torch.bfloat16).eval() for _ in range(blocks)]
+    global_blocks = [HipPagedBlock(rope=True, **kw).to(dev, torch.bfloat16).eval() for _ in range(blocks)]
     m = HipPagedKVCacheManager(blocks, ANCHOR + WINDOW + 16, T, H, D, torch.bfloat16, dev,
                                num_special_tokens=N_SPECIAL, scale_frames=ANCHOR, sliding_window=WINDOW,
                                max_total_frames=256, page_size=PAGE, layout="frame_pages")
@@ -124,12 +125,16 @@ def aggregator_step(torch, blocks: int, steps: int, warmup: int) -> dict:
     ang = torch.rand(1, 1, T, D // 2, generator=g, device=dev) * 6.283185
     freqs = torch.polar(torch.ones_like(ang), ang)
     xs = [torch.randn(1, T, dim, generator=g, device=dev, dtype=torch.float32).to(torch.bfloat16) for _ in range(4)]
+    # (y, x) of every token: specials at (0, 0), patches on the grid shifted by one (lingbot_map/aggregator/base.py:434-440)
+    grid = torch.cartesian_prod(torch.arange(27, device=dev), torch.arange(37, device=dev)) + 1
+    pos2d = torch.cat([torch.zeros(N_SPECIAL, 2, dtype=grid.dtype, device=dev), grid])[None].contiguous()
+    assert pos2d.shape == (1, T, 2)
 
     @torch.no_grad()
     def frame(i: int):
         x = xs[i % len(xs)]
         for b in range(blocks):
-            x = frame_blocks[b](x, pos=freqs, enable_3d_rope=True)
+            x = frame_blocks[b](x, pos=pos2d)
             x = global_blocks[b](x, pos=freqs, enable_3d_rope=True, kv_cache=m, global_idx=b)
         return x
 
@@ -145,7 +150,8 @@ def aggregator_step(torch, blocks: int, steps: int, warmup: int) -> dict:
     return {"value": 1.0 / dt, "unit": "frames/s", "ms_per_step": dt * 1e3, "steps": steps,
             "what": f"{blocks} x (frame block + global block), dim {dim}, {H} heads, MLP {4 * dim}, 1 stream, "
                     f"{T} tokens/frame, steady-state cache of {(ANCHOR + WINDOW) * T} KV tokens; eager PyTorch-ROCm "
-                    f"for linears/norms/GELU/frame attention, HIP kernels for the cache path"}
+                    f"for linears/norms/GELU, HIP kernels for q/k norm + rotary + append, the cache path and "
+                    f"the frame blocks' dense attention"}
 
 
 def main() -> None:
@@ -201,7 +207,7 @@ def main() -> None:
         import ctypes as C
         vp = lambda t: C.c_void_p(t.data_ptr())
         N.check(N.lib.lbm_qkv_prepare(vp(qkv_in), N.DTYPE_BF16, vp(ln[0]), vp(ln[1]), vp(ln[2]), vp(ln[3]), 1e-5,
-                                      vp(rope_cs), vp(q_tmp), None, None, N.DTYPE_BF16, vp(m.kv_caches[block]),
+                                      vp(rope_cs), N.ROPE_INTERLEAVED, vp(q_tmp), None, None, N.DTYPE_BF16, vp(m.kv_caches[block]),
                                       vp(m._append_rows[0]), T, H, D, PAGE, m._stream_handle()))
 
     def frame(i: int) -> None:

@@ -38,6 +38,10 @@ extern "C" {
 #define LBM_LAYOUT_TWO_STREAM 0  /* reference: patch pages + packed special stream         */
 #define LBM_LAYOUT_FRAME_PAGES 1 /* whole frame in pages; eviction compacts index-only     */
 
+/* pairing of the rotary embedding in lbm_qkv_prepare */
+#define LBM_ROPE_INTERLEAVED 0
+#define LBM_ROPE_HALF_SPLIT 1
+
 #define LBM_MAX_STREAMS 16
 
 /* Table operations, executed in this fixed order when several bits are set. */
@@ -158,17 +162,22 @@ int lbm_kv_append(const void* k, const void* v, int32_t src_dtype, void* pool,
  * product and each sum rounded to bf16) and plain fp32 arithmetic when it is fp32.
  *   qkv          [n_tokens][3][num_heads][head_dim], dtype src_dtype
  *   q_norm_w/_b, k_norm_w/_b   [head_dim] float32 LayerNorm affine; all four NULL = no qk-norm
- *   rope_cs      [n_tokens][head_dim / 2][2] float32 (cos, sin), i.e. torch.view_as_real of
- *                the reference's complex freqs; NULL = no rotary embedding
+ *   rope_cs      NULL = no rotary embedding; otherwise float32 (cos, sin) pairs:
+ *                LBM_ROPE_INTERLEAVED  [n_tokens][head_dim / 2][2], element pairs (2i, 2i+1),
+ *                  i.e. torch.view_as_real of the complex freqs of apply_rotary_emb (rope.py:438-461)
+ *                LBM_ROPE_HALF_SPLIT   [n_tokens][head_dim][2], one (cos, sin) per element; in each
+ *                  half of head_dim element j pairs with j + head_dim/4: x*cos + rotate(x)*sin of
+ *                  RotaryPositionEmbedding2D (rope.py:123-198)
  *   q_out        [n_tokens][num_heads][head_dim], dtype dst_dtype (the cache dtype)
  *   k_out, v_out same shape; may be NULL when only the pool copy is wanted (keyframes)
  *   pool, append_rows, page_size   as lbm_kv_append; append_rows NULL = no pool write
  * head_dim must be 64. */
 int lbm_qkv_prepare(const void* qkv, int32_t src_dtype, const float* q_norm_w,
                     const float* q_norm_b, const float* k_norm_w, const float* k_norm_b,
-                    float norm_eps, const float* rope_cs, void* q_out, void* k_out, void* v_out,
-                    int32_t dst_dtype, void* pool, const int32_t* append_rows, int32_t n_tokens,
-                    int32_t num_heads, int32_t head_dim, int32_t page_size, void* stream);
+                    float norm_eps, const float* rope_cs, int32_t rope_layout, void* q_out,
+                    void* k_out, void* v_out, int32_t dst_dtype, void* pool,
+                    const int32_t* append_rows, int32_t n_tokens, int32_t num_heads,
+                    int32_t head_dim, int32_t page_size, void* stream);
 
 /* Bytes of workspace lbm_attn_run needs for this batch (split-KV partial results). */
 size_t lbm_attn_workspace_bytes(const lbm_attn_stream* streams, int32_t n_streams,

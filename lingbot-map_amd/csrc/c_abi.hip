@@ -90,7 +90,7 @@ int lbm_kv_append(const void* k, const void* v, int32_t src_dtype, void* pool, i
 
 int lbm_qkv_prepare(const void* qkv, int32_t src_dtype, const float* q_norm_w, const float* q_norm_b,
                     const float* k_norm_w, const float* k_norm_b, float norm_eps, const float* rope_cs,
-                    void* q_out, void* k_out, void* v_out, int32_t dst_dtype, void* pool,
+                    int32_t rope_layout, void* q_out, void* k_out, void* v_out, int32_t dst_dtype, void* pool,
                     const int32_t* append_rows, int32_t n_tokens, int32_t num_heads, int32_t head_dim,
                     int32_t page_size, void* stream) {
   if (!qkv || !q_out) return lbm_fail(LBM_ERR_INVALID, "lbm_qkv_prepare: null qkv or q_out");
@@ -104,7 +104,9 @@ int lbm_qkv_prepare(const void* qkv, int32_t src_dtype, const float* q_norm_w, c
     return lbm_fail(LBM_ERR_INVALID, "lbm_qkv_prepare: the four LayerNorm arrays go together");
   if ((k_out == nullptr) != (v_out == nullptr)) return lbm_fail(LBM_ERR_INVALID, "lbm_qkv_prepare: k_out and v_out go together");
   if (append_rows && !pool) return lbm_fail(LBM_ERR_INVALID, "lbm_qkv_prepare: append_rows without a pool");
-  return lbm_launch_qkv_prepare(qkv, src_dtype, q_norm_w, q_norm_b, k_norm_w, k_norm_b, norm_eps, rope_cs, q_out,
+  if (rope_cs && rope_layout != LBM_ROPE_INTERLEAVED && rope_layout != LBM_ROPE_HALF_SPLIT)
+    return lbm_fail(LBM_ERR_INVALID, "lbm_qkv_prepare: unknown rope_layout %d", rope_layout);
+  return lbm_launch_qkv_prepare(qkv, src_dtype, q_norm_w, q_norm_b, k_norm_w, k_norm_b, norm_eps, rope_cs, rope_layout, q_out,
                                 k_out, v_out, dst_dtype, pool, append_rows, n_tokens, num_heads, page_size,
                                 (hipStream_t)stream);
 }

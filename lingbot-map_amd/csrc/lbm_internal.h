@@ -25,9 +25,9 @@ int lbm_launch_append(const void* k, const void* v, int src_dtype, void* pool, i
 
 int lbm_launch_qkv_prepare(const void* qkv, int src_dtype, const float* q_norm_w, const float* q_norm_b,
                            const float* k_norm_w, const float* k_norm_b, float norm_eps,
-                           const float* rope_cs, void* q_out, void* k_out, void* v_out, int dst_dtype,
-                           void* pool, const int32_t* append_rows, int n_tokens, int num_heads,
-                           int page_size, hipStream_t stream);
+                           const float* rope_cs, int rope_layout, void* q_out, void* k_out, void* v_out,
+                           int dst_dtype, void* pool, const int32_t* append_rows, int n_tokens,
+                           int num_heads, int page_size, hipStream_t stream);
 
 // Split-KV schedule of one attention call, computed on the host from token counts only.
 struct LbmAttnStreamPlan {

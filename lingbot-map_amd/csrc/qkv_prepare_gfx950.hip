@@ -7,8 +7,9 @@
 //
 // HBM-bound: qkv is read once, q and the pool rows are written once.  Eight lanes own one
 // (token, head) row of 64 elements, 8 elements (16 bytes of bf16) each; the LayerNorm
-// statistics are reduced over those eight lanes with DPP shuffles, the rotary pairs
-// (2i, 2i+1) stay inside a lane.
+// statistics are reduced over those eight lanes with DPP shuffles; the interleaved rotary
+// pairs (2i, 2i+1) of the global blocks stay inside a lane, the half-split pairs (j, j+16) of
+// the frame blocks' 2-D embedding (lingbot_map/layers/rope.py:123-198) sit two lanes apart.
 //
 // Arithmetic follows the reference's order of roundings.  For bf16 activations torch computes
 // the LayerNorm in fp32 and rounds its output to bf16; apply_rotary_emb then rounds cos and
@@ -67,6 +68,7 @@ struct PrepareArgs {
   const float* norm_w[2];  // q, k
   const float* norm_b[2];
   const float* rope_cs;
+  int rope_layout;
   void* out[3];            // q_out, k_out, v_out
   void* pool;
   const int32_t* append_rows;
@@ -116,7 +118,7 @@ __global__ __launch_bounds__(256) void lbm_qkv_prepare_d64_kernel(PrepareArgs a)
         x[i] = SRC == 0 ? round_bf16(y) : y;
       }
     }
-    if (a.rope_cs) {
+    if (a.rope_cs && a.rope_layout == LBM_ROPE_INTERLEAVED) {
       const f32x4* cs = (const f32x4*)(a.rope_cs + ((long long)t * 32 + c * 4) * 2);
 #pragma unroll
       for (int p = 0; p < 2; ++p) {
@@ -134,6 +136,32 @@ __global__ __launch_bounds__(256) void lbm_qkv_prepare_d64_kernel(PrepareArgs a)
           } else {
             x[i] = __fsub_rn(__fmul_rn(x1, co), __fmul_rn(x2, si));
             x[i + 1] = __fadd_rn(__fmul_rn(x1, si), __fmul_rn(x2, co));
+          }
+        }
+      }
+    } else if (a.rope_cs) {
+      // half-split pairs: in each 32-element half, element j < 16 rotates with element j + 16
+      // (x * cos + rotate(x) * sin with rotate = (-second, first), rope.py:123-152); the partner
+      // sits two lanes away in the 8-lane group
+      const f32x4* cs = (const f32x4*)(a.rope_cs + ((long long)t * 64 + c * 8) * 2);
+      const bool first = (c & 2) == 0;
+#pragma unroll
+      for (int p = 0; p < 4; ++p) {
+        const f32x4 q4 = cs[p];  // (cos, sin) of two elements
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+          const int i = 2 * p + j;
+          float co = q4[2 * j], si = q4[2 * j + 1];
+          const float own = x[i];
+          const float other = __shfl_xor(own, 2);
+          if (SRC == 0) {
+            co = round_bf16(co);
+            si = round_bf16(si);
+            const float a0 = round_bf16(__fmul_rn(own, co)), b0 = round_bf16(__fmul_rn(other, si));
+            x[i] = round_bf16(first ? __fsub_rn(a0, b0) : __fadd_rn(a0, b0));
+          } else {
+            const float a0 = __fmul_rn(own, co), b0 = __fmul_rn(other, si);
+            x[i] = first ? __fsub_rn(a0, b0) : __fadd_rn(a0, b0);
           }
         }
       }
@@ -157,14 +185,15 @@ __global__ __launch_bounds__(256) void lbm_qkv_prepare_d64_kernel(PrepareArgs a)
 
 int lbm_launch_qkv_prepare(const void* qkv, int src_dtype, const float* q_norm_w, const float* q_norm_b,
                            const float* k_norm_w, const float* k_norm_b, float norm_eps,
-                           const float* rope_cs, void* q_out, void* k_out, void* v_out, int dst_dtype,
-                           void* pool, const int32_t* append_rows, int n_tokens, int num_heads,
-                           int page_size, hipStream_t stream) {
+                           const float* rope_cs, int rope_layout, void* q_out, void* k_out, void* v_out,
+                           int dst_dtype, void* pool, const int32_t* append_rows, int n_tokens,
+                           int num_heads, int page_size, hipStream_t stream) {
   PrepareArgs a;
   a.qkv = qkv;
   a.norm_w[0] = q_norm_w; a.norm_b[0] = q_norm_b;
   a.norm_w[1] = k_norm_w; a.norm_b[1] = k_norm_b;
   a.rope_cs = rope_cs;
+  a.rope_layout = rope_layout;
   a.out[0] = q_out; a.out[1] = k_out; a.out[2] = v_out;
   a.pool = pool;
   a.append_rows = append_rows;

@@ -6,7 +6,9 @@
 if it has not been built: there is no CPU path.
 """
 from . import _native  # noqa: F401  (loads the library, fails loudly when missing)
-from .block import HipPagedAttention, HipPagedBlock, keyframe_flags, set_skip_append
+from .block import HipPagedAttention, HipPagedBlock, RotaryPositionEmbedding2D, keyframe_flags, set_skip_append
+from .dense import dense_attention
 from .manager import HipPagedKVCacheManager
 
-__all__ = ["HipPagedKVCacheManager", "HipPagedAttention", "HipPagedBlock", "keyframe_flags", "set_skip_append"]
+__all__ = ["HipPagedKVCacheManager", "HipPagedAttention", "HipPagedBlock", "RotaryPositionEmbedding2D",
+           "dense_attention", "keyframe_flags", "set_skip_append"]

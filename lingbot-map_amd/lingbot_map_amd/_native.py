@@ -11,6 +11,7 @@ from .build import LIB_PATH
 OK, ERR_INVALID, ERR_UNSUPPORTED, ERR_WORKSPACE, ERR_HIP = 0, 1, 2, 3, 4
 DTYPE_BF16, DTYPE_F32 = 0, 1
 LAYOUT_TWO_STREAM, LAYOUT_FRAME_PAGES = 0, 1
+ROPE_INTERLEAVED, ROPE_HALF_SPLIT = 0, 1
 MAX_STREAMS = 16
 OP_RESET, OP_ROLLBACK, OP_APPEND, OP_EVICT, OP_PLAN = 1, 2, 4, 8, 16
 TERR_NAMES = {1: "patch page pool exhausted", 2: "special page pool exhausted", 4: "window ring full",
@@ -60,7 +61,7 @@ def _load():
     lib.lbm_kv_append.restype = C.c_int
     lib.lbm_kv_append.argtypes = [vp, vp, i32, vp, i32, vp, i32, i32, i32, i32, vp]
     lib.lbm_qkv_prepare.restype = C.c_int
-    lib.lbm_qkv_prepare.argtypes = [vp, i32, vp, vp, vp, vp, C.c_float, vp, vp, vp, vp, i32, vp, vp, i32, i32, i32, i32, vp]
+    lib.lbm_qkv_prepare.argtypes = [vp, i32, vp, vp, vp, vp, C.c_float, vp, i32, vp, vp, vp, i32, vp, vp, i32, i32, i32, i32, vp]
     lib.lbm_attn_workspace_bytes.restype = C.c_size_t
     lib.lbm_attn_workspace_bytes.argtypes = [p(AttnStream), i32, i32, i32]
     lib.lbm_attn_run.restype = C.c_int

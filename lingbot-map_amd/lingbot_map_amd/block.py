@@ -37,6 +37,65 @@ def apply_rotary_emb(x: Tensor, freqs: Tensor) -> Tensor:
     return torch.stack([x1 * cos - x2 * sin, x1 * sin + x2 * cos], dim=-1).reshape(x.shape)
 
 
+class RotaryPositionEmbedding2D(nn.Module):
+    """2-D rotary embedding of the frame blocks (lingbot_map/layers/rope.py:64-198): head_dim is
+    split into a vertical and a horizontal half; in each, element j rotates with element
+    j + dim/4 by ``pos * frequency^(-4j/dim)``.  ``forward`` is the reference's sequence of
+    torch operations; ``cos_sin_table`` hands the same cos / sin values to the fused producer."""
+
+    def __init__(self, frequency: float = 100.0, scaling_factor: float = 1.0) -> None:
+        super().__init__()
+        self.base_frequency = frequency
+        self.scaling_factor = scaling_factor
+        self.frequency_cache = {}
+        self._table_cache = {}
+
+    def _compute_frequency_components(self, dim: int, seq_len: int, device, dtype):
+        key = (dim, seq_len, device, dtype)
+        if key not in self.frequency_cache:
+            exponents = torch.arange(0, dim, 2, device=device).float() / dim
+            inv_freq = 1.0 / (self.base_frequency ** exponents)
+            positions = torch.arange(seq_len, device=device, dtype=inv_freq.dtype)
+            angles = torch.einsum("i,j->ij", positions, inv_freq).to(dtype)
+            angles = torch.cat((angles, angles), dim=-1)
+            self.frequency_cache[key] = (angles.cos().to(dtype).detach().clone(), angles.sin().to(dtype).detach().clone())
+        return self.frequency_cache[key]
+
+    @staticmethod
+    def _rotate_features(x: Tensor) -> Tensor:
+        d = x.shape[-1]
+        return torch.cat((-x[..., d // 2:], x[..., : d // 2]), dim=-1)
+
+    def _apply_1d_rope(self, tokens: Tensor, positions: Tensor, cos_comp: Tensor, sin_comp: Tensor) -> Tensor:
+        cos = F.embedding(positions, cos_comp)[:, None, :, :]
+        sin = F.embedding(positions, sin_comp)[:, None, :, :]
+        return (tokens * cos) + (self._rotate_features(tokens) * sin)
+
+    def forward(self, tokens: Tensor, positions: Tensor) -> Tensor:
+        assert tokens.size(-1) % 2 == 0, "Feature dimension must be even"
+        assert positions.ndim == 3 and positions.shape[-1] == 2, "Positions must have shape (batch_size, n_tokens, 2)"
+        feature_dim = tokens.size(-1) // 2
+        cos_comp, sin_comp = self._compute_frequency_components(feature_dim, positions.shape[1], tokens.device, tokens.dtype)
+        vertical, horizontal = tokens.chunk(2, dim=-1)
+        vertical = self._apply_1d_rope(vertical, positions[..., 0], cos_comp, sin_comp)
+        horizontal = self._apply_1d_rope(horizontal, positions[..., 1], cos_comp, sin_comp)
+        return torch.cat((vertical, horizontal), dim=-1)
+
+    def cos_sin_table(self, positions: Tensor, head_dim: int, dtype: torch.dtype) -> Tensor:
+        """float32 ``[B * N, head_dim, 2]`` (cos, sin) per token and element, the values ``forward``
+        multiplies with for activations of ``dtype``.  Cached per positions tensor."""
+        key = (positions.data_ptr(), tuple(positions.shape), positions._version, head_dim, dtype)
+        hit = self._table_cache.get("last")
+        if hit is not None and hit[0] == key:
+            return hit[1]
+        cos_comp, sin_comp = self._compute_frequency_components(head_dim // 2, positions.shape[1], positions.device, dtype)
+        cos = torch.cat((F.embedding(positions[..., 0], cos_comp), F.embedding(positions[..., 1], cos_comp)), dim=-1)
+        sin = torch.cat((F.embedding(positions[..., 0], sin_comp), F.embedding(positions[..., 1], sin_comp)), dim=-1)
+        table = torch.stack((cos.float(), sin.float()), dim=-1).reshape(-1, head_dim, 2).contiguous()
+        self._table_cache["last"] = (key, table, positions)   # positions kept alive with its key
+        return table
+
+
 class LayerScale(nn.Module):
     """lingbot_map/layers/layer_scale.py"""
 
@@ -173,6 +232,56 @@ class HipPagedAttention(nn.Module):
                                 cross_frame_special=self.kv_cache_cross_frame_special,
                                 camera_only=self.kv_cache_camera_only)
 
+    def can_fuse_dense(self, x: Tensor, pos, enable_3d_rope: bool) -> bool:
+        """Whether the cache-less attention of a batch of frames can run as fused producer +
+        paged kernel: GPU tensors, head_dim 64, plain LayerNorm or none on q and k, and no rotary
+        embedding, the interleaved one with a complex table, or this package's 2-D one."""
+        from . import _native as N
+        if not (x.is_cuda and self.head_dim == 64 and x.dtype in (torch.bfloat16, torch.float32)):
+            return False
+        if not 1 <= x.shape[0] <= N.MAX_STREAMS:
+            return False
+        norms = (self.q_norm, self.k_norm)
+        if not (all(isinstance(m, nn.Identity) for m in norms) or
+                all(type(m) is nn.LayerNorm and m.elementwise_affine and m.bias is not None for m in norms)):
+            return False
+        if self.rope is None:
+            return True
+        if enable_3d_rope:
+            return torch.is_tensor(pos) and pos.is_complex()
+        return isinstance(self.rope, RotaryPositionEmbedding2D) and torch.is_tensor(pos) and pos.shape[0] in (1, x.shape[0])
+
+    def dense_attend_fused(self, x: Tensor, pos=None, enable_3d_rope: bool = False) -> Tensor:
+        """Attention of every frame of the batch over its own tokens (attention.py:446-465):
+        qkv projection, one producer kernel, the paged kernel over a trivial row table."""
+        import ctypes as C
+        from . import _native as N
+        from .dense import dense_attention
+        B, n, _ = x.shape
+        H, D = self.num_heads, self.head_dim
+        qkv = self.qkv(x).reshape(B * n, -1).contiguous()
+        has_norm = isinstance(self.q_norm, nn.LayerNorm)
+        norm = (self._norm_f32(self.q_norm) + self._norm_f32(self.k_norm)) if has_norm else (None,) * 4
+        table, layout = None, N.ROPE_INTERLEAVED
+        if self.rope is not None and enable_3d_rope:
+            table = torch.view_as_real(pos.to(torch.complex64)).reshape(-1, D // 2, 2)
+            if B > 1:
+                table = table.unsqueeze(0).expand(B, -1, -1, -1).reshape(B * n, D // 2, 2)
+            table = table.contiguous()
+        elif self.rope is not None:
+            positions = pos if pos.shape[0] == B else pos.expand(B, -1, -1)
+            table, layout = self.rope.cos_sin_table(positions, D, x.dtype), N.ROPE_HALF_SPLIT
+        if table is not None:
+            assert table.shape[0] == B * n and table.dtype == torch.float32
+        q, k, v = (torch.empty(B * n, H, D, dtype=x.dtype, device=x.device) for _ in range(3))
+        p = lambda t: None if t is None else C.c_void_p(t.data_ptr())
+        dt = N.DTYPE_BF16 if x.dtype == torch.bfloat16 else N.DTYPE_F32
+        N.check(N.lib.lbm_qkv_prepare(
+            p(qkv), dt, p(norm[0]), p(norm[1]), p(norm[2]), p(norm[3]),
+            float(self.q_norm.eps) if has_norm else 1e-5, p(table), layout, p(q), p(k), p(v), dt, None, None,
+            B * n, H, D, 16, C.c_void_p(torch.cuda.current_stream(x.device).cuda_stream)))
+        return dense_attention(q, k, v, num_streams=B).reshape(B, n, H * D)
+
     def forward(self, x: Tensor, pos=None, num_patches=None, num_special=None, num_frames=None,
                 enable_3d_rope=False, kv_cache=None, global_idx=0, num_frame_per_block=1,
                 num_frame_for_scale=-1, num_register_tokens=4) -> Tensor:
@@ -180,8 +289,11 @@ class HipPagedAttention(nn.Module):
         has_manager = kv_cache is not None and hasattr(kv_cache, "append_frame")
         if not has_manager:
             # batch mode (attention.py:446-465)
-            q, k, v = self._qkv(x, pos, enable_3d_rope)
-            out = F.scaled_dot_product_attention(q, k, v).transpose(1, 2).reshape(B, N, -1)
+            if self.can_fuse_dense(x, pos, enable_3d_rope):
+                out = self.dense_attend_fused(x, pos, enable_3d_rope)
+            else:
+                q, k, v = self._qkv(x, pos, enable_3d_rope)
+                out = F.scaled_dot_product_attention(q, k, v).transpose(1, 2).reshape(B, N, -1)
         elif num_frames is not None and num_frames > 1:
             # anchor pass over several frames: dense attention among them, then one append
             # and eviction per frame (attention.py:475-511)

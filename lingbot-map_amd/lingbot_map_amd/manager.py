@@ -438,7 +438,7 @@ class HipPagedKVCacheManager:
         N.check(N.lib.lbm_qkv_prepare(
             C.c_void_p(qkv.data_ptr()), dt(qkv.dtype),
             norm_ptr[0], norm_ptr[1], norm_ptr[2], norm_ptr[3], float(norm_eps),
-            C.c_void_p(rope_cs.data_ptr()) if rope_cs is not None else None,
+            C.c_void_p(rope_cs.data_ptr()) if rope_cs is not None else None, N.ROPE_INTERLEAVED,
             C.c_void_p(q.data_ptr()), C.c_void_p(k.data_ptr()) if k is not None else None,
             C.c_void_p(v.data_ptr()) if v is not None else None, dt(self.dtype),
             C.c_void_p(self.kv_caches[block_idx].data_ptr()),

@@ -11,6 +11,11 @@ Restated from the reference (paths relative to its checkout):
   to the activations' dtype, plain elementwise arithmetic in that dtype
                                            lingbot_map/layers/rope.py:438-461
 
+* 2-D rotary embedding of the frame blocks: head_dim split into a vertical and a horizontal
+  half, each rotated as x * cos + rotate(x) * sin with rotate = (-second half, first half),
+  angle table pos * base^(-2j/dim) repeated twice, computed and cast in the activations' dtype
+                                           lingbot_map/layers/rope.py:86-198
+
 ``prepare_qkv`` runs the same torch operations in the same order and dtype as the reference,
 so for bf16 activations every intermediate is rounded where the reference rounds it
 (LayerNorm output, cos, sin, each product, each sum).
@@ -20,7 +25,9 @@ degrees maps (a, b) to (-b, a); in fp32 the result equals the complex product
 ``view_as_complex(x) * freqs`` and preserves the norm of every pair; LayerNorm of a
 constant row is the bias and otherwise equals a float64 restatement of
 (x - mean) / sqrt(var + eps) * w + b; v passes through unchanged; the layout is the
-transpose the reference's permutes describe.
+transpose the reference's permutes describe.  ``rope2d``: position (0, 0) is the identity; in
+float64 element j of a half and element j + dim/4 rotate by pos * base^(-4j/dim) (an explicit
+loop restates it), pair norms are kept, the vertical half ignores x and the horizontal half y.
 """
 
 from __future__ import annotations
@@ -42,12 +49,44 @@ def apply_rotary_emb(x: torch.Tensor, freqs: torch.Tensor) -> torch.Tensor:
     return torch.stack([out1, out2], dim=-1).reshape(x.shape)
 
 
+def rope2d_tables(dim: int, seq_len: int, dtype: torch.dtype, base: float = 100.0):
+    """cos / sin tables ``[seq_len, dim]`` of one spatial direction (rope.py:86-122)."""
+    exponents = torch.arange(0, dim, 2).float() / dim
+    inv_freq = 1.0 / (base ** exponents)
+    positions = torch.arange(seq_len, dtype=inv_freq.dtype)
+    angles = torch.einsum("i,j->ij", positions, inv_freq)
+    angles = angles.to(dtype)
+    angles = torch.cat((angles, angles), dim=-1)
+    return angles.cos().to(dtype), angles.sin().to(dtype)
+
+
+def rope2d(tokens: torch.Tensor, positions: torch.Tensor, base: float = 100.0) -> torch.Tensor:
+    """tokens ``[B, H, N, D]``, positions ``[B, N, 2]`` integer (y, x) (rope.py:154-198)."""
+    feature_dim = tokens.size(-1) // 2
+    cos_comp, sin_comp = rope2d_tables(feature_dim, positions.shape[1], tokens.dtype, base)
+
+    def rotate(x):
+        d = x.shape[-1]
+        return torch.cat((-x[..., d // 2:], x[..., : d // 2]), dim=-1)
+
+    def one(x, pos):
+        cos = F.embedding(pos, cos_comp)[:, None, :, :]
+        sin = F.embedding(pos, sin_comp)[:, None, :, :]
+        return (x * cos) + (rotate(x) * sin)
+
+    vert, horiz = tokens.chunk(2, dim=-1)
+    return torch.cat((one(vert, positions[..., 0]), one(horiz, positions[..., 1])), dim=-1)
+
+
 def prepare_qkv(qkv: torch.Tensor, num_heads: int, head_dim: int,
                 q_norm: Optional[Tuple[torch.Tensor, torch.Tensor]] = None,
                 k_norm: Optional[Tuple[torch.Tensor, torch.Tensor]] = None,
-                freqs: Optional[torch.Tensor] = None, eps: float = 1e-5):
+                freqs: Optional[torch.Tensor] = None, eps: float = 1e-5,
+                positions: Optional[torch.Tensor] = None):
     """qkv ``[N, 3 * H * D]`` (one stream, batch of one) -> q, k, v of ``[N, H, D]``
-    (attention.py:412-426).  ``q_norm`` / ``k_norm``: (weight, bias) in the activations' dtype."""
+    (attention.py:412-426).  ``q_norm`` / ``k_norm``: (weight, bias) in the activations' dtype.
+    ``freqs``: complex table of the interleaved embedding (global blocks); ``positions``
+    ``[N, 2]``: the 2-D embedding of the frame blocks instead."""
     n = qkv.shape[0]
     t = qkv.reshape(1, n, 3, num_heads, head_dim).permute(2, 0, 3, 1, 4)
     q, k, v = t.unbind(0)  # each [1, H, N, D]
@@ -57,5 +96,8 @@ def prepare_qkv(qkv: torch.Tensor, num_heads: int, head_dim: int,
     if freqs is not None:
         q = apply_rotary_emb(q, freqs)
         k = apply_rotary_emb(k, freqs)
+    elif positions is not None:
+        q = rope2d(q, positions[None])
+        k = rope2d(k, positions[None])
     nhd = lambda z: z.squeeze(0).permute(1, 0, 2).contiguous()
     return nhd(q), nhd(k), nhd(v)

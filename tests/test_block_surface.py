@@ -62,3 +62,22 @@ def test_keyframe_flags_follow_driver_rule():
     assert keyframe_flags(10, 1, 4) == [True, True, False, False, False, True, False, False, False, True]
     assert sum(keyframe_flags(320, 1, 4)) == 81
     assert all(keyframe_flags(20, 8, 1))
+
+
+def test_rope2d_module_equals_the_oracle_and_its_table():
+    import torch
+    from lingbot_map_amd import RotaryPositionEmbedding2D
+    from oracle.prepare_qkv import rope2d
+    g = torch.Generator().manual_seed(3)
+    B, H, N, D = 2, 3, 20, 64
+    pos = torch.stack([torch.randint(0, N, (B, N), generator=g), torch.randint(0, N, (B, N), generator=g)], -1)
+    rope = RotaryPositionEmbedding2D()
+    for dtype in (torch.float32, torch.bfloat16):
+        x = torch.randn(B, H, N, D, generator=g).to(dtype)
+        assert torch.equal(rope(x, pos), rope2d(x, pos))
+        table = rope.cos_sin_table(pos, D, dtype).reshape(B, N, D, 2)
+        assert table.dtype == torch.float32
+        # x * cos + rotate(x) * sin with the table's values, rounded where torch rounds
+        cos, sin = table[..., 0].to(dtype)[:, None], table[..., 1].to(dtype)[:, None]
+        rot = torch.cat((-x[..., 16:32], x[..., :16], -x[..., 48:], x[..., 32:48]), -1)
+        assert torch.equal(x * cos + rot * sin, rope(x, pos))

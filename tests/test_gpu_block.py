@@ -85,3 +85,39 @@ def test_two_streams_through_one_block():
             for s in range(2):
                 ys = mod(x[s:s + 1], kv_cache=single[s], global_idx=0, num_frames=1)
                 assert (y[s:s + 1].float() - ys.float()).abs().max().item() <= 1e-2
+
+
+@pytest.mark.parametrize("rope", ["none", "2d", "interleaved"])
+def test_frame_block_without_cache_matches_torch_path(rope):
+    """Cache-less frames (the aggregator's frame blocks): fused producer + paged kernel over a
+    trivial row table against the same module's torch operations and SDPA in fp32."""
+    import torch.nn.functional as F
+    from lingbot_map_amd import HipPagedBlock, RotaryPositionEmbedding2D, dense_attention
+    torch.manual_seed(8)
+    dev = torch.device("cuda:0")
+    dim, H, T, B = 256, 4, 333, 3
+    mod = HipPagedBlock(dim, H, init_values=0.1, qk_norm=True,
+                        rope={"none": None, "2d": RotaryPositionEmbedding2D(), "interleaved": True}[rope]).to(dev, torch.bfloat16).eval()
+    for ln in (mod.attn.q_norm, mod.attn.k_norm):
+        ln.weight.data.uniform_(0.5, 1.5)
+        ln.bias.data.uniform_(-0.2, 0.2)
+    x = torch.randn(B, T, dim, device=dev).to(torch.bfloat16)
+    pos, e3 = None, False
+    if rope == "2d":
+        pos = torch.stack([torch.randint(0, 20, (1, T), device=dev), torch.randint(0, 20, (1, T), device=dev)], -1).expand(B, -1, -1).contiguous()
+    if rope == "interleaved":
+        ang = torch.rand(1, 1, T, 32, device=dev) * 6.283185
+        pos, e3 = torch.polar(torch.ones_like(ang), ang), True
+    with torch.no_grad():
+        assert mod.attn.can_fuse_dense(mod.norm1(x), pos, e3)
+        y = mod(x, pos=pos, enable_3d_rope=e3)
+        q, k, v = mod.attn._qkv(mod.norm1(x), pos, e3)
+        a = F.scaled_dot_product_attention(q.float(), k.float(), v.float()).transpose(1, 2).reshape(B, T, dim).to(torch.bfloat16)
+        y_ref = mod.ffn_residual(x + mod.ls1(mod.attn.proj(a)))
+        # the kernel alone, three independent groups in one launch
+        nhd = lambda t: t.permute(0, 2, 1, 3).reshape(B * T, H, 64).contiguous()
+        o = dense_attention(nhd(q), nhd(k), nhd(v), num_streams=B).reshape(B, T, dim)
+    err = (o.float() - a.float()).abs()
+    assert err.max().item() <= 2e-2 and err.mean().item() <= 2e-3
+    err = (y.float() - y_ref.float()).abs()
+    assert err.max().item() <= 3e-2 and err.mean().item() <= 2e-3

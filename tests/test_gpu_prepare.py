@@ -34,7 +34,9 @@ def _inputs(n, H, D, dtype, seed):
     return qkv, (w[0], b[0]), (w[1], b[1]), freqs
 
 
-def run_prepare(qkv, H, D, qn, kn, freqs, dst_dtype, pool=None, rows=None, page_size=16, want_kv=True, eps=1e-5):
+def run_prepare(qkv, H, D, qn, kn, freqs, dst_dtype, pool=None, rows=None, page_size=16, want_kv=True, eps=1e-5,
+                table=None):
+    """freqs: complex table of the interleaved embedding; table: [n, D, 2] (cos, sin) of the half-split one."""
     N = _native()
     dev = torch.device("cuda:0")
     n = qkv.shape[0]
@@ -42,11 +44,14 @@ def run_prepare(qkv, H, D, qn, kn, freqs, dst_dtype, pool=None, rows=None, page_
     f32 = lambda t: t.float().to(dev).contiguous()
     keep = [f32(t) for t in (qn or ()) + (kn or ())]
     cs = torch.view_as_real(freqs).reshape(n, D // 2, 2).float().contiguous().to(dev) if freqs is not None else None
+    layout = N.ROPE_INTERLEAVED
+    if table is not None:
+        cs, layout = table.float().contiguous().to(dev), N.ROPE_HALF_SPLIT
     q = torch.full((n, H, D), float("nan"), dtype=dst_dtype, device=dev)
     k = torch.full_like(q, float("nan")) if want_kv else None
     v = torch.full_like(q, float("nan")) if want_kv else None
     x = qkv.to(dev)
-    N.check(N.lib.lbm_qkv_prepare(ptr(x), dt(qkv.dtype), *( [ptr(t) for t in keep] if keep else [None] * 4), eps, ptr(cs),
+    N.check(N.lib.lbm_qkv_prepare(ptr(x), dt(qkv.dtype), *( [ptr(t) for t in keep] if keep else [None] * 4), eps, ptr(cs), layout,
                                   ptr(q), ptr(k), ptr(v), dt(dst_dtype), ptr(pool), ptr(rows), n, H, D, page_size, None))
     torch.cuda.synchronize()
     return q, k, v
@@ -121,12 +126,12 @@ def test_prepare_argument_checks():
     dev = torch.device("cuda:0")
     x = torch.zeros(4, 3 * 2 * 64, dtype=torch.bfloat16, device=dev)
     q = torch.zeros(4, 2, 64, dtype=torch.bfloat16, device=dev)
-    call = lambda **kw: N.lib.lbm_qkv_prepare(ptr(x), 0, None, None, None, None, 1e-5, None, ptr(q), None, None, 0, None, None,
+    call = lambda **kw: N.lib.lbm_qkv_prepare(ptr(x), 0, None, None, None, None, 1e-5, None, 0, ptr(q), None, None, 0, None, None,
                                               4, 2, kw.get("D", 64), 16, None)
     assert call() == N.OK
     assert call(D=128) != N.OK and b"head_dim 64" in N.lib.lbm_last_error()
     w = torch.ones(64, device=dev)
-    rc = N.lib.lbm_qkv_prepare(ptr(x), 0, ptr(w), None, None, None, 1e-5, None, ptr(q), None, None, 0, None, None, 4, 2, 64, 16, None)
+    rc = N.lib.lbm_qkv_prepare(ptr(x), 0, ptr(w), None, None, None, 1e-5, None, 0, ptr(q), None, None, 0, None, None, 4, 2, 64, 16, None)
     assert rc != N.OK
     torch.cuda.synchronize()
 
@@ -157,3 +162,24 @@ def test_manager_step_qkv_equals_step():
     pa, pb = a.kv_caches[1].float(), b.kv_caches[1].float()
     assert ((pa - pb).abs() / pa.abs().clamp_min(1.0)).max().item() <= 2 ** -7
     assert a.device_header()["error"] == 0 and b.device_header()["error"] == 0
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_prepare_half_split_rope_matches_oracle(dtype):
+    """The 2-D embedding of the frame blocks: pairs (j, j + 16) in each half of head_dim."""
+    from lingbot_map_amd import RotaryPositionEmbedding2D
+    from oracle.prepare_qkv import prepare_qkv
+    n, H, D = 300, 4, 64
+    qkv, qn, kn, _ = _inputs(n, H, D, dtype, seed=31)
+    g = torch.Generator().manual_seed(32)
+    pos = torch.stack([torch.randint(0, 27, (n,), generator=g), torch.randint(0, 37, (n,), generator=g)], -1)
+    rq, rk, rv = prepare_qkv(qkv, H, D, qn, kn, None, positions=pos)
+    table = RotaryPositionEmbedding2D().cos_sin_table(pos[None], D, dtype)
+    q, k, v = run_prepare(qkv, H, D, qn, kn, None, dtype, table=table)
+    assert torch.equal(v.cpu(), rv)
+    _close(q, rq, dtype)
+    _close(k, rk, dtype)
+    if dtype == torch.bfloat16:     # without LayerNorm: the reference's own roundings, bit for bit
+        rq, rk, _ = prepare_qkv(qkv, H, D, None, None, None, positions=pos)
+        q, k, _ = run_prepare(qkv, H, D, None, None, None, dtype, table=table)
+        assert torch.equal(q.cpu(), rq) and torch.equal(k.cpu(), rk)

@@ -3,7 +3,7 @@ import math
 
 import torch
 
-from oracle.prepare_qkv import apply_rotary_emb, prepare_qkv
+from oracle.prepare_qkv import apply_rotary_emb, prepare_qkv, rope2d
 
 
 def _freqs(n, d, seed=0, angle=None):
@@ -77,3 +77,31 @@ def test_bf16_rounds_where_the_reference_rounds():
     assert q16.dtype == torch.bfloat16
     err = (q16.float() - q32).abs() / q32.abs().clamp_min(1.0)
     assert 0 < err.max().item() < 4 * 2 ** -8
+
+
+def test_rope2d_identity_explicit_rotation_and_separation():
+    g = torch.Generator().manual_seed(8)
+    B, H, N, D = 1, 2, 12, 64
+    x = torch.randn(B, H, N, D, generator=g, dtype=torch.float64)
+    zero = torch.zeros(B, N, 2, dtype=torch.long)
+    assert torch.equal(rope2d(x, zero), x)
+    pos = torch.stack([torch.randint(0, N, (N,), generator=g), torch.randint(0, N, (N,), generator=g)], -1)[None]
+    y = rope2d(x, pos)
+    want = torch.empty_like(x)
+    for n in range(N):
+        for half in range(2):                      # 0: vertical (y), 1: horizontal (x)
+            p = float(pos[0, n, half])
+            for j in range(16):
+                ang = p * 100.0 ** (-(2 * j) / 32)
+                a, b = x[0, :, n, half * 32 + j], x[0, :, n, half * 32 + j + 16]
+                want[0, :, n, half * 32 + j] = a * math.cos(ang) - b * math.sin(ang)
+                want[0, :, n, half * 32 + j + 16] = b * math.cos(ang) + a * math.sin(ang)
+    # the table's angles go through float32 (inv_freq is computed in float32)
+    assert (y - want).abs().max().item() < 1e-5
+    pair = lambda t: torch.stack([t[..., :16], t[..., 16:32], t[..., 32:48], t[..., 48:]], -1)
+    n_in = (pair(x)[..., 0] ** 2 + pair(x)[..., 1] ** 2).sqrt()
+    n_out = (pair(y)[..., 0] ** 2 + pair(y)[..., 1] ** 2).sqrt()
+    assert (n_in - n_out).abs().max().item() < 1e-6
+    only_y = pos.clone(); only_y[..., 1] = 0
+    assert torch.equal(rope2d(x, only_y)[..., :32], y[..., :32])
+    assert torch.equal(rope2d(x, only_y)[..., 32:], x[..., 32:])
