@@ -8,7 +8,8 @@ if it has not been built: there is no CPU path.
 from . import _native  # noqa: F401  (loads the library, fails loudly when missing)
 from .block import HipPagedAttention, HipPagedBlock, RotaryPositionEmbedding2D, keyframe_flags, set_skip_append
 from .dense import dense_attention
+from .graph import GraphedFrame
 from .manager import HipPagedKVCacheManager
 
 __all__ = ["HipPagedKVCacheManager", "HipPagedAttention", "HipPagedBlock", "RotaryPositionEmbedding2D",
-           "dense_attention", "keyframe_flags", "set_skip_append"]
+           "dense_attention", "GraphedFrame", "keyframe_flags", "set_skip_append"]

@@ -453,6 +453,41 @@ class HipPagedKVCacheManager:
         return t if (t.dtype == torch.float32 and t.is_contiguous() and t.device == self.device) else \
             t.detach().to(device=self.device, dtype=torch.float32).contiguous()
 
+    def steady_state(self, cross_frame_special: bool = True, camera_only: bool = False) -> bool:
+        """True when one more keyframe step of every active stream would launch exactly what
+        the last one launched: same table operations, same visible token counts, same attention
+        schedule.  That holds once anchor and window are full and evicted frames leave no
+        memory tokens behind; it is the condition under which a captured HIP graph of a frame
+        may be replayed (the page ids live on the device and keep evolving across replays)."""
+        if self._skip_append or self._defer_eviction or not any(self._active):
+            return False
+        keep = self._keep_tokens(cross_frame_special, camera_only)
+        for ts in range(self._n_sets):
+            for b in range(self.num_streams):
+                if not self._active[b]:
+                    continue
+                c = self._counts[ts][b]
+                probe = _StreamCounts(0, 0)
+                for f in _StreamCounts.__slots__:
+                    setattr(probe, f, getattr(c, f))
+                before = self._visible_tokens(c)
+                self._mirror_append(probe, 0)
+                self._mirror_evict(probe, self._windows[b], keep, 0)
+                same = all(getattr(probe, f) == getattr(c, f) for f in _StreamCounts.__slots__ if f != "frame_count")
+                if not same or self._visible_tokens(probe) != before or not self._plan_valid[ts]:
+                    return False
+        return True
+
+    def note_replayed_frames(self, n: int = 1) -> None:
+        """Book-keeping after replaying a captured steady-state frame ``n`` times: the device
+        tables advanced, the host's frame counters follow."""
+        for i in range(self.num_blocks):
+            self.frame_count[i] += n
+        for ts in range(self._n_sets):
+            for b in range(self.num_streams):
+                if self._active[b]:
+                    self._counts[ts][b].frame_count += n
+
     def _step_tables(self, block_idx: int, keyframe: Optional[Sequence[bool]], cross_frame_special: bool,
                      camera_only: bool):
         """Table work of one streamed frame (allocate, evict, visible rows; one launch on the
