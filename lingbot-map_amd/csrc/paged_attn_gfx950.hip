@@ -60,7 +60,6 @@ constexpr int kStages = 3;              // LDS ring depth
 constexpr int kKStride = 72;            // bf16 per LDS row of K: 144 B, b128 reads hit 64 distinct banks
 constexpr int kVStride = 96;            // bf16 per LDS row of V: 192 B, 4-row transpose reads conflict-free
 constexpr float kHeadroom = 11.0f;      // the softmax reference is set this far above the row maxima (log2 units)
-constexpr int kTargetWgs = 256;         // one 8-wave workgroup per CU
 
 struct AttnArgs {
   const unsigned short* q;
@@ -705,36 +704,133 @@ __global__ __launch_bounds__(256) void lbm_attn_f32_d64_kernel(AttnArgsF32 a) {
 }
 
 // ---------------------------------------------------------------------------- schedule
+// How many KV splits each stream gets.  All workgroups of one launch compete for the 256 CUs
+// (one 8-wave workgroup per CU at a time, handed out in blockIdx order), so the choice is a
+// small scheduling problem: few long workgroups leave CUs idle at the end, many short ones
+// pay the per-workgroup prologue/epilogue and more split-KV partials.  A handful of candidate
+// tile counts per workgroup is priced with the measured costs below by simulating the
+// hand-out (streams with the longest workgroups first), and the cheapest wins.  The result
+// depends on row and tile counts only and is remembered for the next call with the same ones
+// (every block of a frame asks for the same schedule).
+namespace {
+constexpr double kTileUs = 1.95;      // one 64-token tile iteration of a workgroup
+constexpr double kWgTiles = 3.0;      // prologue + epilogue of a workgroup, in tile iterations
+constexpr double kCombineUs = 2.5;    // launch + latency of the combine kernel
+constexpr double kCombineBytesPerUs = 5.0e6;
+
+struct ScheduleKey {
+  int n_streams = -1, num_heads = 0;
+  int q_rows[LBM_MAX_STREAMS], n_tiles[LBM_MAX_STREAMS];
+  int order[LBM_MAX_STREAMS], n_splits[LBM_MAX_STREAMS];
+};
+thread_local ScheduleKey g_last_schedule;
+
+double price_candidate(const int* qt, const int* nt, int n_streams, int num_heads, int tps, const int* q_rows,
+                       int* n_splits_out) {
+  // streams sorted by tiles per workgroup, longest first
+  int tiles[LBM_MAX_STREAMS], order[LBM_MAX_STREAMS];
+  double part_bytes = 0;
+  for (int i = 0; i < n_streams; ++i) {
+    int ns = nt[i] > 0 ? (nt[i] + tps - 1) / tps : 1;
+    if (ns > 64) ns = 64;
+    if (ns < 1) ns = 1;
+    tiles[i] = nt[i] > 0 ? (nt[i] + ns - 1) / ns : 0;
+    n_splits_out[i] = nt[i] > 0 ? (nt[i] + tiles[i] - 1) / tiles[i] : 1;
+    if (n_splits_out[i] > 1) part_bytes += (double)n_splits_out[i] * q_rows[i] * num_heads * (64 * 2 + 4);
+    order[i] = i;
+  }
+  for (int i = 1; i < n_streams; ++i)
+    for (int j = i; j > 0 && tiles[order[j]] > tiles[order[j - 1]]; --j) { int t = order[j]; order[j] = order[j - 1]; order[j - 1] = t; }
+  // hand the workgroups out to the CUs in order; each goes to the CU that frees up first.  A
+  // binary heap over 256 finish times.
+  double heap[256];
+  for (int i = 0; i < 256; ++i) heap[i] = 0.0;
+  double makespan = 0.0;
+  for (int oi = 0; oi < n_streams; ++oi) {
+    const int i = order[oi];
+    const long long wgs = (long long)qt[i] * num_heads * n_splits_out[i];
+    const double dur = kWgTiles + tiles[i];
+    for (long long w = 0; w < wgs; ++w) {
+      const double t = heap[0] + dur;
+      if (t > makespan) makespan = t;
+      // replace the root and sift down
+      int k = 0;
+      for (;;) {
+        int c = 2 * k + 1;
+        if (c >= 256) break;
+        if (c + 1 < 256 && heap[c + 1] < heap[c]) ++c;
+        if (heap[c] >= t) break;
+        heap[k] = heap[c];
+        k = c;
+      }
+      heap[k] = t;
+    }
+  }
+  return makespan * kTileUs + (part_bytes > 0 ? kCombineUs + 2.0 * part_bytes / kCombineBytesPerUs : 0.0);
+}
+}  // namespace
+
 void lbm_attn_schedule(const lbm_attn_stream* streams, int n_streams, int num_heads,
                        LbmAttnSchedule* out) {
-  // Aim at one 8-wave workgroup on each of the 256 CUs, all with about the same number of tiles.
-  const long long target_wgs = kTargetWgs;
   LbmAttnSchedule& sch = *out;
   sch = LbmAttnSchedule{};
   sch.n_streams = n_streams;
+  int qt[LBM_MAX_STREAMS], nt[LBM_MAX_STREAMS], q_rows[LBM_MAX_STREAMS];
   long long work = 0;
+  int max_nt = 0;
   for (int i = 0; i < n_streams; ++i) {
-    const long long qt = (streams[i].q_rows + kQTile - 1) / kQTile;
-    const long long nt = (streams[i].kv_tokens + kKvTile - 1) / kKvTile;
-    work += qt * num_heads * nt;
+    q_rows[i] = streams[i].q_rows;
+    qt[i] = (streams[i].q_rows + kQTile - 1) / kQTile;
+    nt[i] = (streams[i].kv_tokens + kKvTile - 1) / kKvTile;
+    work += (long long)qt[i] * num_heads * nt[i];
+    if (nt[i] > max_nt) max_nt = nt[i];
   }
-  long long tps_target = (work + target_wgs - 1) / target_wgs;
-  if (tps_target < 4) tps_target = 4;
+  ScheduleKey& memo = g_last_schedule;
+  bool hit = memo.n_streams == n_streams && memo.num_heads == num_heads;
+  for (int i = 0; hit && i < n_streams; ++i) hit = memo.q_rows[i] == q_rows[i] && memo.n_tiles[i] == nt[i];
+  if (!hit) {
+    int best_splits[LBM_MAX_STREAMS], cand_splits[LBM_MAX_STREAMS];
+    double best = -1.0;
+    auto consider = [&](long long tps) {
+      if (tps < 2) tps = 2;
+      if (tps > max_nt) tps = max_nt > 0 ? max_nt : 1;
+      const double c = price_candidate(qt, nt, n_streams, num_heads, (int)tps, q_rows, cand_splits);
+      if (best < 0 || c < best) {
+        best = c;
+        for (int i = 0; i < n_streams; ++i) best_splits[i] = cand_splits[i];
+      }
+    };
+    // the longest stream cut into 1..12 pieces, and the total work spread over 1..3 rounds of 256
+    for (int k = 1; k <= 12; ++k) consider((max_nt + k - 1) / k);
+    for (int k = 1; k <= 3; ++k) consider((work + 256LL * k - 1) / (256LL * k));
+    memo.n_streams = n_streams;
+    memo.num_heads = num_heads;
+    int tiles[LBM_MAX_STREAMS];
+    for (int i = 0; i < n_streams; ++i) {
+      memo.q_rows[i] = q_rows[i];
+      memo.n_tiles[i] = nt[i];
+      memo.n_splits[i] = best_splits[i];
+      memo.order[i] = i;
+      tiles[i] = nt[i] > 0 ? (nt[i] + best_splits[i] - 1) / best_splits[i] : 0;
+    }
+    for (int i = 1; i < n_streams; ++i)
+      for (int j = i; j > 0 && tiles[memo.order[j]] > tiles[memo.order[j - 1]]; --j) {
+        int t = memo.order[j]; memo.order[j] = memo.order[j - 1]; memo.order[j - 1] = t;
+      }
+  }
   int wg = 0;
   long long part = 0;
-  for (int i = 0; i < n_streams; ++i) {
-    LbmAttnStreamPlan& p = sch.s[i];
+  for (int oi = 0; oi < n_streams; ++oi) {
+    const int i = memo.order[oi];
+    LbmAttnStreamPlan& p = sch.s[oi];   // plans in launch order: blockIdx ranges ascend with the index
     p.q_begin = streams[i].q_begin;
     p.q_rows = streams[i].q_rows;
     p.kv_row_begin = streams[i].kv_row_begin;
     p.kv_tokens = streams[i].kv_tokens;
-    p.n_qtiles = (p.q_rows + kQTile - 1) / kQTile;
-    const int nt = (p.kv_tokens + kKvTile - 1) / kKvTile;
-    int ns = (int)((nt + tps_target - 1) / tps_target);
-    if (ns < 1) ns = 1;
-    if (ns > 64) ns = 64;
-    p.tiles_per_split = nt > 0 ? (nt + ns - 1) / ns : 1;
-    p.n_splits = nt > 0 ? (nt + p.tiles_per_split - 1) / p.tiles_per_split : 1;
+    p.n_qtiles = qt[i];
+    const int ns = memo.n_splits[i];
+    p.tiles_per_split = nt[i] > 0 ? (nt[i] + ns - 1) / ns : 1;
+    p.n_splits = nt[i] > 0 ? (nt[i] + p.tiles_per_split - 1) / p.tiles_per_split : 1;
     // keep each stream's first workgroup on XCD 0 so the in-kernel XCD mapping lines up
     wg = (wg + 7) & ~7;
     p.wg_begin = wg;
