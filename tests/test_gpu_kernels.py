@@ -204,6 +204,49 @@ def test_attention_closed_forms():
     assert (out.float() - mean).abs().max().item() <= 1e-2
 
 
+def test_attention_edge_shapes():
+    """Empty and ragged extremes through the C ABI: a stream with nothing visible gets zeros (the
+    reference returns zeros before the first append, flashinfer_cache.py:368-370) next to streams
+    that do attend; a stream without query rows; sixteen streams (the maximum) of 1..16 tokens."""
+    from oracle.sdpa_cache import sdpa_nhd
+    dev = torch.device("cuda:0")
+    g = torch.Generator().manual_seed(41)
+    H, D, S = 2, 64, 16
+    n_pages = 16
+    pool = torch.randn(n_pages, 2, S, H, D, generator=g).to(torch.bfloat16)
+    flat_k = pool[:, 0].reshape(-1, H, D)
+    flat_v = pool[:, 1].reshape(-1, H, D)
+    slot_row = lambda s: (s // S) * 2 * S + s % S
+    # three streams: 5 queries x 0 tokens, 7 queries x 20 tokens, 0 queries x 9 tokens
+    q = torch.randn(12, H, D, generator=g).to(torch.bfloat16)
+    slots = torch.randperm(n_pages * S, generator=g)[:29]
+    rows = torch.tensor([slot_row(int(x)) for x in slots], dtype=torch.int32)
+    out = run_attention(q.to(dev), pool.to(dev), rows.to(dev), [(0, 5, 0, 0), (5, 7, 0, 20), (12, 0, 20, 9)], S).cpu()
+    assert torch.equal(out[:5], torch.zeros(5, H, D, dtype=torch.bfloat16))
+    check_bf16(out[5:], sdpa_nhd(q[5:], flat_k[slots[:20]], flat_v[slots[:20]]))
+    # sixteen streams, stream i has i + 1 query rows and i + 1 visible tokens
+    n = sum(range(1, 17))
+    q = torch.randn(n, H, D, generator=g).to(torch.bfloat16)
+    assert n <= n_pages * S
+    slots = torch.randperm(n_pages * S, generator=g)[:n]
+    rows = torch.tensor([slot_row(int(x)) for x in slots], dtype=torch.int32)
+    assert rows.numel() == n          # the row table covers every token the streams name
+    streams, off = [], 0
+    for i in range(16):
+        streams.append((off, i + 1, off, i + 1))
+        off += i + 1
+    out = run_attention(q.to(dev), pool.to(dev), rows.to(dev), streams, S).cpu()
+    for (b, nq, kb, nk) in streams:
+        check_bf16(out[b:b + nq], sdpa_nhd(q[b:b + nq], flat_k[slots[kb:kb + nk]], flat_v[slots[kb:kb + nk]]))
+    # a seventeenth stream is refused, nothing is launched
+    N = _native()
+    arr = (N.AttnStream * 17)(*[N.AttnStream(0, 1, 0, 1) for _ in range(17)])
+    assert N.lib.lbm_attn_workspace_bytes(arr, 17, H, D) == 0
+    rc = N.lib.lbm_attn_run(ptr(q.to(dev)), ptr(pool.to(dev)), ptr(out.to(dev)), None, None, ptr(rows.to(dev)), arr, 17,
+                            H, D, S, N.DTYPE_BF16, 0.125, None, 0, None)
+    assert rc != N.OK and b"n_streams" in N.lib.lbm_last_error()
+
+
 @pytest.mark.parametrize("src,dst", [(torch.bfloat16, torch.bfloat16), (torch.float32, torch.bfloat16),
                                      (torch.float32, torch.float32), (torch.bfloat16, torch.float32)])
 def test_append_is_exact_and_gated(src, dst):
