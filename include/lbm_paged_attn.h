@@ -188,7 +188,14 @@ size_t lbm_attn_workspace_bytes(const lbm_attn_stream* streams, int32_t n_stream
  * gather + F.scaled_dot_product_attention bridge (:324-347, :372-383).
  *   q, out         [rows][num_heads][head_dim], dtype = pool dtype
  *   self_k, self_v the caller's K/V of the current frames, same indexing as q (only read
- *                  for negative kv_rows entries; may be NULL otherwise) */
+ *                  for negative kv_rows entries; may be NULL otherwise)
+ *   kv_rows        device array; stream i reads entries kv_row_begin .. kv_row_begin + kv_tokens - 1,
+ *                  each a K row of the pool (page * 2 * page_size + slot) or -1 - r for row r of
+ *                  self_k / self_v.  The entries are trusted: the library cannot see the sizes of
+ *                  the pool or of this array, so a table that is too short or names rows outside
+ *                  the pool makes the kernel read out of bounds.  Tables written by
+ *                  lbm_tables_step / lbm_rows_from_pages satisfy this by construction.
+ *   A stream with kv_tokens == 0 gets zeros; a stream with q_rows == 0 launches nothing. */
 int lbm_attn_run(const void* q, const void* pool, void* out, const void* self_k,
                  const void* self_v, const int32_t* kv_rows, const lbm_attn_stream* streams,
                  int32_t n_streams, int32_t num_heads, int32_t head_dim, int32_t page_size,
