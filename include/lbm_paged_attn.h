@@ -99,7 +99,11 @@ typedef struct lbm_step_op {
                                caller's tensors, never stored) after the cached tokens     */
   int32_t q_begin;          /* first row of this stream in the batched q/k/v tensors       */
   int32_t kv_row_begin;     /* PLAN: first entry of this stream in kv_rows                 */
-  int32_t expect_kv_tokens; /* PLAN: the host's count of visible tokens                    */
+  int32_t expect_kv_tokens; /* PLAN: >= 0: the host's count of visible tokens (a mismatch sets
+                               LBM_TERR_KV_COUNT); < 0: the host does not track the count and
+                               -expect_kv_tokens is the capacity of this stream's part of
+                               kv_rows (more visible tokens than that set the error bit and
+                               the count is clamped)                                        */
   int32_t page_out_begin;   /* PLAN: first entry of this stream in kv_page_ids/_lens       */
 } lbm_step_op;
 
@@ -109,6 +113,8 @@ typedef struct lbm_attn_stream {
   int32_t q_rows;       /* number of query rows                                            */
   int32_t kv_row_begin; /* first entry in kv_rows                                          */
   int32_t kv_tokens;    /* number of entries                                               */
+  int32_t live_at;      /* lbm_attn_run_live only: index of this stream's token count in
+                           live_kv_tokens                                                  */
 } lbm_attn_stream;
 
 int lbm_abi_version(void);
@@ -151,6 +157,19 @@ int lbm_rows_from_pages(const int32_t* kv_page_ids, const int32_t* kv_page_lens,
 int lbm_kv_append(const void* k, const void* v, int32_t src_dtype, void* pool,
                   int32_t pool_dtype, const int32_t* append_rows, int32_t n_tokens,
                   int32_t num_heads, int32_t head_dim, int32_t page_size, void* stream);
+
+/* lbm_attn_run with the token counts read on the device: stream i attends to
+ * live_kv_tokens[streams[i].live_at] entries of its row table instead of streams[i].kv_tokens,
+ * which then only sizes the launch (number of KV splits, workspace) and should be the host's
+ * best knowledge of the count.  Every argument of the call is then the same from frame to frame
+ * while the cache grows, so the call can sit in a captured HIP graph; lbm_tables_step with a
+ * negative expect_kv_tokens maintains the count (header word LBM_HDR_PLAN_KV_TOKENS).  No
+ * counterpart in the reference, whose plan lives on the host (flashinfer_cache.py:385-414). */
+int lbm_attn_run_live(const void* q, const void* pool, void* out, const void* self_k,
+                      const void* self_v, const int32_t* kv_rows, const int32_t* live_kv_tokens,
+                      const lbm_attn_stream* streams, int32_t n_streams, int32_t num_heads,
+                      int32_t head_dim, int32_t page_size, int32_t dtype, float sm_scale,
+                      void* workspace, size_t workspace_bytes, void* stream);
 
 /* Fused pre-attention producer: per-head LayerNorm of q and k, rotary embedding of q and k
  * (interleaved pairs), [token][head][dim] layout and the keyframe-gated paged append of k and

@@ -47,7 +47,7 @@ int lbm_tables_step(int32_t* tables, const lbm_cache_geom* geom, int32_t n_strea
       return lbm_fail(LBM_ERR_INVALID, "lbm_tables_step: stream %d has unknown op bits 0x%x", i, o.ops);
     if ((o.ops & LBM_OP_PLAN) && !kv_rows && !(kv_page_ids && kv_page_lens))
       return lbm_fail(LBM_ERR_INVALID, "lbm_tables_step: PLAN needs kv_rows or the page table outputs");
-    if ((o.ops & LBM_OP_PLAN) && (o.expect_kv_tokens < 0 || o.kv_row_begin < 0 || o.page_out_begin < 0))
+    if ((o.ops & LBM_OP_PLAN) && (o.expect_kv_tokens == INT32_MIN || o.kv_row_begin < 0 || o.page_out_begin < 0))
       return lbm_fail(LBM_ERR_INVALID, "lbm_tables_step: stream %d has a negative plan offset or count", i);
     if ((o.ops & LBM_OP_EVICT) && o.sliding_window < 0)
       return lbm_fail(LBM_ERR_INVALID, "lbm_tables_step: stream %d has a negative sliding_window", i);
@@ -129,23 +129,46 @@ size_t lbm_attn_workspace_bytes(const lbm_attn_stream* streams, int32_t n_stream
   return lbm_attn_schedule_bytes(sch, num_heads, head_dim);
 }
 
+static int lbm_attn_run_impl(const char* who, const void* q, const void* pool, void* out, const void* self_k,
+                             const void* self_v, const int32_t* kv_rows, const int32_t* live_kv_tokens,
+                             const lbm_attn_stream* streams, int32_t n_streams, int32_t num_heads,
+                             int32_t head_dim, int32_t page_size, int32_t dtype, float sm_scale,
+                             void* workspace, size_t workspace_bytes, void* stream) {
+  int rc = lbm_check_attn_streams(streams, n_streams, who);
+  if (rc != LBM_OK) return rc;
+  if (!q || !pool || !out || !kv_rows) return lbm_fail(LBM_ERR_INVALID, "%s: null q, pool, out or kv_rows", who);
+  if (num_heads <= 0 || head_dim <= 0 || page_size <= 0) return lbm_fail(LBM_ERR_INVALID, "%s: non-positive size", who);
+  if ((self_k == nullptr) != (self_v == nullptr)) return lbm_fail(LBM_ERR_INVALID, "%s: self_k and self_v go together", who);
+  if (live_kv_tokens)
+    for (int i = 0; i < n_streams; ++i)
+      if (streams[i].live_at < 0) return lbm_fail(LBM_ERR_INVALID, "%s: stream %d has a negative live_at", who, i);
+  LbmAttnSchedule sch;
+  lbm_attn_schedule(streams, n_streams, num_heads, &sch);
+  const size_t need = lbm_attn_schedule_bytes(sch, num_heads, head_dim);
+  if (need > 0 && (!workspace || workspace_bytes < need))
+    return lbm_fail(LBM_ERR_WORKSPACE, "%s: workspace of %zu bytes, %zu needed", who, workspace_bytes, need);
+  return lbm_launch_attention(q, pool, out, self_k, self_v, kv_rows, live_kv_tokens, sch, num_heads, head_dim,
+                              page_size, dtype, sm_scale, workspace, (hipStream_t)stream);
+}
+
 int lbm_attn_run(const void* q, const void* pool, void* out, const void* self_k,
                  const void* self_v, const int32_t* kv_rows, const lbm_attn_stream* streams,
                  int32_t n_streams, int32_t num_heads, int32_t head_dim, int32_t page_size,
                  int32_t dtype, float sm_scale, void* workspace, size_t workspace_bytes,
                  void* stream) {
-  int rc = lbm_check_attn_streams(streams, n_streams, "lbm_attn_run");
-  if (rc != LBM_OK) return rc;
-  if (!q || !pool || !out || !kv_rows) return lbm_fail(LBM_ERR_INVALID, "lbm_attn_run: null q, pool, out or kv_rows");
-  if (num_heads <= 0 || head_dim <= 0 || page_size <= 0) return lbm_fail(LBM_ERR_INVALID, "lbm_attn_run: non-positive size");
-  if ((self_k == nullptr) != (self_v == nullptr)) return lbm_fail(LBM_ERR_INVALID, "lbm_attn_run: self_k and self_v go together");
-  LbmAttnSchedule sch;
-  lbm_attn_schedule(streams, n_streams, num_heads, &sch);
-  const size_t need = lbm_attn_schedule_bytes(sch, num_heads, head_dim);
-  if (need > 0 && (!workspace || workspace_bytes < need))
-    return lbm_fail(LBM_ERR_WORKSPACE, "lbm_attn_run: workspace of %zu bytes, %zu needed", workspace_bytes, need);
-  return lbm_launch_attention(q, pool, out, self_k, self_v, kv_rows, sch, num_heads, head_dim,
-                              page_size, dtype, sm_scale, workspace, (hipStream_t)stream);
+  return lbm_attn_run_impl("lbm_attn_run", q, pool, out, self_k, self_v, kv_rows, nullptr, streams, n_streams,
+                           num_heads, head_dim, page_size, dtype, sm_scale, workspace, workspace_bytes, stream);
+}
+
+int lbm_attn_run_live(const void* q, const void* pool, void* out, const void* self_k,
+                      const void* self_v, const int32_t* kv_rows, const int32_t* live_kv_tokens,
+                      const lbm_attn_stream* streams, int32_t n_streams, int32_t num_heads,
+                      int32_t head_dim, int32_t page_size, int32_t dtype, float sm_scale,
+                      void* workspace, size_t workspace_bytes, void* stream) {
+  if (!live_kv_tokens) return lbm_fail(LBM_ERR_INVALID, "lbm_attn_run_live: null live_kv_tokens");
+  return lbm_attn_run_impl("lbm_attn_run_live", q, pool, out, self_k, self_v, kv_rows, live_kv_tokens, streams,
+                           n_streams, num_heads, head_dim, page_size, dtype, sm_scale, workspace, workspace_bytes,
+                           stream);
 }
 
 }  // extern "C"

@@ -31,7 +31,7 @@ int lbm_launch_qkv_prepare(const void* qkv, int src_dtype, const float* q_norm_w
 
 // Split-KV schedule of one attention call, computed on the host from token counts only.
 struct LbmAttnStreamPlan {
-  int32_t q_begin, q_rows, kv_row_begin, kv_tokens;
+  int32_t q_begin, q_rows, kv_row_begin, kv_tokens, live_at;
   int32_t n_qtiles, n_splits, tiles_per_split;
   int32_t wg_begin;    // first workgroup of this stream
   int32_t part_begin;  // first partial-result row (unit: q row of one split) in the workspace
@@ -47,7 +47,8 @@ void lbm_attn_schedule(const lbm_attn_stream* streams, int n_streams, int num_he
 size_t lbm_attn_schedule_bytes(const LbmAttnSchedule& sch, int num_heads, int head_dim);
 
 int lbm_launch_attention(const void* q, const void* pool, void* out, const void* self_k,
-                         const void* self_v, const int32_t* kv_rows, const LbmAttnSchedule& sch,
+                         const void* self_v, const int32_t* kv_rows, const int32_t* live_kv_tokens,
+                         const LbmAttnSchedule& sch,
                          int num_heads, int head_dim, int page_size, int dtype, float sm_scale,
                          void* workspace, hipStream_t stream);
 

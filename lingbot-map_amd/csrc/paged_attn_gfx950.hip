@@ -68,6 +68,7 @@ struct AttnArgs {
   const unsigned short* self_k;
   const unsigned short* self_v;
   const int32_t* kv_rows;
+  const int32_t* live_kv_tokens;  // device-side token counts (NULL: the host's counts in the plan)
   unsigned short* part_o;  // split-KV partial outputs, normalised, bf16
   float* part_lse;
   int num_heads;
@@ -126,7 +127,10 @@ __global__ __launch_bounds__(kThreads, 1) void lbm_attn_bf16_d64_kernel(AttnArgs
   }
   if (local >= sp.n_qtiles * n_hs) return;  // padding between streams
   const int head = hs % H, split = hs / H;
-  if (sp.kv_tokens <= 0) {
+  // With device-side token counts the split count stays the host's choice (it fixes the grid
+  // and the workspace layout) and the tiles are dealt to the splits from the live count.
+  const int kv_tokens = a.live_kv_tokens ? a.live_kv_tokens[sp.live_at] : sp.kv_tokens;
+  if (kv_tokens <= 0 && sp.n_splits == 1) {
     // nothing visible: the reference returns zeros (lingbot_map/layers/flashinfer_cache.py:368-370)
     for (int k = 0; k < kQPerWave / 8; ++k) {
       const int r = qt * kQTile + wave * kQPerWave + k * 8 + (lane >> 3);
@@ -135,9 +139,10 @@ __global__ __launch_bounds__(kThreads, 1) void lbm_attn_bf16_d64_kernel(AttnArgs
     }
     return;
   }
-  const int n_tiles = (sp.kv_tokens + kKvTile - 1) / kKvTile;
-  const int t0 = split * sp.tiles_per_split;
-  const int t1 = min(t0 + sp.tiles_per_split, n_tiles);
+  const int n_tiles = (max(kv_tokens, 0) + kKvTile - 1) / kKvTile;
+  const int tiles_per_split = a.live_kv_tokens ? max((n_tiles + sp.n_splits - 1) / sp.n_splits, 1) : sp.tiles_per_split;
+  const int t0 = split * tiles_per_split;
+  const int t1 = min(t0 + tiles_per_split, n_tiles);  // an empty split (t1 <= t0) contributes weight 0
   const int n = t1 - t0;
   const unsigned row_bytes = (unsigned)H * 128u;
 
@@ -197,10 +202,10 @@ __global__ __launch_bounds__(kThreads, 1) void lbm_attn_bf16_d64_kernel(AttnArgs
   const char* own_k = (const char*)(a.self_k + (size_t)head * 64 + ld_c);
   const char* own_v = (const char*)(a.self_v + (size_t)head * 64 + ld_c);
   const int32_t* rows = a.kv_rows + sp.kv_row_begin;
-  const int last_token = sp.kv_tokens - 1;
+  const int last_token = max(kv_tokens - 1, 0);
   // Tiles past the end of this split re-read its last tile: the data lands in ring stages
   // nobody reads any more, and the code stays free of branches.
-  auto row_entry = [&](int t) -> int { return rows[min(min(t, t1 - 1) * kKvTile + ld_r, last_token)]; };
+  auto row_entry = [&](int t) -> int { return rows[min(max(min(t, t1 - 1), 0) * kKvTile + ld_r, last_token)]; };
   auto fetch = [&](int e, const char* pool_base, const char* own_base) -> u32x4 {
     // negative entries name rows of the caller's own K/V (read-only tail of a non-keyframe)
     const char* base = e < 0 ? own_base : pool_base;
@@ -425,7 +430,7 @@ __global__ __launch_bounds__(kThreads, 1) void lbm_attn_bf16_d64_kernel(AttnArgs
     for (int kk = 0; kk < 2; ++kk) pB[qb][kk] = __builtin_bit_cast(bf16x8, u32x4{0u, 0u, 0u, 0u});
   int ek = row_entry(t0 + 2), ev = row_entry(t0 + 1);
   __syncthreads();
-  qk_half(0, 0, sp.kv_tokens - t0 * kKvTile, sA);
+  qk_half(0, 0, kv_tokens - t0 * kKvTile, sA);
   {
     // the reference starts at the maxima of the first half
     float mx[2];
@@ -446,7 +451,7 @@ __global__ __launch_bounds__(kThreads, 1) void lbm_attn_bf16_d64_kernel(AttnArgs
     int st_k1 = st_k + 1; if (st_k1 >= kStages) st_k1 -= kStages;
     int st_k2 = st_k1 + 1; if (st_k2 >= kStages) st_k2 -= kStages;
     int st_v1 = st_v + 1; if (st_v1 >= kStages) st_v1 -= kStages;
-    const int n_valid = sp.kv_tokens - t * kKvTile;
+    const int n_valid = kv_tokens - t * kKvTile;
     bool hot;
 
     // global fetches of K(i+2), V(i+1) start here and land in the ring at the end of the step
@@ -552,6 +557,7 @@ __global__ __launch_bounds__(256) void lbm_attn_combine_bf16_kernel(AttnArgs a) 
 #pragma unroll
     for (int j = 0; j < 8; ++j) mx = fmaxf(mx, t[j]);
   }
+  if (mx == -INFINITY) mx = 0.f;  // every split empty (no visible token): weights 0, output 0
   float wsum = 0.f;
   f32x8 acc;
 #pragma unroll
@@ -575,7 +581,7 @@ __global__ __launch_bounds__(256) void lbm_attn_combine_bf16_kernel(AttnArgs a) 
       for (int e = 0; e < 8; ++e) acc[e] += w * vf[e];
     }
   }
-  const float inv = 1.0f / wsum;
+  const float inv = wsum > 0.f ? 1.0f / wsum : 0.f;
   const long long r = rh / H, h = rh % H;
   unsigned short* op = a.out + ((size_t)(sp.q_begin + r) * H + h) * 64 + d8 * 8;
 #pragma unroll
@@ -598,6 +604,7 @@ struct AttnArgsF32 {
   const float* self_k;
   const float* self_v;
   const int32_t* kv_rows;
+  const int32_t* live_kv_tokens;
   int num_heads;
   int page_size;
   float scale_log2;
@@ -614,7 +621,8 @@ __global__ __launch_bounds__(256) void lbm_attn_f32_d64_kernel(AttnArgsF32 a) {
   int b = 0;
   for (int i = 1; i < a.n_streams; ++i)
     if ((int)blockIdx.x >= a.wg_begin[i]) b = i;
-  const lbm_attn_stream sp = a.s[b];
+  lbm_attn_stream sp = a.s[b];
+  if (a.live_kv_tokens) sp.kv_tokens = max(a.live_kv_tokens[sp.live_at], 0);
   const int H = a.num_heads;
   const int local = (int)blockIdx.x - a.wg_begin[b];
   const int head = local % H, qt = local / H;
@@ -827,6 +835,7 @@ void lbm_attn_schedule(const lbm_attn_stream* streams, int n_streams, int num_he
     p.q_rows = streams[i].q_rows;
     p.kv_row_begin = streams[i].kv_row_begin;
     p.kv_tokens = streams[i].kv_tokens;
+    p.live_at = streams[i].live_at;
     p.n_qtiles = qt[i];
     const int ns = memo.n_splits[i];
     p.tiles_per_split = nt[i] > 0 ? (nt[i] + ns - 1) / ns : 1;
@@ -848,7 +857,8 @@ size_t lbm_attn_schedule_bytes(const LbmAttnSchedule& sch, int num_heads, int he
 }
 
 int lbm_launch_attention(const void* q, const void* pool, void* out, const void* self_k,
-                         const void* self_v, const int32_t* kv_rows, const LbmAttnSchedule& sch,
+                         const void* self_v, const int32_t* kv_rows, const int32_t* live_kv_tokens,
+                         const LbmAttnSchedule& sch,
                          int num_heads, int head_dim, int page_size, int dtype, float sm_scale,
                          void* workspace, hipStream_t stream) {
   if (head_dim != 64)
@@ -861,16 +871,17 @@ int lbm_launch_attention(const void* q, const void* pool, void* out, const void*
     f.self_k = (const float*)self_k;
     f.self_v = (const float*)self_v;
     f.kv_rows = kv_rows;
+    f.live_kv_tokens = live_kv_tokens;
     f.num_heads = num_heads;
     f.page_size = page_size;
     f.scale_log2 = sm_scale * 1.4426950408889634f;
     f.n_streams = sch.n_streams;
     int wg = 0;
     for (int i = 0; i < LBM_MAX_STREAMS; ++i) {
-      f.s[i] = lbm_attn_stream{0, 0, 0, 0};
+      f.s[i] = lbm_attn_stream{0, 0, 0, 0, 0};
       f.wg_begin[i] = wg;
       if (i < sch.n_streams) {
-        f.s[i] = lbm_attn_stream{sch.s[i].q_begin, sch.s[i].q_rows, sch.s[i].kv_row_begin, sch.s[i].kv_tokens};
+        f.s[i] = lbm_attn_stream{sch.s[i].q_begin, sch.s[i].q_rows, sch.s[i].kv_row_begin, sch.s[i].kv_tokens, sch.s[i].live_at};
         wg += ((sch.s[i].q_rows + kF32Rows - 1) / kF32Rows) * num_heads;
       }
     }
@@ -887,6 +898,7 @@ int lbm_launch_attention(const void* q, const void* pool, void* out, const void*
   a.self_k = (const unsigned short*)self_k;
   a.self_v = (const unsigned short*)self_v;
   a.kv_rows = kv_rows;
+  a.live_kv_tokens = live_kv_tokens;
   a.part_o = (unsigned short*)workspace;
   a.part_lse = (float*)(a.part_o + (size_t)sch.part_rows * num_heads * head_dim);
   a.num_heads = num_heads;

@@ -214,8 +214,10 @@ LBM_HD void lbm_phase_evict(int32_t* st, const lbm_cache_geom& g, const LbmTable
 // ---------------------------------------------------------------------------- plan
 // build_visible_page_table + compute_last_page_len (flashinfer_cache.py:438-470) with a
 // valid length per page, plus the dense row table the attention kernel gathers through.
-// Writes exactly op.expect_kv_tokens row entries so a host/device disagreement can never
-// make the attention kernel read outside the table (it sets LBM_TERR_KV_COUNT instead).
+// Never writes more row entries than the host says the table holds (op.expect_kv_tokens, or the
+// capacity it gives instead) and publishes a count within that bound, so a host/device
+// disagreement cannot make the attention kernel read outside the table (it sets
+// LBM_TERR_KV_COUNT instead).
 LBM_HD void lbm_phase_plan(int32_t* st, const lbm_cache_geom& g, const LbmTablesLayout& L,
                            const lbm_step_op& op, int32_t* kv_rows, int32_t* page_ids,
                            int32_t* page_lens, int tid, int nthr, LbmHdr& h) {
@@ -224,9 +226,12 @@ LBM_HD void lbm_phase_plan(int32_t* st, const lbm_cache_geom& g, const LbmTables
   const int nfr = h.na + h.wc;
   const int frame_tokens = nfr * L.tpf;
   const int self_n = op.self_tokens > 0 ? op.self_tokens : 0;
-  const int total = frame_tokens + h.stc + self_n;
-  const int limit = op.expect_kv_tokens;
-  if (total != limit) h.err |= LBM_TERR_KV_COUNT;
+  int total = frame_tokens + h.stc + self_n;
+  // expect_kv_tokens >= 0: the host's own count, which must agree; < 0: the host does not track
+  // the count and gives the capacity of this stream's part of kv_rows instead
+  const bool counted = op.expect_kv_tokens >= 0;
+  const int limit = counted ? op.expect_kv_tokens : -op.expect_kv_tokens;
+  if (counted ? total != limit : total > limit) h.err |= LBM_TERR_KV_COUNT;
   const int32_t* anchor = st + L.off_anchor;
   const int32_t* win = st + L.off_window;
   if (kv_rows) {
@@ -251,8 +256,10 @@ LBM_HD void lbm_phase_plan(int32_t* st, const lbm_cache_geom& g, const LbmTables
     }
     for (int t = tid; t < self_n; t += nthr)
       if (frame_tokens + h.stc + t < limit) out[frame_tokens + h.stc + t] = -1 - (op.q_begin + t);
-    for (int i = total + tid; i < limit; i += nthr) out[i] = 0;
+    if (counted)
+      for (int i = total + tid; i < limit; i += nthr) out[i] = 0;
   }
+  if (total > limit) total = limit;  // what the attention may read
   int n_pages = nfr * L.ppf + (two ? h.nsp : h.nmp);
   if (page_ids && page_lens) {
     int32_t* ids = page_ids + op.page_out_begin;

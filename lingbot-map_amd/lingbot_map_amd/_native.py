@@ -36,11 +36,11 @@ class StepOp(C.Structure):
 
 
 class AttnStream(C.Structure):
-    _fields_ = [(n, C.c_int32) for n in ("q_begin", "q_rows", "kv_row_begin", "kv_tokens")]
+    _fields_ = [(n, C.c_int32) for n in ("q_begin", "q_rows", "kv_row_begin", "kv_tokens", "live_at")]
 
 
 SYMBOLS = ("lbm_abi_version", "lbm_last_error", "lbm_tables_words", "lbm_tables_step",
-           "lbm_rows_from_pages", "lbm_kv_append", "lbm_qkv_prepare", "lbm_attn_workspace_bytes", "lbm_attn_run")
+           "lbm_rows_from_pages", "lbm_kv_append", "lbm_qkv_prepare", "lbm_attn_workspace_bytes", "lbm_attn_run", "lbm_attn_run_live")
 
 
 def _load():
@@ -67,6 +67,9 @@ def _load():
     lib.lbm_attn_run.restype = C.c_int
     lib.lbm_attn_run.argtypes = [vp, vp, vp, vp, vp, vp, p(AttnStream), i32, i32, i32, i32, i32,
                                  C.c_float, vp, C.c_size_t, vp]
+    lib.lbm_attn_run_live.restype = C.c_int
+    lib.lbm_attn_run_live.argtypes = [vp, vp, vp, vp, vp, vp, vp, p(AttnStream), i32, i32, i32, i32, i32,
+                                      C.c_float, vp, C.c_size_t, vp]
     if lib.lbm_abi_version() != ABI_VERSION:
         raise RuntimeError(f"{LIB_PATH}: ABI version {lib.lbm_abi_version()}, binding expects {ABI_VERSION}")
     return lib

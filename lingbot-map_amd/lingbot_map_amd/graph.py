@@ -18,8 +18,9 @@ from torch import Tensor
 class GraphedFrame:
     """``frame_fn(*inputs) -> Tensor`` runs one streamed frame of every stream through all blocks
     (it calls the manager's ``step`` / ``step_qkv`` for each block).  The manager must be in
-    ``steady_state`` (anchor and window full, evicted frames leaving no memory tokens) and every
-    frame replayed must be a keyframe; anything else has to go through the eager path.
+    ``steady_state`` (anchor and window full; evicted frames leaving no memory tokens unless the
+    manager was built with ``device_token_counts=True``) and every frame replayed must be a
+    keyframe; anything else has to go through the eager path.
 
     Calls overlap with nothing else on the manager: like the manager itself this is not
     re-entrant."""
@@ -30,6 +31,7 @@ class GraphedFrame:
             raise RuntimeError("GraphedFrame: the cache is not in a replayable steady state "
                                "(anchor and window full, no trajectory-memory growth, keyframes only)")
         self.manager = manager
+        self._evict_args = (cross_frame_special, camera_only)
         self._inputs = [t.clone() for t in example_inputs]
         # one eager frame on a side stream first (library handles, workspaces, autotuning)
         side = torch.cuda.Stream()
@@ -41,7 +43,7 @@ class GraphedFrame:
         with torch.cuda.graph(self.graph), torch.no_grad():
             self._output = frame_fn(*self._inputs)
         # the capture ran the host side of one frame without executing it on the device
-        manager.note_replayed_frames(-1)
+        manager.note_replayed_frames(-1, cross_frame_special, camera_only)
         if not manager.steady_state(cross_frame_special, camera_only):
             raise RuntimeError("GraphedFrame: the captured frame left the steady state")
 
@@ -50,5 +52,5 @@ class GraphedFrame:
         for dst, src in zip(self._inputs, inputs):
             dst.copy_(src)
         self.graph.replay()
-        self.manager.note_replayed_frames(1)
+        self.manager.note_replayed_frames(1, *self._evict_args)
         return self._output

@@ -18,6 +18,9 @@ Extensions beyond the reference signature (all keyword-only, defaults = referenc
 ``num_streams``      independent streams batched in every call (k, v, q are the streams'
                      frames concatenated on the token axis)
 ``per_block_tables`` one table set per block instead of one shared by all blocks
+``device_token_counts`` the attention kernels read each stream's visible-token count from the
+                     device tables instead of the launch arguments, so that a frame's launches
+                     stay identical while the trajectory memory grows (HIP-graph replay)
 
 With shared tables block 0 leads, as the reference's ``plan()`` at ``block_idx == 0`` does
 (flashinfer_cache.py:385-414): table operations run when ``block_idx == 0`` and the other
@@ -74,6 +77,7 @@ class HipPagedKVCacheManager:
         layout: str = "two_stream",
         num_streams: int = 1,
         per_block_tables: bool = False,
+        device_token_counts: bool = False,
     ):
         device = torch.device(device)
         if device.type != "cuda":
@@ -110,6 +114,7 @@ class HipPagedKVCacheManager:
         self.layout = layout
         self.num_streams = num_streams
         self.per_block_tables = per_block_tables
+        self.device_token_counts = bool(device_token_counts)
         self.force_fp32 = force_fp32
         if force_fp32:  # flashinfer_cache.py:121-127
             self.dtype = torch.float32
@@ -205,6 +210,11 @@ class HipPagedKVCacheManager:
             C.c_void_p(self._page_ids.data_ptr()) if pages else None,
             C.c_void_p(self._page_lens.data_ptr()) if pages else None,
             self._stream_handle()))
+
+    def _expect(self, n: int) -> int:
+        """PLAN's token argument: the host's count, or - with device-side counts - minus the
+        capacity of the stream's row table."""
+        return -self._rows_cap if self.device_token_counts else n
 
     def _visible_tokens(self, c: _StreamCounts) -> int:
         return (c.n_anchor + c.win_count) * self._tpf + c.special_tokens
@@ -373,7 +383,8 @@ class HipPagedKVCacheManager:
             tail = self.tokens_per_frame if self_tail[b] else 0
             n = self._visible_tokens(c) + tail if self._active[b] else 0
             self._plan_tokens[ts][b] = n
-            per.append({"ops": N.OP_PLAN if self._active[b] else 0, "self_tokens": tail, "expect_kv_tokens": n})
+            per.append({"ops": N.OP_PLAN if self._active[b] else 0, "self_tokens": tail,
+                        "expect_kv_tokens": self._expect(n)})
         self._tables_step(ts, self._ops(per), kv_rows=True, pages=pages)
         self._plan_valid[ts] = True
 
@@ -455,10 +466,11 @@ class HipPagedKVCacheManager:
 
     def steady_state(self, cross_frame_special: bool = True, camera_only: bool = False) -> bool:
         """True when one more keyframe step of every active stream would launch exactly what
-        the last one launched: same table operations, same visible token counts, same attention
-        schedule.  That holds once anchor and window are full and evicted frames leave no
-        memory tokens behind; it is the condition under which a captured HIP graph of a frame
-        may be replayed (the page ids live on the device and keep evolving across replays)."""
+        the last one launched - the condition under which a captured HIP graph of a frame may be
+        replayed (page ids live on the device and keep evolving across replays).  Anchor and
+        window must be full.  With host-side token counts the visible token count must not change
+        either, i.e. evicted frames must leave no memory tokens; with ``device_token_counts`` the
+        kernels read the count on the device and the trajectory memory may grow."""
         if self._skip_append or self._defer_eviction or not any(self._active):
             return False
         keep = self._keep_tokens(cross_frame_special, camera_only)
@@ -473,20 +485,41 @@ class HipPagedKVCacheManager:
                 before = self._visible_tokens(c)
                 self._mirror_append(probe, 0)
                 self._mirror_evict(probe, self._windows[b], keep, 0)
-                same = all(getattr(probe, f) == getattr(c, f) for f in _StreamCounts.__slots__ if f != "frame_count")
-                if not same or self._visible_tokens(probe) != before or not self._plan_valid[ts]:
+                grows = ("frame_count", "n_memory", "n_memory_pages", "special_tokens", "n_free_patch") \
+                    if self.device_token_counts and self.layout == "frame_pages" else ("frame_count",)
+                same = all(getattr(probe, f) == getattr(c, f) for f in _StreamCounts.__slots__ if f not in grows)
+                if not same or not self._plan_valid[ts]:
+                    return False
+                if not self.device_token_counts and self._visible_tokens(probe) != before:
                     return False
         return True
 
-    def note_replayed_frames(self, n: int = 1) -> None:
-        """Book-keeping after replaying a captured steady-state frame ``n`` times: the device
-        tables advanced, the host's frame counters follow."""
+    def note_replayed_frames(self, n: int = 1, cross_frame_special: bool = True, camera_only: bool = False) -> None:
+        """Book-keeping after replaying a captured steady-state keyframe ``n`` times (``n = -1``
+        takes back the host side of a frame that was only captured, not executed): the device
+        tables advanced, the host's mirror follows."""
+        keep = self._keep_tokens(cross_frame_special, camera_only)
         for i in range(self.num_blocks):
             self.frame_count[i] += n
         for ts in range(self._n_sets):
             for b in range(self.num_streams):
-                if self._active[b]:
-                    self._counts[ts][b].frame_count += n
+                if not self._active[b]:
+                    continue
+                c = self._counts[ts][b]
+                if n < 0 or keep == 0:
+                    c.frame_count += n
+                    if n < 0 and keep:   # undo the memory growth of the captured frame
+                        kp = _ceil_div(keep, self.page_size)
+                        c.n_memory += n
+                        c.n_memory_pages += n * kp
+                        c.special_tokens += n * keep
+                        c.n_free_patch -= n * kp
+                    self._plan_tokens[ts][b] = self._visible_tokens(c)
+                    continue
+                for _ in range(n):
+                    self._mirror_append(c, 0)
+                    self._mirror_evict(c, self._windows[b], keep, 0)
+                self._plan_tokens[ts][b] = self._visible_tokens(c)
 
     def _step_tables(self, block_idx: int, keyframe: Optional[Sequence[bool]], cross_frame_special: bool,
                      camera_only: bool):
@@ -515,7 +548,8 @@ class HipPagedKVCacheManager:
                     n = self._visible_tokens(c) + self.tokens_per_frame
                 self._plan_tokens[ts][b] = n
                 per.append({"ops": ops, "sliding_window": self._windows[b], "keep_tokens": keep,
-                            "self_tokens": self.tokens_per_frame if tail[b] else 0, "expect_kv_tokens": n})
+                            "self_tokens": self.tokens_per_frame if tail[b] else 0,
+                            "expect_kv_tokens": self._expect(n)})
             self._tables_step(ts, self._ops(per), append_rows=True, kv_rows=True)
             self._plan_valid[ts] = True
         return ts, keyframe, tail
@@ -536,7 +570,7 @@ class HipPagedKVCacheManager:
         for b in range(self.num_streams):
             kv = self._plan_tokens[ts][b]
             if kv > 0:
-                streams[n] = N.AttnStream(b * T, T, b * self._rows_cap, kv)
+                streams[n] = N.AttnStream(b * T, T, b * self._rows_cap, kv, b * self._table_words)
                 n += 1
         if n < self.num_streams:
             out.zero_()
@@ -545,12 +579,19 @@ class HipPagedKVCacheManager:
         need = N.lib.lbm_attn_workspace_bytes(streams, n, self.num_heads, self.head_dim)
         if need > self.workspace_buffer.numel():
             self.workspace_buffer = torch.empty(int(need * 1.25) + 256, dtype=torch.uint8, device=self.device)
-        N.check(N.lib.lbm_attn_run(
-            C.c_void_p(qc.data_ptr()), C.c_void_p(self.kv_caches[block_idx].data_ptr()), C.c_void_p(out.data_ptr()),
-            C.c_void_p(self_k.data_ptr()) if has_tail else None, C.c_void_p(self_v.data_ptr()) if has_tail else None,
-            C.c_void_p(self._kv_rows[ts].data_ptr()), streams, n, self.num_heads, self.head_dim, self.page_size,
-            N.DTYPE_BF16 if self.dtype == torch.bfloat16 else N.DTYPE_F32, 1.0 / math.sqrt(self.head_dim),
-            C.c_void_p(self.workspace_buffer.data_ptr()), self.workspace_buffer.numel(), self._stream_handle()))
+        common = (streams, n, self.num_heads, self.head_dim, self.page_size,
+                  N.DTYPE_BF16 if self.dtype == torch.bfloat16 else N.DTYPE_F32, 1.0 / math.sqrt(self.head_dim),
+                  C.c_void_p(self.workspace_buffer.data_ptr()), self.workspace_buffer.numel(), self._stream_handle())
+        tensors = (C.c_void_p(qc.data_ptr()), C.c_void_p(self.kv_caches[block_idx].data_ptr()), C.c_void_p(out.data_ptr()),
+                   C.c_void_p(self_k.data_ptr()) if has_tail else None, C.c_void_p(self_v.data_ptr()) if has_tail else None,
+                   C.c_void_p(self._kv_rows[ts].data_ptr()))
+        if self.device_token_counts:
+            # the kernels read each stream's visible-token count from its table header, where the
+            # last plan left it; the host's count above only sizes the launch
+            live = self._tables[ts].data_ptr() + 4 * N.HDR["plan_kv_tokens"]
+            N.check(N.lib.lbm_attn_run_live(*tensors, C.c_void_p(live), *common))
+        else:
+            N.check(N.lib.lbm_attn_run(*tensors, *common))
         return out
 
     def reset(self) -> None:

@@ -44,7 +44,7 @@ def test_binding_constants_match_header():
     assert (defs["LBM_DTYPE_BF16"], defs["LBM_DTYPE_F32"]) == (N.DTYPE_BF16, N.DTYPE_F32)
     assert (defs["LBM_LAYOUT_TWO_STREAM"], defs["LBM_LAYOUT_FRAME_PAGES"]) == (N.LAYOUT_TWO_STREAM, N.LAYOUT_FRAME_PAGES)
     # struct sizes: plain int32 fields, no padding
-    assert C.sizeof(N.CacheGeom) == 9 * 4 and C.sizeof(N.StepOp) == 8 * 4 and C.sizeof(N.AttnStream) == 4 * 4
+    assert C.sizeof(N.CacheGeom) == 9 * 4 and C.sizeof(N.StepOp) == 8 * 4 and C.sizeof(N.AttnStream) == 5 * 4
 
 
 def test_host_side_argument_checks_need_no_gpu():
