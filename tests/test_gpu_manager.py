@@ -159,3 +159,58 @@ def test_fused_step_matches_method_by_method():
         assert torch.equal(a._tables[..., :11], b._tables[..., :11])
         assert a.build_visible_page_table(0) == b.build_visible_page_table(0)
     assert torch.equal(a.kv_caches[1], b.kv_caches[1])
+
+
+@pytest.mark.parametrize("layout,page_size", [("two_stream", None), ("frame_pages", 16)])
+def test_flow_keyframe_protocol_of_the_windowed_driver(layout, page_size):
+    """The windowed driver decides after the forward pass whether a frame is a keyframe
+    (lingbot_map/models/gct_stream_window.py:362-420): eviction is deferred, every block appends
+    and attends, then either every block rolls the frame back or every block runs the deferred
+    eviction; the cache is reset between windows.  Ids, counters, pool and outputs against the
+    oracle after every frame."""
+    from oracle.page_policy import PagePolicy
+    from oracle.sdpa_cache import PagedStreamOracle
+    T, n_sp, scale, window, H, blocks = 53, 5, 2, 3, 4, 3
+    m = make(layout, page_size, T=T, n_sp=n_sp, scale=scale, window=window, max_total=64, H=H, blocks=blocks)
+    pol = [PagePolicy(T, n_sp, page_size, scale, window, 64, layout=layout) for _ in range(blocks)]
+    orc = [PagedStreamOracle(p, H, 64, torch.bfloat16) for p in pol]
+    g = torch.Generator().manual_seed(19)
+    for win in range(2):
+        for f in range(18):
+            accept = f < scale or bool(torch.rand(1, generator=g).item() < 0.6)
+            m._defer_eviction = True
+            for p in pol:
+                p._defer_eviction = True
+            for b in range(blocks):
+                q, k, v = frame(T, H, g)
+                orc[b].append_frame(k, v)
+                pol[b].evict_frames(scale, window)               # suppressed while deferred
+                ref = orc[b].compute_attention(q)
+                m.append_frame(b, k.cuda(), v.cuda())
+                m.evict_frames(b, scale, window)
+                out = m.compute_attention(b, q.cuda())
+                err = (out.float().cpu() - ref.float()).abs()
+                assert err.max().item() <= BF16_MAX_ABS and err.mean().item() <= BF16_MEAN_ABS, (win, f, b)
+            for b in range(blocks):
+                if accept:
+                    m.execute_deferred_eviction(b, scale_frames=scale, sliding_window=window)
+                    pol[b].execute_deferred_eviction(scale, window)
+                else:
+                    m.rollback_last_frame(b)
+                    pol[b].rollback_last_frame()
+            m._defer_eviction = False
+            for p in pol:
+                p._defer_eviction = False
+            assert m.build_visible_page_table(0) == pol[0].build_visible_page_table(), (win, f)
+            assert m.build_visible_page_lens(0) == pol[0].build_visible_page_lens()
+            assert m.get_cache_stats(0) == pol[0].get_cache_stats()
+            assert m.device_header()["error"] == 0
+        for b in range(blocks):
+            ids, lens = pol[b].build_visible_page_table(), pol[b].build_visible_page_lens()
+            dev_pool = m.kv_caches[b].cpu()
+            for p, n in zip(ids, lens):
+                assert torch.equal(dev_pool[p, :, :n], orc[b].pool[p, :, :n])
+        m.reset()
+        for p in pol:
+            p.reset()
+        assert m.num_frames == 0 and m.build_visible_page_table(0) == []
