@@ -247,6 +247,59 @@ def test_attention_edge_shapes():
     assert rc != N.OK and b"n_streams" in N.lib.lbm_last_error()
 
 
+@pytest.mark.parametrize("seed", range(6))
+def test_attention_random_shapes(seed):
+    """Seeded sweep over shapes the fixed cases do not hit: 1-3 streams with unrelated query
+    and KV sizes (1..1100 rows, 1..6000 tokens), 1..16 heads, page sizes 1..64, rows scattered
+    over the pool, sometimes a read-only tail, score spread from flat to peaked (for which the
+    bar is doubled, see below)."""
+    from oracle.sdpa_cache import sdpa_nhd
+    dev = torch.device("cuda:0")
+    g = torch.Generator().manual_seed(1000 + seed)
+    ri = lambda lo, hi: int(torch.randint(lo, hi + 1, (1,), generator=g))
+    for case in range(5):
+        H, D = [1, 2, 3, 8, 16][ri(0, 4)], 64
+        S = [1, 4, 16, 64][ri(0, 3)]
+        n_streams = ri(1, 3)
+        qn = [ri(1, 1100) if ri(0, 2) else ri(1, 70) for _ in range(n_streams)]
+        kn = [ri(1, 6000) if ri(0, 2) else ri(1, 130) for _ in range(n_streams)]
+        tail = ri(0, 2) == 0
+        spread = [0.05, 1.0, 3.0][ri(0, 2)]
+        n_slots = sum(kn) + 37
+        pages = -(-n_slots // S)
+        pool = torch.randn(pages, 2, S, H, D, generator=g)
+        pool[:, 0] *= spread
+        pool = pool.to(torch.bfloat16)
+        flat_k, flat_v = pool[:, 0].reshape(-1, H, D), pool[:, 1].reshape(-1, H, D)
+        q = torch.randn(sum(qn), H, D, generator=g).to(torch.bfloat16)
+        sk = (spread * torch.randn(sum(qn), H, D, generator=g)).to(torch.bfloat16)
+        sv = torch.randn(sum(qn), H, D, generator=g).to(torch.bfloat16)
+        perm = torch.randperm(pages * S, generator=g)
+        rows, streams, refs, qo, ko = [], [], [], 0, 0
+        for b in range(n_streams):
+            slots = perm[ko:ko + kn[b]]
+            r = ((slots // S) * 2 * S + slots % S).to(torch.int32)
+            kk, vv = flat_k[slots], flat_v[slots]
+            if tail:   # the stream also attends to its own rows
+                r = torch.cat([r, (-1 - torch.arange(qo, qo + qn[b])).to(torch.int32)])
+                kk, vv = torch.cat([kk, sk[qo:qo + qn[b]]]), torch.cat([vv, sv[qo:qo + qn[b]]])
+            streams.append((qo, qn[b], sum(x.numel() for x in rows), r.numel()))
+            rows.append(r)
+            refs.append(sdpa_nhd(q[qo:qo + qn[b]], kk, vv))
+            qo += qn[b]
+            ko += kn[b]
+        out = run_attention(q.to(dev), pool.to(dev), torch.cat(rows).to(dev), streams, S,
+                            sk.to(dev) if tail else None, sv.to(dev) if tail else None).cpu()
+        for (qb, nq, _, _), ref in zip(streams, refs):
+            err = (out[qb:qb + nq].float() - ref.float()).abs()
+            assert torch.isfinite(out[qb:qb + nq].float()).all()
+            # peaked scores (keys three times as long): the kernel rounds q * scale * log2(e) to
+            # bf16 once more than the reference does, which costs about 1 % of the output there
+            bar = 1.0 if spread <= 1.0 else 2.0
+            assert err.max().item() <= bar * BF16_MAX_ABS and err.mean().item() <= bar * BF16_MEAN_ABS, (
+                seed, case, H, S, qn, kn, tail, spread, err.max().item())
+
+
 @pytest.mark.parametrize("src,dst", [(torch.bfloat16, torch.bfloat16), (torch.float32, torch.bfloat16),
                                      (torch.float32, torch.float32), (torch.bfloat16, torch.float32)])
 def test_append_is_exact_and_gated(src, dst):
