@@ -593,10 +593,11 @@ __global__ __launch_bounds__(256) void lbm_attn_combine_bf16_kernel(AttnArgs a) 
 // Same contract as the bf16 kernel for pools kept in fp32 (the reference's force_fp32 mode,
 // lingbot_map/layers/flashinfer_cache.py:118-127,372-383).  Accuracy path, not a speed path:
 // plain fp32 FMAs, one workgroup per (64 query rows, head), four threads per query row that
-// each own 16 of the 64 head dimensions; exact running maximum, no split-KV.
+// each own a quarter of the head dimensions; exact running maximum, no split-KV.  head_dim 64,
+// and 128 for the camera head's one-token-per-frame cache (lingbot_map/heads/camera_head.py:
+// 284-377: 16 heads of 128, fp32).
 namespace {
 constexpr int kF32Rows = 64;
-constexpr int kF32Tile = 64;
 struct AttnArgsF32 {
   const float* q;
   const float* pool;
@@ -614,9 +615,14 @@ struct AttnArgsF32 {
 };
 }  // namespace
 
-__global__ __launch_bounds__(256) void lbm_attn_f32_d64_kernel(AttnArgsF32 a) {
-  __shared__ __attribute__((aligned(16))) float lds_k[kF32Tile][64];
-  __shared__ __attribute__((aligned(16))) float lds_v[kF32Tile][64];
+template <int D>
+__global__ __launch_bounds__(256) void lbm_attn_f32_kernel(AttnArgsF32 a) {
+  constexpr int kTile = D == 64 ? 64 : 32;     // KV tokens per tile: 32 KiB of LDS either way
+  constexpr int kStageThreads = 256 / kTile;   // threads that stage one row: 16 floats each
+  constexpr int DQ = D / 4;                    // head dims per compute thread
+  static_assert(D / kStageThreads == 16, "staging moves 16 floats per thread");
+  __shared__ __attribute__((aligned(16))) float lds_k[kTile][D];
+  __shared__ __attribute__((aligned(16))) float lds_v[kTile][D];
   const int tid = threadIdx.x;
   int b = 0;
   for (int i = 1; i < a.n_streams; ++i)
@@ -627,24 +633,24 @@ __global__ __launch_bounds__(256) void lbm_attn_f32_d64_kernel(AttnArgsF32 a) {
   const int local = (int)blockIdx.x - a.wg_begin[b];
   const int head = local % H, qt = local / H;
   const int r = qt * kF32Rows + (tid >> 2), c = tid & 3;  // query row, quarter of the head dim
-  const size_t row_elems = (size_t)H * 64;
+  const size_t row_elems = (size_t)H * D;
   const bool row_ok = r < sp.q_rows;
 
-  float q[16], o[16];
+  float q[DQ], o[DQ];
   {
-    const float* qp = a.q + ((size_t)(sp.q_begin + (row_ok ? r : 0)) * H + head) * 64 + c * 16;
+    const float* qp = a.q + ((size_t)(sp.q_begin + (row_ok ? r : 0)) * H + head) * D + c * DQ;
 #pragma unroll
-    for (int d = 0; d < 16; ++d) {
+    for (int d = 0; d < DQ; ++d) {
       q[d] = row_ok ? qp[d] * a.scale_log2 : 0.f;
       o[d] = 0.f;
     }
   }
   float m = -INFINITY, l = 0.f;
 
-  const int ld_r = tid >> 2, ld_c = (tid & 3) * 16;  // each thread stages 16 floats of one K and V row
-  const int n_tiles = (sp.kv_tokens + kF32Tile - 1) / kF32Tile;
+  const int ld_r = tid / kStageThreads, ld_c = (tid % kStageThreads) * 16;
+  const int n_tiles = (sp.kv_tokens + kTile - 1) / kTile;
   for (int t = 0; t < n_tiles; ++t) {
-    const int kvi = t * kF32Tile + ld_r;
+    const int kvi = t * kTile + ld_r;
     f32x4 kk[4], vv[4];
 #pragma unroll
     for (int i = 0; i < 4; ++i) kk[i] = vv[i] = f32x4{0.f, 0.f, 0.f, 0.f};
@@ -652,10 +658,10 @@ __global__ __launch_bounds__(256) void lbm_attn_f32_d64_kernel(AttnArgsF32 a) {
       const int e = a.kv_rows[sp.kv_row_begin + kvi];
       const float *kp, *vp;
       if (e >= 0) {
-        kp = a.pool + ((size_t)e * H + head) * 64 + ld_c;
+        kp = a.pool + ((size_t)e * H + head) * D + ld_c;
         vp = kp + (size_t)a.page_size * row_elems;
       } else {
-        const size_t off = ((size_t)(-1 - e) * H + head) * 64 + ld_c;
+        const size_t off = ((size_t)(-1 - e) * H + head) * D + ld_c;
         kp = a.self_k + off;
         vp = a.self_v + off;
       }
@@ -672,7 +678,7 @@ __global__ __launch_bounds__(256) void lbm_attn_f32_d64_kernel(AttnArgsF32 a) {
       *(f32x4*)&lds_v[ld_r][ld_c + 4 * i] = vv[i];
     }
     __syncthreads();
-    const int n_valid = min(kF32Tile, sp.kv_tokens - t * kF32Tile);
+    const int n_valid = min(kTile, sp.kv_tokens - t * kTile);
     for (int j0 = 0; j0 < n_valid; j0 += 8) {
       float sc[8];
 #pragma unroll
@@ -680,7 +686,7 @@ __global__ __launch_bounds__(256) void lbm_attn_f32_d64_kernel(AttnArgsF32 a) {
         const int j = j0 + jj;
         float acc = 0.f;
 #pragma unroll
-        for (int d = 0; d < 16; ++d) acc = __builtin_fmaf(q[d], lds_k[j][c * 16 + d], acc);
+        for (int d = 0; d < DQ; ++d) acc = __builtin_fmaf(q[d], lds_k[j][c * DQ + d], acc);
         acc += __shfl_xor(acc, 1);
         acc += __shfl_xor(acc, 2);
         sc[jj] = j < n_valid ? acc : -INFINITY;
@@ -692,22 +698,22 @@ __global__ __launch_bounds__(256) void lbm_attn_f32_d64_kernel(AttnArgsF32 a) {
       m = mx;
       l *= alpha;
 #pragma unroll
-      for (int d = 0; d < 16; ++d) o[d] *= alpha;
+      for (int d = 0; d < DQ; ++d) o[d] *= alpha;
 #pragma unroll
       for (int jj = 0; jj < 8; ++jj) {
         const float p = exp2f(sc[jj] - m);
         l += p;
-        const int j = min(j0 + jj, kF32Tile - 1);
+        const int j = min(j0 + jj, kTile - 1);
 #pragma unroll
-        for (int d = 0; d < 16; ++d) o[d] = __builtin_fmaf(p, lds_v[j][c * 16 + d], o[d]);
+        for (int d = 0; d < DQ; ++d) o[d] = __builtin_fmaf(p, lds_v[j][c * DQ + d], o[d]);
       }
     }
   }
   if (row_ok) {
     const float inv = l > 0.f ? 1.0f / l : 0.f;
-    float* op = a.out + ((size_t)(sp.q_begin + r) * H + head) * 64 + c * 16;
+    float* op = a.out + ((size_t)(sp.q_begin + r) * H + head) * D + c * DQ;
 #pragma unroll
-    for (int d = 0; d < 16; ++d) op[d] = o[d] * inv;
+    for (int d = 0; d < DQ; ++d) op[d] = o[d] * inv;
   }
 }
 
@@ -861,8 +867,8 @@ int lbm_launch_attention(const void* q, const void* pool, void* out, const void*
                          const LbmAttnSchedule& sch,
                          int num_heads, int head_dim, int page_size, int dtype, float sm_scale,
                          void* workspace, hipStream_t stream) {
-  if (head_dim != 64)
-    return lbm_fail(LBM_ERR_UNSUPPORTED, "attention kernels cover head_dim 64 (got %d)", head_dim);
+  if (head_dim != 64 && !(head_dim == 128 && dtype == LBM_DTYPE_F32))
+    return lbm_fail(LBM_ERR_UNSUPPORTED, "attention kernels cover head_dim 64 (bf16, fp32) and 128 (fp32), got %d", head_dim);
   if (dtype == LBM_DTYPE_F32) {
     AttnArgsF32 f;
     f.q = (const float*)q;
@@ -887,8 +893,9 @@ int lbm_launch_attention(const void* q, const void* pool, void* out, const void*
     }
     f.wg_begin[LBM_MAX_STREAMS] = wg;
     if (wg == 0) return LBM_OK;
-    hipLaunchKernelGGL(lbm_attn_f32_d64_kernel, dim3(wg), dim3(256), 0, stream, f);
-    return lbm_check_launch("lbm_attn_f32_d64_kernel");
+    if (head_dim == 64) hipLaunchKernelGGL(lbm_attn_f32_kernel<64>, dim3(wg), dim3(256), 0, stream, f);
+    else hipLaunchKernelGGL(lbm_attn_f32_kernel<128>, dim3(wg), dim3(256), 0, stream, f);
+    return lbm_check_launch("lbm_attn_f32_kernel");
   }
   if (dtype != LBM_DTYPE_BF16) return lbm_fail(LBM_ERR_INVALID, "unknown dtype %d", dtype);
   AttnArgs a;

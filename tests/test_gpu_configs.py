@@ -193,3 +193,34 @@ def test_config5_four_ragged_streams():
         assert m.build_visible_page_lens(0, stream=b) == pols[b].build_visible_page_lens()
         assert pols[b].visible_tokens() == (1 + windows[b]) * T + 5 * (19 - 1 - windows[b])
     assert m.device_header()["error"] == 0
+
+
+@pytest.mark.parametrize("layout,page_size", [("two_stream", None), ("frame_pages", 1), ("frame_pages", 8)])
+def test_camera_head_cache_one_token_per_frame_head_dim_128(layout, page_size):
+    """The camera head keeps one token per frame in 16 heads of 128 and never evicts
+    (lingbot_map/heads/camera_head.py:284-377; lingbot_map/layers/attention.py:307: its eviction
+    guard is false for one-token frames), in fp32.  The same manager holds that cache: every
+    frame appends one token per block and attends to all of them; 1e-5 against float64."""
+    from lingbot_map_amd import HipPagedKVCacheManager
+    dev = torch.device("cuda:0")
+    H, D, blocks, frames = 16, 128, 4, 150
+    m = HipPagedKVCacheManager(blocks, frames + 8, 1, H, D, torch.float32, dev, num_special_tokens=0, scale_frames=8,
+                               sliding_window=frames, max_total_frames=frames + 8, force_fp32=True,
+                               page_size=page_size, layout=layout)
+    assert m.dtype == torch.float32
+    g = torch.Generator().manual_seed(21)
+    ks = [[] for _ in range(blocks)]
+    vs = [[] for _ in range(blocks)]
+    for f in range(frames):
+        for b in range(blocks):
+            q, k, v = (torch.randn(1, H, D, generator=g) for _ in range(3))
+            ks[b].append(k); vs[b].append(v)
+            m.append_frame(b, k.to(dev), v.to(dev))
+            m.evict_frames(b, 8, frames)
+            out = m.compute_attention(b, q.to(dev)).cpu()
+            if f % 37 == 0 or f == frames - 1:
+                K, V = torch.cat(ks[b]).double(), torch.cat(vs[b]).double()          # [f+1, H, D]
+                s = torch.einsum("qhd,khd->hqk", q.double(), K) / D ** 0.5
+                ref = torch.einsum("hqk,khd->qhd", torch.softmax(s, -1), V)
+                assert (out.double() - ref).abs().max().item() <= 1e-5, (f, b)
+    assert m.num_frames == frames and m.device_header()["error"] == 0
