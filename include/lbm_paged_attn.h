@@ -24,7 +24,7 @@
 extern "C" {
 #endif
 
-#define LBM_ABI_VERSION 1
+#define LBM_ABI_VERSION 2
 
 #define LBM_OK 0
 #define LBM_ERR_INVALID 1     /* bad argument (null pointer, negative size, bad enum)      */

@@ -20,7 +20,7 @@ HDR = {"frame_count": 0, "n_anchor": 1, "win_head": 2, "win_count": 3, "n_free_p
        "n_free_special": 5, "n_special_pages": 6, "special_tokens": 7, "n_memory": 8,
        "n_memory_pages": 9, "error": 10, "plan_kv_tokens": 11, "plan_n_pages": 12}
 HDR_WORDS = 16
-ABI_VERSION = 1
+ABI_VERSION = 2
 
 
 class CacheGeom(C.Structure):
