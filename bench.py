@@ -88,7 +88,7 @@ def cpu_baseline(torch, kv_tokens: int, blocks: int) -> dict:
     for _ in range(2):
         one()
     times = []
-    for _ in range(5):
+    for _ in range(15):
         t0 = time.perf_counter()
         one()
         times.append(time.perf_counter() - t0)
@@ -96,7 +96,7 @@ def cpu_baseline(torch, kv_tokens: int, blocks: int) -> dict:
     flops = 4.0 * T * kv_tokens * H * D
     return {
         "value": 1.0 / (t * blocks), "unit": "frames/s", "cores": torch.get_num_threads(), "kind": "port",
-        "sample": f"2 warm-up + 5 timed layer-steps of gather + SDPA (q {T} x kv {kv_tokens}, {H} heads, "
+        "sample": f"2 warm-up + 15 timed layer-steps of gather + SDPA (q {T} x kv {kv_tokens}, {H} heads, "
                   f"bf16 storage, fp32 math), median {t * 1e3:.1f} ms = {flops / t * 1e-9:.0f} GFLOP/s; "
                   f"frames/s = 1 / ({blocks} x median)",
     }
