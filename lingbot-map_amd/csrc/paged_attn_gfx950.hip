@@ -20,7 +20,7 @@
 // is >= 2 (or infinite) exactly when the top bit of its exponent field is set.
 //
 // Why it is built this way.  Measured on MI355X with two wavefronts per SIMD: v_exp_f32 issues
-// every ~4.6 ns per SIMD, v_cvt_pk_bf16_f32 / v_max3_f32 / v_dot2c_f32_bf16 every ~2.7 ns, plain
+// every ~4.6 ns per SIMD, v_cvt_pk_bf16_f32 (like v_max3_f32, v_dot2c_f32_bf16) every ~2.7 ns, plain
 // fp32 adds and multiplies every ~1.4 ns, and a 32x32x16 MFMA occupies the matrix pipe for
 // 13.8 ns.  With head_dim 64 every score needs one exp2 and half a packing instruction, so the
 // vector ALU, not the matrix pipe, bounds the loop; everything that can run as an MFMA (scale,
@@ -166,9 +166,9 @@ __global__ __launch_bounds__(kThreads, 1) void lbm_attn_bf16_d64_kernel(AttnArgs
       qf[qb][ks] = __builtin_convertvector(f, bf16x8);
     }
   }
-  // One more 16-wide step of the QK contraction carries the running reference maximum:
-  // K side is the constant row (-1, -1, 0, ...), Q side is (m_hi, m_lo, 0, ...) with
-  // m_hi + m_lo = m_run exactly, so S arrives as score*scale - m_run at no vector-ALU cost.
+  // One more 16-wide step of the QK contraction carries the softmax reference: K side is the
+  // constant row (-1, -1, 0, ...), Q side is (m_hi, m_lo, 0, ...) with m_hi + m_lo = m_run
+  // exactly, so S arrives as score*scale - m_run at no vector-ALU cost.
   // A third element masks the rows past the last token: K side -1 on such rows (0 elsewhere),
   // Q side 2^100, so their scores arrive as about -2^100 and their numerators are exactly 0.
   u32x4 kaug_bits = {0u, 0u, 0u, 0u};
@@ -305,10 +305,10 @@ __global__ __launch_bounds__(kThreads, 1) void lbm_attn_bf16_d64_kernel(AttnArgs
   };
   // Rare path of a half-step: a numerator of `cur` came out as 2 or more, i.e. a score
   // exceeded the reference by at least 1 (in log2 units; an overflow to infinity included).
-  // Nothing has consumed these numerators yet.  Raise the reference to the row maxima, rescale
-  // what is already expressed in the old one (O, the row sums, and the scores of `cur` and of
-  // `next`, which the MFMAs of this half-step produced with the old reference) and recompute
-  // the numerators, which are then at most 1.
+  // Nothing has consumed these numerators yet.  Raise the reference to kHeadroom above the row
+  // maxima, rescale what is already expressed in the old one (O, the row sums, and the scores
+  // of `cur` and of `next`, which the MFMAs of this half-step produced with the old reference)
+  // and recompute the numerators, which are then at most 2^-kHeadroom.
   auto raise_reference = [&](f32x16 (&cur)[2], bf16x8 (&pd)[2][2], f32x16 (&next)[2]) {
     float mx[2];
     row_max(cur, mx);
