@@ -103,12 +103,14 @@ def cpu_baseline(torch, kv_tokens: int, blocks: int) -> dict:
 
 
 def aggregator_step(torch, blocks: int, steps: int, warmup: int) -> dict:
-    """One streamed frame through `blocks` groups of (frame block, global block) at ViT-L size
-    (dim 1024, 16 heads, MLP 4096, LayerNorm, qk-norm, rotary embedding, LayerScale), random
-    init, bf16: the aggregator's alternating-attention trunk (lingbot_map/aggregator/stream.py:
-    415-529).  The global blocks run the HIP cache path; linears, norms, GELU and the frame
-    blocks' dense attention are PyTorch-ROCm library calls.  Patch embedding, the image encoder
-    and the prediction heads are not part of the step."""
+    """One streamed frame (a 3 x 378 x 518 image) through the image encoder's ViT-L trunk (patch
+    embedding, 24 blocks; lingbot_map/layers/vision_transformer.py:383-394) and through `blocks`
+    groups of (frame block, global block) of the aggregator (lingbot_map/aggregator/stream.py:
+    415-529), all at ViT-L size (dim 1024, 16 heads, MLP 4096, LayerNorm, LayerScale; qk-norm and
+    rotary embedding in the aggregator blocks), random init, bf16.  The global blocks run the HIP
+    cache path, every block's pre-attention producer and cache-less attention are HIP kernels
+    too; linears, LayerNorm, GELU and the patch-embedding convolution are PyTorch-ROCm library
+    calls.  The prediction heads are not part of the step."""
     from lingbot_map_amd import HipPagedBlock, HipPagedKVCacheManager, RotaryPositionEmbedding2D
     dev = torch.device("cuda:0")
     dim = H * D
@@ -120,20 +122,27 @@ def aggregator_step(torch, blocks: int, steps: int, warmup: int) -> dict:
     rope2d = RotaryPositionEmbedding2D()    # frame blocks: 2-D embedding over the 27 x 37 patch grid
     frame_blocks = [HipPagedBlock(rope=rope2d, **kw).to(dev, torch.bfloat16).eval() for _ in range(blocks)]
     global_blocks = [HipPagedBlock(rope=True, **kw).to(dev, torch.bfloat16).eval() for _ in range(blocks)]
+    encoder_blocks = [HipPagedBlock(dim=dim, num_heads=H, mlp_ratio=4.0, init_values=1.0).to(dev, torch.bfloat16).eval()
+                      for _ in range(24)]
+    patch_embed = torch.nn.Conv2d(3, dim, kernel_size=14, stride=14).to(dev, torch.bfloat16).eval()
+    special = torch.randn(1, N_SPECIAL, dim, device=dev).to(torch.bfloat16)      # class + register tokens
     m = HipPagedKVCacheManager(blocks, ANCHOR + WINDOW + 16, T, H, D, torch.bfloat16, dev,
                                num_special_tokens=N_SPECIAL, scale_frames=ANCHOR, sliding_window=WINDOW,
                                max_total_frames=256, page_size=PAGE, layout="frame_pages")
     g = torch.Generator(device=dev).manual_seed(4)
     ang = torch.rand(1, 1, T, D // 2, generator=g, device=dev) * 6.283185
     freqs = torch.polar(torch.ones_like(ang), ang)
-    xs = [torch.randn(1, T, dim, generator=g, device=dev, dtype=torch.float32).to(torch.bfloat16) for _ in range(4)]
+    xs = [torch.rand(1, 3, 378, 518, generator=g, device=dev, dtype=torch.float32).to(torch.bfloat16) for _ in range(4)]
     # (y, x) of every token: specials at (0, 0), patches on the grid shifted by one (lingbot_map/aggregator/base.py:434-440)
     grid = torch.cartesian_prod(torch.arange(27, device=dev), torch.arange(37, device=dev)) + 1
     pos2d = torch.cat([torch.zeros(N_SPECIAL, 2, dtype=grid.dtype, device=dev), grid])[None].contiguous()
     assert pos2d.shape == (1, T, 2)
 
     @torch.no_grad()
-    def frame_x(x):
+    def frame_x(image):
+        x = torch.cat([special, patch_embed(image).flatten(2).transpose(1, 2)], dim=1)   # [1, 1004, 1024]
+        for blk in encoder_blocks:
+            x = blk(x)
         for b in range(blocks):
             x = frame_blocks[b](x, pos=pos2d)
             x = global_blocks[b](x, pos=freqs, enable_3d_rope=True, kv_cache=m, global_idx=b)
@@ -165,10 +174,10 @@ def aggregator_step(torch, blocks: int, steps: int, warmup: int) -> dict:
     assert torch.isfinite(out.float()).all() and m.device_header()["error"] == 0
     return {"value": 1.0 / dt, "unit": "frames/s", "ms_per_step": dt * 1e3, "steps": steps,
             "hip_graph": {"value": 1.0 / dt_graph, "unit": "frames/s", "ms_per_step": dt_graph * 1e3},
-            "what": f"{blocks} x (frame block + global block), dim {dim}, {H} heads, MLP {4 * dim}, 1 stream, "
-                    f"{T} tokens/frame, steady-state cache of {(ANCHOR + WINDOW) * T} KV tokens; eager PyTorch-ROCm "
-                    f"for linears/norms/GELU, HIP kernels for q/k norm + rotary + append, the cache path and "
-                    f"the frame blocks' dense attention"}
+            "what": f"patch embedding + 24 encoder blocks + {blocks} x (frame block + global block), dim {dim}, {H} heads, "
+                    f"MLP {4 * dim}, 1 stream, {T} tokens/frame, steady-state cache of {(ANCHOR + WINDOW) * T} KV tokens; "
+                    f"PyTorch-ROCm for linears / LayerNorm / GELU / convolution, HIP kernels for q/k norm + rotary + "
+                    f"append, the cache path and every block's cache-less attention; prediction heads excluded"}
 
 
 def main() -> None:
