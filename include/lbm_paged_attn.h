@@ -158,6 +158,17 @@ int lbm_kv_append(const void* k, const void* v, int32_t src_dtype, void* pool,
                   int32_t pool_dtype, const int32_t* append_rows, int32_t n_tokens,
                   int32_t num_heads, int32_t head_dim, int32_t page_size, void* stream);
 
+/* Residual update of a block fused with the LayerNorm that follows it, one pass over the rows:
+ *     x_out = x + y * gamma        (x + ls(y): block.py:283, layer_scale.py:21-22)
+ *     n_out = LayerNorm(x_out)     (norm2 in front of the MLP: block.py:194-195)
+ *   x, y, x_out, n_out  [rows][cols], dtype (bf16 or fp32); x_out may alias x
+ *   gamma               [cols] float32 LayerScale, NULL = plain x + y
+ *   norm_w, norm_b      [cols] float32, both NULL = no LayerNorm (n_out unused)
+ * cols: a multiple of 8, at most 8192.  Roundings follow torch's sequence for the dtype. */
+int lbm_residual_norm(const void* x, const void* y, int32_t dtype, const float* gamma,
+                      const float* norm_w, const float* norm_b, float norm_eps, void* x_out,
+                      void* n_out, int32_t rows, int32_t cols, void* stream);
+
 /* lbm_attn_run with the token counts read on the device: stream i attends to
  * live_kv_tokens[streams[i].live_at] entries of its row table instead of streams[i].kv_tokens,
  * which then only sizes the launch (number of KV splits, workspace) and should be the host's

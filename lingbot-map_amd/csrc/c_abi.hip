@@ -111,6 +111,17 @@ int lbm_qkv_prepare(const void* qkv, int32_t src_dtype, const float* q_norm_w, c
                                 (hipStream_t)stream);
 }
 
+int lbm_residual_norm(const void* x, const void* y, int32_t dtype, const float* gamma, const float* norm_w,
+                      const float* norm_b, float norm_eps, void* x_out, void* n_out, int32_t rows, int32_t cols,
+                      void* stream) {
+  if (!x || !y || !x_out) return lbm_fail(LBM_ERR_INVALID, "lbm_residual_norm: null x, y or x_out");
+  if (rows < 0 || cols <= 0) return lbm_fail(LBM_ERR_INVALID, "lbm_residual_norm: bad shape %d x %d", rows, cols);
+  if (dtype != LBM_DTYPE_BF16 && dtype != LBM_DTYPE_F32) return lbm_fail(LBM_ERR_INVALID, "lbm_residual_norm: unknown dtype");
+  if ((norm_w == nullptr) != (norm_b == nullptr)) return lbm_fail(LBM_ERR_INVALID, "lbm_residual_norm: norm_w and norm_b go together");
+  if (norm_w && !n_out) return lbm_fail(LBM_ERR_INVALID, "lbm_residual_norm: LayerNorm asked for without n_out");
+  return lbm_launch_residual_norm(x, y, dtype, gamma, norm_w, norm_b, norm_eps, x_out, n_out, rows, cols, (hipStream_t)stream);
+}
+
 static int lbm_check_attn_streams(const lbm_attn_stream* s, int n, const char* who) {
   if (!s) return lbm_fail(LBM_ERR_INVALID, "%s: null streams", who);
   if (n < 1 || n > LBM_MAX_STREAMS) return lbm_fail(LBM_ERR_INVALID, "%s: n_streams %d outside [1, %d]", who, n, LBM_MAX_STREAMS);

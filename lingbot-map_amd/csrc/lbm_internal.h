@@ -29,6 +29,10 @@ int lbm_launch_qkv_prepare(const void* qkv, int src_dtype, const float* q_norm_w
                            int dst_dtype, void* pool, const int32_t* append_rows, int n_tokens,
                            int num_heads, int page_size, hipStream_t stream);
 
+int lbm_launch_residual_norm(const void* x, const void* y, int dtype, const float* gamma, const float* norm_w,
+                             const float* norm_b, float eps, void* x_out, void* n_out, int rows, int cols,
+                             hipStream_t stream);
+
 // Split-KV schedule of one attention call, computed on the host from token counts only.
 struct LbmAttnStreamPlan {
   int32_t q_begin, q_rows, kv_row_begin, kv_tokens, live_at;

@@ -1,0 +1,150 @@
+// Residual update of a transformer block fused with the LayerNorm that follows it:
+//     x_out = x + y * gamma            (x + ls(y), lingbot_map/layers/block.py:283,
+//                                       lingbot_map/layers/layer_scale.py:21-22)
+//     n_out = LayerNorm(x_out)         (the block's norm2 in front of the MLP, block.py:194-195)
+// One pass over the rows instead of three elementwise / normalisation kernels.  HBM-bound:
+// reads x and y once, writes x_out and n_out once.
+//
+// One 128-thread workgroup per row; a thread owns 8 consecutive elements per 1024-element
+// chunk of the row (up to 8 chunks), kept in registers between the statistics and the output.
+// Rounding follows torch for bf16 activations: y * gamma rounded to bf16, the sum rounded to
+// bf16, the LayerNorm computed in fp32 on those bf16 values (two-pass mean / variance) and
+// rounded once.  For fp32 activations every step is a separately rounded fp32 operation.
+#include <hip/hip_runtime.h>
+#include "lbm_internal.h"
+
+typedef __attribute__((ext_vector_type(4))) unsigned int u32x4;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+
+namespace {
+
+constexpr int kThreads = 128;
+constexpr int kMaxChunks = 8;  // rows of up to 8192 elements
+
+__device__ __forceinline__ float round_bf16(float f) { return (float)(__bf16)f; }
+
+template <int DT>
+__device__ __forceinline__ void load8(const void* base, long long elem, float (&x)[8]) {
+  if (DT == 0) {
+    const u32x4 a = *(const u32x4*)((const unsigned short*)base + elem);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      x[2 * i] = __builtin_bit_cast(float, a[i] << 16);
+      x[2 * i + 1] = __builtin_bit_cast(float, a[i] & 0xffff0000u);
+    }
+  } else {
+    const f32x4* p = (const f32x4*)((const float*)base + elem);
+    const f32x4 a = p[0], b = p[1];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      x[i] = a[i];
+      x[4 + i] = b[i];
+    }
+  }
+}
+template <int DT>
+__device__ __forceinline__ void store8(void* base, long long elem, const float (&x)[8]) {
+  if (DT == 0) {
+    bf16x8 a;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) a[i] = (__bf16)x[i];
+    *(bf16x8*)((unsigned short*)base + elem) = a;
+  } else {
+    f32x4* p = (f32x4*)((float*)base + elem);
+    p[0] = f32x4{x[0], x[1], x[2], x[3]};
+    p[1] = f32x4{x[4], x[5], x[6], x[7]};
+  }
+}
+
+// sum over the 128 threads of the workgroup (two wavefronts)
+__device__ __forceinline__ float block_sum(float v, float* lds2) {
+#pragma unroll
+  for (int o = 32; o >= 1; o >>= 1) v += __shfl_xor(v, o);
+  const int wave = threadIdx.x >> 6;
+  __syncthreads();  // lds2 may still be read from the previous reduction
+  if ((threadIdx.x & 63) == 0) lds2[wave] = v;
+  __syncthreads();
+  return lds2[0] + lds2[1];
+}
+
+struct ResidualNormArgs {
+  const void* x;
+  const void* y;
+  const float* gamma;   // LayerScale, or NULL for x + y
+  const float* norm_w;  // NULL: no LayerNorm output
+  const float* norm_b;
+  void* x_out;
+  void* n_out;
+  float eps;
+  int rows, cols;
+};
+
+template <int DT>
+__global__ __launch_bounds__(kThreads) void lbm_residual_norm_kernel(ResidualNormArgs a) {
+  __shared__ float lds2[2];
+  const int row = blockIdx.x;
+  const long long base = (long long)row * a.cols;
+  const int n_chunks = (a.cols + 1023) >> 10;
+  float v[kMaxChunks][8];
+  float sum = 0.f;
+#pragma unroll
+  for (int c = 0; c < kMaxChunks; ++c) {
+    const int col = c * 1024 + threadIdx.x * 8;
+    if (c < n_chunks && col < a.cols) {
+      float x[8], y[8];
+      load8<DT>(a.x, base + col, x);
+      load8<DT>(a.y, base + col, y);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        float t = y[i];
+        if (a.gamma) t = DT == 0 ? round_bf16(__fmul_rn(t, a.gamma[col + i])) : __fmul_rn(t, a.gamma[col + i]);
+        const float s = __fadd_rn(x[i], t);
+        v[c][i] = DT == 0 ? round_bf16(s) : s;
+        sum += v[c][i];
+      }
+      store8<DT>(a.x_out, base + col, v[c]);
+    } else {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) v[c][i] = 0.f;
+    }
+  }
+  if (!a.norm_w) return;  // uniform: a launch parameter
+  const float mean = block_sum(sum, lds2) / (float)a.cols;
+  float sq = 0.f;
+#pragma unroll
+  for (int c = 0; c < kMaxChunks; ++c) {
+    const int col = c * 1024 + threadIdx.x * 8;
+    if (c < n_chunks && col < a.cols) {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) sq += (v[c][i] - mean) * (v[c][i] - mean);
+    }
+  }
+  const float rstd = __builtin_amdgcn_rsqf(block_sum(sq, lds2) / (float)a.cols + a.eps);
+#pragma unroll
+  for (int c = 0; c < kMaxChunks; ++c) {
+    const int col = c * 1024 + threadIdx.x * 8;
+    if (c < n_chunks && col < a.cols) {
+      float o[8];
+#pragma unroll
+      for (int i = 0; i < 8; ++i)
+        o[i] = __fadd_rn(__fmul_rn(__fmul_rn(v[c][i] - mean, rstd), a.norm_w[col + i]), a.norm_b[col + i]);
+      store8<DT>(a.n_out, base + col, o);
+    }
+  }
+}
+
+}  // namespace
+
+int lbm_launch_residual_norm(const void* x, const void* y, int dtype, const float* gamma, const float* norm_w,
+                             const float* norm_b, float eps, void* x_out, void* n_out, int rows, int cols,
+                             hipStream_t stream) {
+  if (rows == 0) return LBM_OK;
+  if (cols % 8 != 0 || cols > 1024 * kMaxChunks)
+    return lbm_fail(LBM_ERR_UNSUPPORTED, "lbm_residual_norm: cols must be a multiple of 8 and at most %d (got %d)",
+                    1024 * kMaxChunks, cols);
+  ResidualNormArgs a{x, y, gamma, norm_w, norm_b, x_out, n_out, eps, rows, cols};
+  if (dtype == LBM_DTYPE_BF16) hipLaunchKernelGGL(lbm_residual_norm_kernel<0>, dim3(rows), dim3(kThreads), 0, stream, a);
+  else hipLaunchKernelGGL(lbm_residual_norm_kernel<1>, dim3(rows), dim3(kThreads), 0, stream, a);
+  return lbm_check_launch("lbm_residual_norm_kernel");
+}

@@ -40,7 +40,7 @@ class AttnStream(C.Structure):
 
 
 SYMBOLS = ("lbm_abi_version", "lbm_last_error", "lbm_tables_words", "lbm_tables_step",
-           "lbm_rows_from_pages", "lbm_kv_append", "lbm_qkv_prepare", "lbm_attn_workspace_bytes", "lbm_attn_run", "lbm_attn_run_live")
+           "lbm_rows_from_pages", "lbm_kv_append", "lbm_qkv_prepare", "lbm_residual_norm", "lbm_attn_workspace_bytes", "lbm_attn_run", "lbm_attn_run_live")
 
 
 def _load():
@@ -62,6 +62,8 @@ def _load():
     lib.lbm_kv_append.argtypes = [vp, vp, i32, vp, i32, vp, i32, i32, i32, i32, vp]
     lib.lbm_qkv_prepare.restype = C.c_int
     lib.lbm_qkv_prepare.argtypes = [vp, i32, vp, vp, vp, vp, C.c_float, vp, i32, vp, vp, vp, i32, vp, vp, i32, i32, i32, i32, vp]
+    lib.lbm_residual_norm.restype = C.c_int
+    lib.lbm_residual_norm.argtypes = [vp, vp, i32, vp, vp, vp, C.c_float, vp, vp, i32, i32, vp]
     lib.lbm_attn_workspace_bytes.restype = C.c_size_t
     lib.lbm_attn_workspace_bytes.argtypes = [p(AttnStream), i32, i32, i32]
     lib.lbm_attn_run.restype = C.c_int

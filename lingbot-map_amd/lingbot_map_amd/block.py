@@ -342,6 +342,46 @@ class HipPagedBlock(nn.Module):
         self.drop_path2 = nn.Identity()
         self.sample_drop_ratio = drop_path
 
+    # ------------------------------------------------------------------ fused residual path
+    def _f32(self, t: Tensor) -> Tensor:
+        """float32 copy of a parameter, cached until the parameter changes."""
+        cache = self.__dict__.setdefault("_f32_cache", {})
+        key = (t._version, t.data_ptr(), t.device)
+        hit = cache.get(id(t))
+        if hit is None or hit[0] != key:
+            cache[id(t)] = hit = (key, t.detach().float().contiguous())
+        return hit[1]
+
+    def _can_fuse_residual(self, x: Tensor) -> bool:
+        return (x.is_cuda and x.dtype in (torch.bfloat16, torch.float32) and x.shape[-1] % 8 == 0
+                and x.shape[-1] <= 8192 and type(self.norm2) is nn.LayerNorm and self.norm2.elementwise_affine
+                and self.norm2.bias is not None and isinstance(self.ls1, (LayerScale, nn.Identity))
+                and isinstance(self.ls2, (LayerScale, nn.Identity)) and not torch.is_grad_enabled())
+
+    def _residual(self, x: Tensor, y: Tensor, ls, norm: Optional[nn.LayerNorm]):
+        """x + ls(y) and, when ``norm`` is given, norm(x + ls(y)), in one kernel (block.py:283 and
+        :194-195; layer_scale.py:21-22)."""
+        import ctypes as C
+        from . import _native as N
+        x, y = x.contiguous(), y.contiguous().to(x.dtype)
+        x_out = torch.empty_like(x)
+        n_out = torch.empty_like(x) if norm is not None else None
+        p = lambda t: None if t is None else C.c_void_p(t.data_ptr())
+        gamma = self._f32(ls.gamma) if isinstance(ls, LayerScale) else None
+        w, b = (self._f32(norm.weight), self._f32(norm.bias)) if norm is not None else (None, None)
+        N.check(N.lib.lbm_residual_norm(
+            p(x), p(y), N.DTYPE_BF16 if x.dtype == torch.bfloat16 else N.DTYPE_F32, p(gamma), p(w), p(b),
+            float(norm.eps) if norm is not None else 0.0, p(x_out), p(n_out), x.numel() // x.shape[-1], x.shape[-1],
+            C.c_void_p(torch.cuda.current_stream(x.device).cuda_stream)))
+        return x_out, n_out
+
+    def _finish(self, x: Tensor, attn_out: Tensor) -> Tensor:
+        """x + ls1(attn_out), then the MLP branch (block.py:283-285)."""
+        if self._can_fuse_residual(x):
+            x, n = self._residual(x, attn_out, self.ls1, self.norm2)
+            return self._residual(x, self.mlp(n), self.ls2, None)[0]
+        return self.ffn_residual(x + self.ls1(attn_out))
+
     def attn_pre(self, x: Tensor, pos=None, enable_3d_rope: bool = False):
         """norm1 + projections + qk-norm + RoPE, ready for the cache (block.py:217-227)."""
         return self.attn.prepare_qkv(self.norm1(x), pos=pos, enable_3d_rope=enable_3d_rope)
@@ -360,14 +400,12 @@ class HipPagedBlock(nn.Module):
                 q, k, v = self.attn_pre(x, pos=pos, enable_3d_rope=enable_3d_rope)
                 attn_x = self.attn.stream_attend(kv_cache, global_idx, q, k, v, num_register_tokens)
             attn_x = attn_x.reshape(x.shape[0], x.shape[1], self.attn.num_heads * self.attn.head_dim).to(x.dtype)
-            x = x + self.ls1(self.attn.proj(attn_x))
-        else:
-            x = x + self.ls1(self.attn(
-                self.norm1(x), pos=pos, num_patches=num_patches, num_special=num_special, num_frames=num_frames,
-                enable_3d_rope=enable_3d_rope, kv_cache=kv_cache, global_idx=global_idx,
-                num_frame_per_block=num_frame_per_block, num_frame_for_scale=num_frame_for_scale,
-                num_register_tokens=num_register_tokens))
-        return self.ffn_residual(x)
+            return self._finish(x, self.attn.proj(attn_x))
+        return self._finish(x, self.attn(
+            self.norm1(x), pos=pos, num_patches=num_patches, num_special=num_special, num_frames=num_frames,
+            enable_3d_rope=enable_3d_rope, kv_cache=kv_cache, global_idx=global_idx,
+            num_frame_per_block=num_frame_per_block, num_frame_for_scale=num_frame_for_scale,
+            num_register_tokens=num_register_tokens))
 
 
 def keyframe_flags(num_frames: int, scale_frames: int, keyframe_interval: int):

@@ -183,3 +183,41 @@ def test_prepare_half_split_rope_matches_oracle(dtype):
         rq, rk, _ = prepare_qkv(qkv, H, D, None, None, None, positions=pos)
         q, k, _ = run_prepare(qkv, H, D, None, None, None, dtype, table=table)
         assert torch.equal(q.cpu(), rq) and torch.equal(k.cpu(), rk)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("rows,C", [(3, 256), (1004, 1024), (17, 2048 + 8)])
+def test_residual_norm_matches_oracle(dtype, rows, C):
+    """x + y * gamma and the LayerNorm of it in one kernel.  bf16: x_out bit-exact (products and
+    sums rounded where torch rounds them), the LayerNorm within one bf16 ulp; fp32: 2e-6."""
+    from oracle.block_ops import residual_norm
+    N = _native()
+    dev = torch.device("cuda:0")
+    g = torch.Generator().manual_seed(rows + C)
+    x, y = (torch.randn(rows, C, generator=g).to(dtype) for _ in range(2))
+    gamma = (0.1 * torch.randn(C, generator=g)).to(dtype)
+    w, b = (1 + 0.2 * torch.randn(C, generator=g)).to(dtype), (0.1 * torch.randn(C, generator=g)).to(dtype)
+    rx, rn = residual_norm(x, y, gamma, w, b, 1e-5)
+    dt = N.DTYPE_BF16 if dtype == torch.bfloat16 else N.DTYPE_F32
+    xd, yd = x.to(dev), y.to(dev)
+    f32 = [t.float().to(dev) for t in (gamma, w, b)]
+    xo, no = torch.full_like(xd, float("nan")), torch.full_like(xd, float("nan"))
+    N.check(N.lib.lbm_residual_norm(ptr(xd), ptr(yd), dt, ptr(f32[0]), ptr(f32[1]), ptr(f32[2]), 1e-5, ptr(xo), ptr(no),
+                                    rows, C, None))
+    torch.cuda.synchronize()
+    if dtype == torch.bfloat16:
+        assert torch.equal(xo.cpu(), rx)
+    else:
+        assert ((xo.cpu() - rx).abs() / rx.abs().clamp_min(1.0)).max().item() <= 2e-6
+    _close(no, rn, dtype) if dtype == torch.float32 else None
+    if dtype == torch.bfloat16:
+        rel = (no.float().cpu() - rn.float()).abs() / rn.float().abs().clamp_min(1.0)
+        assert rel.max().item() <= 2 ** -7 and (no.cpu() != rn).float().mean().item() < 2e-3
+    # without LayerScale and without LayerNorm: x + y, in place
+    rx2, _ = residual_norm(x, y, None)
+    N.check(N.lib.lbm_residual_norm(ptr(xd), ptr(yd), dt, None, None, None, 0.0, ptr(xd), None, rows, C, None))
+    torch.cuda.synchronize()
+    assert torch.equal(xd.cpu(), rx2) if dtype == torch.bfloat16 else ((xd.cpu() - rx2).abs().max().item() <= 1e-6)
+    # argument checks
+    assert N.lib.lbm_residual_norm(ptr(xd), ptr(yd), dt, None, ptr(f32[1]), None, 0.0, ptr(xd), None, rows, C, None) != N.OK
+    assert N.lib.lbm_residual_norm(ptr(xd), ptr(yd), dt, None, None, None, 0.0, ptr(xd), None, rows, 12, None) != N.OK

@@ -105,3 +105,23 @@ def test_rope2d_identity_explicit_rotation_and_separation():
     only_y = pos.clone(); only_y[..., 1] = 0
     assert torch.equal(rope2d(x, only_y)[..., :32], y[..., :32])
     assert torch.equal(rope2d(x, only_y)[..., 32:], x[..., 32:])
+
+
+def test_residual_norm_closed_forms_and_float64_restatement():
+    from oracle.block_ops import residual_norm
+    g = torch.Generator().manual_seed(9)
+    rows, C = 5, 1024
+    x, y = torch.randn(rows, C, generator=g), torch.randn(rows, C, generator=g)
+    gamma, w, b = torch.randn(C, generator=g), torch.randn(C, generator=g), torch.randn(C, generator=g)
+    assert torch.equal(residual_norm(x, y, torch.zeros(C))[0], x)
+    assert torch.equal(residual_norm(x, y, torch.ones(C))[0], x + y)
+    assert torch.equal(residual_norm(x, y, None)[0], x + y)
+    xn, n = residual_norm(x, y, gamma, w, b, 1e-5)
+    want = x.double() + y.double() * gamma.double()
+    assert (xn.double() - want).abs().max().item() < 1e-6
+    mean = want.mean(-1, keepdim=True)
+    var = ((want - mean) ** 2).mean(-1, keepdim=True)
+    assert (n.double() - ((want - mean) / torch.sqrt(var + 1e-5) * w.double() + b.double())).abs().max().item() < 1e-5
+    # an update that makes the row constant: the LayerNorm is the bias
+    _, n = residual_norm(x, 3.0 - x, torch.ones(C), w, b, 1e-5)
+    assert (n - b).abs().max().item() < 2e-3     # (x + (3 - x)) is 3 up to fp32 rounding of the sum
