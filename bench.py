@@ -189,8 +189,8 @@ def main() -> None:
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-aggregator", action="store_true",
                     help="skip the full aggregator-trunk step (frame + global blocks) timed after the hot path")
-    ap.add_argument("--mode", choices=["full", "attention", "append", "prepare", "tables", "copy"], default="full",
-                    help="full = the benchmark line; attention/append/prepare/tables launch one kernel --steps "
+    ap.add_argument("--mode", choices=["full", "attention", "append", "prepare", "residual", "tables", "copy"], default="full",
+                    help="full = the benchmark line; attention/append/prepare/residual/tables launch one kernel --steps "
                          "times on the steady-state cache (for rocprofv3 runs); copy = a plain 256 MiB "
                          "device copy, the known-size kernel the HBM counters are calibrated on")
     args = ap.parse_args()
@@ -236,6 +236,19 @@ def main() -> None:
                                       vp(rope_cs), N.ROPE_INTERLEAVED, vp(q_tmp), None, None, N.DTYPE_BF16, vp(m.kv_caches[block]),
                                       vp(m._append_rows[0]), T, H, D, PAGE, m._stream_handle()))
 
+    # inputs of the fused residual update + LayerNorm (one frame of the 1024-wide trunk)
+    res_x = torch.randn(T, H * D, generator=g, device=dev, dtype=torch.float32).to(torch.bfloat16)
+    res_y = torch.randn(T, H * D, generator=g, device=dev, dtype=torch.float32).to(torch.bfloat16)
+    res_p = [torch.rand(H * D, generator=g, device=dev) + 0.5 for _ in range(3)]
+    res_o = [torch.empty_like(res_x) for _ in range(2)]
+
+    def residual() -> None:
+        from lingbot_map_amd import _native as N
+        import ctypes as C
+        vp = lambda t: C.c_void_p(t.data_ptr())
+        N.check(N.lib.lbm_residual_norm(vp(res_x), vp(res_y), N.DTYPE_BF16, vp(res_p[0]), vp(res_p[1]), vp(res_p[2]), 1e-5,
+                                        vp(res_o[0]), vp(res_o[1]), T, H * D, m._stream_handle()))
+
     def frame(i: int) -> None:
         for b in range(blocks):
             j = (i + b) % n_sets
@@ -256,6 +269,7 @@ def main() -> None:
         fn = {"attention": lambda: m._attend_planned(1, qs[0], None, None),
               "append": lambda: m._scatter(1, 0, ks[0], vs[0]),
               "prepare": lambda: prepare(1),
+              "residual": residual,
               "tables": lambda: m._tables_step(0, ops, kv_rows=True)}[args.mode]
         for _ in range(args.warmup):
             fn()
@@ -289,6 +303,9 @@ def main() -> None:
     prepare_ms = kernel_time_ms(lambda: prepare(1), 100, torch)
     prepare_bytes = (3 + 3) * T * H * D * 2 + rope_cs.numel() * 4   # read qkv, write q and the K/V rows, read the table
     prepare_gbps = prepare_bytes / (prepare_ms * 1e-3) * 1e-9
+    residual_ms = kernel_time_ms(residual, 100, torch)
+    residual_bytes = 4 * T * H * D * 2    # read x and y, write x_out and the LayerNorm output
+    residual_gbps = residual_bytes / (residual_ms * 1e-3) * 1e-9
 
     line = {
         "metric": METRIC, "value": fps, "unit": "frames/s", "n_gpus": 1, "steps": args.steps,
@@ -311,6 +328,10 @@ def main() -> None:
                         "avg_launch_us": prepare_ms * 1e3,
                         "what": "fused q/k LayerNorm + rotary + layout + paged append (replaces the append pass "
                                 "when the block feeds the qkv projection output; not in `value`'s timed loop)"},
+        "residual_norm": {"bound": "hbm", "achieved": residual_gbps, "peak": PEAK_HBM_GBPS, "unit": "GB/s",
+                          "frac": residual_gbps / PEAK_HBM_GBPS, "bytes_per_launch": residual_bytes,
+                          "avg_launch_us": residual_ms * 1e3,
+                          "what": "x + ls(y) fused with the following LayerNorm, 1004 x 1024 bf16 (not in `value`'s timed loop)"},
         "tables_step_us": tables_ms * 1e3,
     }
     if not args.no_aggregator:
