@@ -111,7 +111,8 @@ def aggregator_step(torch, blocks: int, steps: int, warmup: int) -> dict:
     cache path, every block's pre-attention producer and cache-less attention are HIP kernels
     too; linears, LayerNorm, GELU and the patch-embedding convolution are PyTorch-ROCm library
     calls.  The prediction heads are not part of the step."""
-    from lingbot_map_amd import HipPagedBlock, HipPagedKVCacheManager, RotaryPositionEmbedding2D
+    from lingbot_map_amd import (HipPagedBlock, HipPagedKVCacheManager, PositionGetter, RotaryPositionEmbedding2D,
+                                 RotaryPositionEmbedding3D)
     dev = torch.device("cuda:0")
     dim = H * D
     torch.manual_seed(4)
@@ -130,11 +131,13 @@ def aggregator_step(torch, blocks: int, steps: int, warmup: int) -> dict:
                                num_special_tokens=N_SPECIAL, scale_frames=ANCHOR, sliding_window=WINDOW,
                                max_total_frames=256, page_size=PAGE, layout="frame_pages")
     g = torch.Generator(device=dev).manual_seed(4)
-    ang = torch.rand(1, 1, T, D // 2, generator=g, device=dev) * 6.283185
-    freqs = torch.polar(torch.ones_like(ang), ang)
+    # rotary table of the global blocks for frame 40 of a stream (frame / row / column pairs 10 / 11 / 11)
+    rope3d = RotaryPositionEmbedding3D(attention_head_dim=D, patch_size=(1, 14, 14), max_seq_len=1024)
+    freqs = rope3d(ppf=1, pph=27, ppw=37, patch_start_idx=N_SPECIAL, device=dev, f_start=40, f_end=41)
+    assert freqs.shape == (1, 1, T, D // 2)
     xs = [torch.rand(1, 3, 378, 518, generator=g, device=dev, dtype=torch.float32).to(torch.bfloat16) for _ in range(4)]
     # (y, x) of every token: specials at (0, 0), patches on the grid shifted by one (lingbot_map/aggregator/base.py:434-440)
-    grid = torch.cartesian_prod(torch.arange(27, device=dev), torch.arange(37, device=dev)) + 1
+    grid = PositionGetter()(1, 27, 37, dev)[0] + 1
     pos2d = torch.cat([torch.zeros(N_SPECIAL, 2, dtype=grid.dtype, device=dev), grid])[None].contiguous()
     assert pos2d.shape == (1, T, 2)
 

@@ -6,10 +6,12 @@
 if it has not been built: there is no CPU path.
 """
 from . import _native  # noqa: F401  (loads the library, fails loudly when missing)
-from .block import HipPagedAttention, HipPagedBlock, RotaryPositionEmbedding2D, keyframe_flags, set_skip_append
+from .block import (HipPagedAttention, HipPagedBlock, PositionGetter, RotaryPositionEmbedding2D,
+                    RotaryPositionEmbedding3D, WanRotaryPosEmbed, keyframe_flags, set_skip_append)
 from .dense import dense_attention
 from .graph import GraphedFrame
 from .manager import HipPagedKVCacheManager
 
 __all__ = ["HipPagedKVCacheManager", "HipPagedAttention", "HipPagedBlock", "RotaryPositionEmbedding2D",
+           "RotaryPositionEmbedding3D", "WanRotaryPosEmbed", "PositionGetter",
            "dense_attention", "GraphedFrame", "keyframe_flags", "set_skip_append"]

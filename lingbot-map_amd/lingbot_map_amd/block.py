@@ -96,6 +96,93 @@ class RotaryPositionEmbedding2D(nn.Module):
         return table
 
 
+class PositionGetter:
+    """(y, x) grid coordinates of a frame's patches, ``[B, height * width, 2]`` int64, row-major
+    (lingbot_map/layers/rope.py:26-61).  One grid per (height, width, device) is kept."""
+
+    def __init__(self) -> None:
+        self.position_cache = {}
+
+    def __call__(self, batch_size: int, height: int, width: int, device) -> Tensor:
+        key = (height, width, torch.device(device))
+        if key not in self.position_cache:
+            idx = torch.arange(height * width, device=device)
+            self.position_cache[key] = torch.stack((idx // width, idx % width), dim=-1)
+        return self.position_cache[key].view(1, height * width, 2).expand(batch_size, -1, -1).clone()
+
+
+class RotaryPositionEmbedding3D(nn.Module):
+    """Complex rotary table of the global blocks (the reference's ``WanRotaryPosEmbed``,
+    lingbot_map/layers/rope.py:279-432): the ``head_dim / 2`` interleaved pairs are dealt to
+    the frame, row and column axes (10 / 11 / 11 pairs for head_dim 64) and pair j of an axis
+    that owns ``dim`` elements rotates by ``coordinate * theta^(-2j/dim)``.  Special token i of
+    frame f sits at (f, i, i); patch (y, x) at (f, n_special + y, n_special + x), or at
+    (f, y, x) when there are no special tokens.  Frames count from ``f_start``.
+
+    The reference precomputes ``exp(i * pos * freq)`` for every position below ``max_seq_len``
+    and assembles a frame's table by slicing, expanding and concatenating; here each token's
+    three integer coordinates are written down and the angles are one float64 product, which
+    gives the same complex128 values and has no table to keep on the device."""
+
+    def __init__(self, attention_head_dim: int, patch_size=(1, 14, 14), max_seq_len: int = 1024,
+                 theta: float = 10000.0, fhw_dim=(20, 22, 22)) -> None:
+        super().__init__()
+        self.attention_head_dim = attention_head_dim
+        self.patch_size = patch_size
+        self.max_seq_len = max_seq_len
+        self.theta = theta
+        if fhw_dim is not None:
+            assert attention_head_dim == sum(fhw_dim), \
+                f"attention_head_dim {attention_head_dim} must match sum(fhw_dim) {sum(fhw_dim)}"
+            t_dim, h_dim, w_dim = fhw_dim
+        else:
+            h_dim = w_dim = 2 * (attention_head_dim // 6)
+            t_dim = attention_head_dim - h_dim - w_dim
+        assert t_dim % 2 == 0 and h_dim % 2 == 0 and w_dim % 2 == 0, "every axis owns whole pairs"
+        self.fhw_dim = (t_dim, h_dim, w_dim)
+        inv_freq, axis = [], []
+        for a, dim in enumerate(self.fhw_dim):
+            inv_freq.append(1.0 / (theta ** (torch.arange(0, dim, 2, dtype=torch.float64) / dim)))
+            axis.append(torch.full((dim // 2,), a, dtype=torch.int64))
+        self.register_buffer("inv_freq", torch.cat(inv_freq), persistent=False)   # [D/2] float64
+        self.register_buffer("pair_axis", torch.cat(axis), persistent=False)      # [D/2] in {0, 1, 2}
+
+    def coordinates(self, ppf: int, pph: int, ppw: int, patch_start_idx: int, device,
+                    f_start: int = 0, f_end: Optional[int] = None) -> Tensor:
+        """int64 ``[frames * (patch_start_idx + pph * ppw), 3]``: (frame, row, column) per token,
+        specials first within each frame."""
+        if f_end is not None:
+            ppf = f_end - f_start
+        else:
+            f_start = 0
+        assert 0 <= f_start and f_start + ppf <= self.max_seq_len, \
+            f"frames [{f_start}, {f_start + ppf}) outside the {self.max_seq_len} positions of the table"
+        assert patch_start_idx + max(pph, ppw) <= self.max_seq_len
+        special = torch.arange(patch_start_idx, device=device)
+        grid = torch.arange(pph * ppw, device=device)
+        row = torch.cat((special, patch_start_idx + grid // ppw))
+        col = torch.cat((special, patch_start_idx + grid % ppw))
+        frame = torch.arange(f_start, f_start + ppf, device=device)
+        n = row.numel()
+        return torch.stack((frame[:, None].expand(ppf, n), row[None].expand(ppf, n), col[None].expand(ppf, n)),
+                           dim=-1).reshape(ppf * n, 3)
+
+    def angles(self, coords: Tensor) -> Tensor:
+        """float64 ``[N, D/2]`` rotation angle of every pair."""
+        inv_freq = self.inv_freq.to(coords.device)
+        return coords.to(torch.float64)[:, self.pair_axis.to(coords.device)] * inv_freq
+
+    def forward(self, ppf: int, pph: int, ppw: int, patch_start_idx: int, device,
+                f_start: int = 0, f_end: Optional[int] = None) -> Tensor:
+        """complex128 ``[1, 1, N, D/2]``, the argument ``pos`` of a global block with
+        ``enable_3d_rope=True``."""
+        ang = self.angles(self.coordinates(ppf, pph, ppw, patch_start_idx, device, f_start, f_end))
+        return torch.polar(torch.ones_like(ang), ang)[None, None]
+
+
+WanRotaryPosEmbed = RotaryPositionEmbedding3D   # the reference's name for it
+
+
 class LayerScale(nn.Module):
     """lingbot_map/layers/layer_scale.py"""
 

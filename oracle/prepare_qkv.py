@@ -16,6 +16,12 @@ Restated from the reference (paths relative to its checkout):
   angle table pos * base^(-2j/dim) repeated twice, computed and cast in the activations' dtype
                                            lingbot_map/layers/rope.py:86-198
 
+* complex table of the global blocks' 3-D rotary embedding: one 1-D table
+  exp(i * pos * theta^(-2j/dim)) per axis in float64, concatenated along the pair axis, then
+  sliced per axis (frames f_start..f_end, rows and columns offset by the number of special
+  tokens, special token i at row i and column i), expanded and concatenated per frame
+                                           lingbot_map/layers/rope.py:202-276, :279-432
+
 ``prepare_qkv`` runs the same torch operations in the same order and dtype as the reference,
 so for bf16 activations every intermediate is rounded where the reference rounds it
 (LayerNorm output, cos, sin, each product, each sum).
@@ -28,6 +34,10 @@ constant row is the bias and otherwise equals a float64 restatement of
 transpose the reference's permutes describe.  ``rope2d``: position (0, 0) is the identity; in
 float64 element j of a half and element j + dim/4 rotate by pos * base^(-4j/dim) (an explicit
 loop restates it), pair norms are kept, the vertical half ignores x and the horizontal half y.
+``rope3d_freqs``: every entry has modulus 1; the entry of a named token and pair equals
+exp(i * coordinate * theta^(-2j/dim)) written out by hand for the camera token, a register
+token and two patches; shifting f_start changes the frame pairs only; frame 0 of a two-frame
+table equals the one-frame table; without special tokens the patch grid starts at (0, 0).
 """
 
 from __future__ import annotations
@@ -76,6 +86,38 @@ def rope2d(tokens: torch.Tensor, positions: torch.Tensor, base: float = 100.0) -
 
     vert, horiz = tokens.chunk(2, dim=-1)
     return torch.cat((one(vert, positions[..., 0]), one(horiz, positions[..., 1])), dim=-1)
+
+
+def rope3d_axis_table(dim: int, n_pos: int, theta: float = 10000.0) -> torch.Tensor:
+    """complex128 ``[n_pos, dim / 2]`` of one axis (rope.py:202-276 with freqs_dtype float64)."""
+    freqs = 1.0 / (theta ** (torch.arange(0, dim, 2, dtype=torch.float64)[: dim // 2] / dim))
+    ang = torch.outer(torch.arange(n_pos), freqs)
+    return torch.polar(torch.ones_like(ang), ang)
+
+
+def rope3d_freqs(ppf: int, pph: int, ppw: int, patch_start_idx: int, head_dim: int = 64,
+                 fhw_dim=(20, 22, 22), max_seq_len: int = 1024, theta: float = 10000.0,
+                 f_start: int = 0, f_end: Optional[int] = None) -> torch.Tensor:
+    """complex128 ``[1, 1, frames * (patch_start_idx + pph * ppw), head_dim / 2]``
+    (rope.py:299-432)."""
+    assert sum(fhw_dim) == head_dim
+    tab_f, tab_h, tab_w = (rope3d_axis_table(d, max_seq_len, theta) for d in fhw_dim)
+    if f_end is not None:
+        ppf = f_end - f_start
+        tab_f = tab_f[f_start:f_end]
+    else:
+        tab_f = tab_f[:ppf]
+    s = patch_start_idx
+    per_frame = []
+    if s > 0:
+        per_frame.append(torch.cat((tab_f.reshape(ppf, 1, -1).expand(ppf, s, -1),
+                                    tab_h[:s].reshape(1, s, -1).expand(ppf, s, -1),
+                                    tab_w[:s].reshape(1, s, -1).expand(ppf, s, -1)), dim=-1))
+    patches = torch.cat((tab_f.reshape(ppf, 1, 1, -1).expand(ppf, pph, ppw, -1),
+                         tab_h[s:s + pph].reshape(1, pph, 1, -1).expand(ppf, pph, ppw, -1),
+                         tab_w[s:s + ppw].reshape(1, 1, ppw, -1).expand(ppf, pph, ppw, -1)), dim=-1)
+    per_frame.append(patches.reshape(ppf, pph * ppw, -1))
+    return torch.cat(per_frame, dim=1).reshape(1, 1, ppf * (s + pph * ppw), -1)
 
 
 def prepare_qkv(qkv: torch.Tensor, num_heads: int, head_dim: int,

@@ -1,6 +1,7 @@
 """Call surface of the block that stands in for the reference's FlashInferBlock (CPU only):
 parameter names a reference state dict carries, the attributes the reference's compile
 recipe reaches into, batch mode without a cache, and the driver's keyframe rule."""
+import pytest
 import torch
 
 
@@ -81,3 +82,25 @@ def test_rope2d_module_equals_the_oracle_and_its_table():
         cos, sin = table[..., 0].to(dtype)[:, None], table[..., 1].to(dtype)[:, None]
         rot = torch.cat((-x[..., 16:32], x[..., :16], -x[..., 48:], x[..., 32:48]), -1)
         assert torch.equal(x * cos + rot * sin, rope(x, pos))
+
+
+def test_rope3d_module_equals_the_oracle_table():
+    """The coordinate-based table against the oracle's slice-and-concatenate restatement."""
+    from lingbot_map_amd import PositionGetter, RotaryPositionEmbedding3D, WanRotaryPosEmbed
+    from oracle.prepare_qkv import rope3d_freqs
+    assert WanRotaryPosEmbed is RotaryPositionEmbedding3D
+    m = RotaryPositionEmbedding3D(attention_head_dim=64, patch_size=(1, 14, 14), max_seq_len=512)
+    assert m.fhw_dim == (20, 22, 22) and not list(m.state_dict())
+    for kw in (dict(ppf=1, pph=27, ppw=37, patch_start_idx=6), dict(ppf=3, pph=5, ppw=4, patch_start_idx=6),
+               dict(ppf=1, pph=27, ppw=37, patch_start_idx=6, f_start=100, f_end=101),
+               dict(ppf=9, pph=3, ppw=7, patch_start_idx=0), dict(ppf=2, pph=2, ppw=2, patch_start_idx=5, f_start=3, f_end=7)):
+        got = m(device="cpu", **kw)
+        want = rope3d_freqs(head_dim=64, max_seq_len=512, **kw)
+        assert got.dtype == want.dtype and got.shape == want.shape
+        assert (got - want).abs().max().item() < 1e-13, kw
+    auto = RotaryPositionEmbedding3D(attention_head_dim=128, fhw_dim=None)
+    assert auto.fhw_dim == (44, 42, 42)
+    with pytest.raises(AssertionError):
+        m(ppf=1, pph=2, ppw=2, patch_start_idx=0, device="cpu", f_start=511, f_end=513)
+    pos = PositionGetter()(2, 3, 4, "cpu")
+    assert pos.shape == (2, 12, 2) and pos[1, 7].tolist() == [1, 3] and pos[0, 11].tolist() == [2, 3]

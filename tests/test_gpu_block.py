@@ -25,10 +25,13 @@ class ReferenceSurfaceOnly:
 @pytest.mark.parametrize("reference_calls,rope", [(False, False), (True, False), (False, True), (True, True)])
 def test_block_stream_matches_dense_cache(reference_calls, rope):
     """reference_calls=False takes the fused producer + `step_qkv`; True the reference's own
-    method sequence.  rope=True adds the interleaved-pair rotary embedding of the global blocks."""
-    from lingbot_map_amd import HipPagedBlock, HipPagedKVCacheManager, keyframe_flags, set_skip_append
+    method sequence.  rope=True adds the global blocks' 3-D rotary embedding (interleaved pairs,
+    complex table per frame)."""
+    from lingbot_map_amd import (HipPagedBlock, HipPagedKVCacheManager, RotaryPositionEmbedding3D, keyframe_flags,
+                                 set_skip_append)
     from oracle.sdpa_cache import DictCacheOracle
     torch.manual_seed(5)
+    rope3d = RotaryPositionEmbedding3D(attention_head_dim=64)
     dev = torch.device("cuda:0")
     dim, H, T, n_sp, scale, window, blocks = 256, 4, 53, 5, 1, 3, 2
     mods = [HipPagedBlock(dim, H, init_values=0.1, qk_norm=True, rope=True if rope else None,
@@ -48,9 +51,9 @@ def test_block_stream_matches_dense_cache(reference_calls, rope):
         for f, kf in enumerate(flags):
             x = torch.randn(1, T, dim, device=dev).to(torch.bfloat16)
             pos = None
-            if rope:
-                ang = torch.rand(1, 1, T, 32, device=dev) * 6.283185
-                pos = torch.polar(torch.ones_like(ang), ang)
+            if rope:   # complex128 table of frame f: 5 special tokens + a 6 x 8 patch grid
+                pos = rope3d(ppf=1, pph=6, ppw=8, patch_start_idx=n_sp, device=dev, f_start=f, f_end=f + 1)
+                assert pos.shape == (1, 1, T, 32) and pos.dtype == torch.complex128
             set_skip_append(cache, not kf)
             y, y_ref = x, x
             for b, mod in enumerate(mods):

@@ -125,3 +125,42 @@ def test_residual_norm_closed_forms_and_float64_restatement():
     # an update that makes the row constant: the LayerNorm is the bias
     _, n = residual_norm(x, 3.0 - x, torch.ones(C), w, b, 1e-5)
     assert (n - b).abs().max().item() < 2e-3     # (x + (3 - x)) is 3 up to fp32 rounding of the sum
+
+
+def test_rope3d_table_hand_written_entries_and_structure():
+    """518x378 frames: 27 x 37 patches after 6 special tokens; pairs 0-9 follow the frame,
+    10-20 the row, 21-31 the column; each entry is exp(i * coordinate * 10000^(-2j/dim))."""
+    from oracle.prepare_qkv import rope3d_freqs
+    pph, ppw, s = 27, 37, 6
+    n = s + pph * ppw
+    t = rope3d_freqs(2, pph, ppw, s, f_start=40, f_end=42)
+    assert t.shape == (1, 1, 2 * n, 32) and t.dtype == torch.complex128
+    assert (t.abs() - 1).abs().max().item() < 1e-15
+
+    def expect(coord, j, dim):
+        a = coord * 10000.0 ** (-2.0 * j / dim)
+        return complex(math.cos(a), math.sin(a))
+
+    def close(z, w):
+        return abs(complex(z) - w) < 1e-12
+
+    cam0 = t[0, 0, 0]                       # camera token of frame 40: (40, 0, 0)
+    assert close(cam0[0], expect(40, 0, 20)) and close(cam0[9], expect(40, 9, 20))
+    assert close(cam0[10], 1.0) and close(cam0[31], 1.0)
+    reg3 = t[0, 0, n + 3]                   # special token 3 of frame 41: (41, 3, 3)
+    assert close(reg3[4], expect(41, 4, 20)) and close(reg3[10 + 2], expect(3, 2, 22)) and close(reg3[21 + 7], expect(3, 7, 22))
+    p = t[0, 0, s + 5 * ppw + 11]           # patch (5, 11) of frame 40: (40, 6 + 5, 6 + 11)
+    assert close(p[10 + 1], expect(11, 1, 22)) and close(p[21 + 10], expect(17, 10, 22)) and close(p[3], expect(40, 3, 20))
+    last = t[0, 0, 2 * n - 1]               # patch (26, 36) of frame 41
+    assert close(last[10], expect(32, 0, 22)) and close(last[21], expect(42, 0, 22)) and close(last[0], expect(41, 0, 20))
+
+    # the frame index moves the frame pairs only; a one-frame table is the first frame of a longer one
+    u = rope3d_freqs(2, pph, ppw, s, f_start=7, f_end=9)
+    assert torch.equal(u[..., 10:], t[..., 10:]) and not torch.equal(u[..., :10], t[..., :10])
+    one = rope3d_freqs(1, pph, ppw, s)
+    two = rope3d_freqs(2, pph, ppw, s)
+    assert torch.equal(two[:, :, :n], one) and one[0, 0, 0].eq(1).all()
+    # without special tokens the grid starts at (0, 0)
+    z = rope3d_freqs(1, 3, 4, 0)
+    assert z.shape == (1, 1, 12, 32) and z[0, 0, 0].eq(1).all() and close(z[0, 0, 1 * 4 + 2][10 + 1], expect(1, 1, 22))
+    assert close(z[0, 0, 1 * 4 + 2][21 + 1], expect(2, 1, 22))
