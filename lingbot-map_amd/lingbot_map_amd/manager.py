@@ -30,7 +30,7 @@ from __future__ import annotations
 
 import ctypes as C
 import math
-from typing import List, Optional, Sequence
+from typing import Dict, List, Optional, Sequence
 
 import torch
 from torch import Tensor
@@ -178,6 +178,9 @@ class HipPagedKVCacheManager:
         # visible-token counts and self-tail flags of the latest plan of each table set
         self._plan_tokens = [[0] * num_streams for _ in range(self._n_sets)]
         self._plan_valid = [False] * self._n_sets
+        # append rows of frames block 0 wrote while other blocks were still behind (anchor pass)
+        self._rows_log: Dict[int, Tensor] = {}
+        self._n_appends: List[int] = [0] * num_blocks    # appends ever made per block (rollbacks do not count down)
         self.reset()
 
     # =========================================================================
@@ -306,23 +309,56 @@ class HipPagedKVCacheManager:
         if v.dtype != k.dtype:
             v = v.to(k.dtype)
         ts = self._set(block_idx)
+        rows = self._append_rows[ts]
         if self._leads(block_idx):
+            if self._others_behind():
+                # the anchor pass appends several frames block by block (attention.py:497-511):
+                # the other blocks still have to write the frame appended last, keep its rows
+                self._rows_log[self._n_appends[0] - 1] = rows.clone()
             for b in range(self.num_streams):
                 if self._active[b]:
                     self._mirror_append(self._counts[ts][b], block_idx)
             ops = self._ops([{"ops": N.OP_APPEND if self._active[b] else 0} for b in range(self.num_streams)])
             self._tables_step(ts, ops, append_rows=True)
             self._plan_valid[ts] = False
-        self._scatter(block_idx, ts, k, v)
+        else:
+            n, lead = self._n_appends[block_idx], self._n_appends[0]
+            if n >= lead:
+                raise RuntimeError(f"block {block_idx} makes its append number {n} before block 0 has: with shared "
+                                   "page tables block 0 goes first (or build the manager with per_block_tables=True)")
+            if n < lead - 1:
+                rows = self._rows_log.get(n)
+                if rows is None:
+                    raise RuntimeError(f"block {block_idx} has made {n} appends, block 0 {lead}, and the rows of "
+                                       "that frame are no longer known (evicted or rolled back in between)")
+        self._scatter(block_idx, rows, k, v)
         self.frame_count[block_idx] += 1
+        self._n_appends[block_idx] += 1
+        if self._rows_log and not self._leads(block_idx):
+            done = min(self._n_appends[1:])
+            for f in [f for f in self._rows_log if f < done]:
+                del self._rows_log[f]
 
-    def _scatter(self, block_idx: int, ts: int, k: Tensor, v: Tensor) -> None:
+    def _others_behind(self) -> bool:
+        """Shared page tables only: some block has not yet written the frame block 0 appended last."""
+        return (not self.per_block_tables and self.num_blocks > 1
+                and min(self._n_appends[1:]) < self._n_appends[0])
+
+    def _in_step(self, block_idx: int, what: str) -> None:
+        """Shared page tables describe the frames block 0 has appended; another block may use
+        them only once it has written the same frames."""
+        if not self._leads(block_idx) and self._n_appends[block_idx] != self._n_appends[0]:
+            raise RuntimeError(f"{what}: block {block_idx} has made {self._n_appends[block_idx]} appends, block 0 "
+                               f"{self._n_appends[0]}; with shared page tables every block handles a frame before "
+                               "block 0 moves on (only the anchor pass may append block by block)")
+
+    def _scatter(self, block_idx: int, rows: Tensor, k: Tensor, v: Tensor) -> None:
         N.check(N.lib.lbm_kv_append(
             C.c_void_p(k.data_ptr()), C.c_void_p(v.data_ptr()),
             N.DTYPE_BF16 if k.dtype == torch.bfloat16 else N.DTYPE_F32,
             C.c_void_p(self.kv_caches[block_idx].data_ptr()),
             N.DTYPE_BF16 if self.dtype == torch.bfloat16 else N.DTYPE_F32,
-            C.c_void_p(self._append_rows[ts].data_ptr()), k.shape[0], self.num_heads, self.head_dim,
+            C.c_void_p(rows.data_ptr()), k.shape[0], self.num_heads, self.head_dim,
             self.page_size, self._stream_handle()))
 
     def evict_frames(self, block_idx: int, scale_frames: int, sliding_window: int,
@@ -349,6 +385,7 @@ class HipPagedKVCacheManager:
                 todo = True
         if not todo:
             return
+        self._rows_log.clear()   # evicted pages may be handed out again: a block still behind raises
         ops = self._ops([{"ops": N.OP_EVICT if self._active[b] else 0, "sliding_window": self._window_of(b, sliding_window),
                           "keep_tokens": keep} for b in range(self.num_streams)])
         self._tables_step(ts, ops)
@@ -358,6 +395,7 @@ class HipPagedKVCacheManager:
         assert self.frame_count[block_idx] > 0, f"block {block_idx}: cannot rollback, frame_count is 0"
         if self._leads(block_idx):
             ts = self._set(block_idx)
+            self._rows_log.clear()
             for b in range(self.num_streams):
                 if self._active[b]:
                     self._mirror_rollback(self._counts[ts][b], block_idx)
@@ -399,6 +437,7 @@ class HipPagedKVCacheManager:
         if self.frame_count[block_idx] == 0 and not has_tail:
             return torch.zeros_like(q)  # flashinfer_cache.py:368-370
         ts = self._set(block_idx)
+        self._in_step(block_idx, "compute_attention")
         if self._leads(block_idx) or not self._plan_valid[ts]:
             self._plan(ts, [has_tail and self._active[b] for b in range(self.num_streams)])
         return self._attend_planned(block_idx, q, self_k, self_v)
@@ -413,8 +452,9 @@ class HipPagedKVCacheManager:
             v = v.to(k.dtype)
         ts, keyframe, tail = self._step_tables(block_idx, keyframe, cross_frame_special, camera_only)
         if any(keyframe):
-            self._scatter(block_idx, ts, k, v)
+            self._scatter(block_idx, self._append_rows[ts], k, v)
             self.frame_count[block_idx] += 1
+            self._n_appends[block_idx] += 1
         return self._attend_planned(block_idx, q, k if any(tail) else None, v if any(tail) else None)
 
     def step_qkv(self, block_idx: int, qkv: Tensor, q_norm=None, k_norm=None, rope_cs: Optional[Tensor] = None,
@@ -457,6 +497,7 @@ class HipPagedKVCacheManager:
             rows, H, D, self.page_size, self._stream_handle()))
         if any(keyframe):
             self.frame_count[block_idx] += 1
+            self._n_appends[block_idx] += 1
         return self._attend_planned(block_idx, q, k, v)
 
     def _as_f32(self, t: Tensor, n: int) -> Tensor:
@@ -501,6 +542,7 @@ class HipPagedKVCacheManager:
         keep = self._keep_tokens(cross_frame_special, camera_only)
         for i in range(self.num_blocks):
             self.frame_count[i] += n
+            self._n_appends[i] += n
         for ts in range(self._n_sets):
             for b in range(self.num_streams):
                 if not self._active[b]:
@@ -531,6 +573,9 @@ class HipPagedKVCacheManager:
         tail = [self._active[b] and not keyframe[b] for b in range(self.num_streams)]
         ts = self._set(block_idx)
         if self._leads(block_idx):
+            if self._others_behind():
+                raise RuntimeError(f"step: block 0 starts a frame while another block has made "
+                                   f"{min(self._n_appends[1:])} of its {self._n_appends[0]} appends")
             keep = self._keep_tokens(cross_frame_special, camera_only)
             per = []
             for b in range(self.num_streams):
@@ -552,6 +597,9 @@ class HipPagedKVCacheManager:
                             "expect_kv_tokens": self._expect(n)})
             self._tables_step(ts, self._ops(per), append_rows=True, kv_rows=True)
             self._plan_valid[ts] = True
+        elif self._n_appends[block_idx] + (1 if any(keyframe) else 0) != self._n_appends[0]:
+            raise RuntimeError(f"step: block {block_idx} has made {self._n_appends[block_idx]} appends, block 0 "
+                               f"{self._n_appends[0]}: with shared page tables every block takes the frame block 0 took")
         return ts, keyframe, tail
 
     def _attend_planned(self, block_idx: int, q: Tensor, self_k: Optional[Tensor], self_v: Optional[Tensor]) -> Tensor:
@@ -605,6 +653,8 @@ class HipPagedKVCacheManager:
             self._plan_tokens[ts] = [0] * self.num_streams
         for i in range(self.num_blocks):
             self.frame_count[i] = 0
+            self._n_appends[i] = 0
+        self._rows_log.clear()
         self._active = [True] * self.num_streams
 
     # ----- table read-back (synchronises; for tests, debugging and parity checks) -----

@@ -124,3 +124,121 @@ def test_frame_block_without_cache_matches_torch_path(rope):
     assert err.max().item() <= 2e-2 and err.mean().item() <= 2e-3
     err = (y.float() - y_ref.float()).abs()
     assert err.max().item() <= 3e-2 and err.mean().item() <= 2e-3
+
+
+def test_camera_trunk_blocks_one_token_per_frame_fp32():
+    """The camera head's trunk (lingbot_map/heads/camera_head.py:212-219, :296-346): blocks of 128-wide
+    heads in fp32 over one camera token per frame at coordinates (f, 0, 0), the anchor frames in
+    one call and every later frame on its own, nothing ever evicted (attention.py:307).  Checked
+    against attention over the concatenation of every frame's K/V in float64."""
+    from lingbot_map_amd import HipPagedBlock, HipPagedKVCacheManager, RotaryPositionEmbedding3D
+    torch.manual_seed(9)
+    dev = torch.device("cuda:0")
+    dim, H, D, blocks, anchor, frames = 256, 2, 128, 4, 3, 45
+    rope3d = RotaryPositionEmbedding3D(attention_head_dim=D, patch_size=(1024, 1, 1), fhw_dim=(40, 44, 44))
+    mods = [HipPagedBlock(dim, H, init_values=0.5, qk_norm=True, rope=True, kv_cache_sliding_window=frames,
+                          kv_cache_scale_frames=anchor).to(dev).eval() for _ in range(blocks)]
+    m = HipPagedKVCacheManager(blocks, frames + 8, 1, H, D, torch.float32, dev, num_special_tokens=0,
+                               scale_frames=anchor, sliding_window=frames, max_total_frames=frames + 8,
+                               force_fp32=True, page_size=16, layout="frame_pages")
+    seen_k = [[] for _ in range(blocks)]
+    seen_v = [[] for _ in range(blocks)]
+    f = 0
+    with torch.no_grad():
+        while f < frames:
+            S = anchor if f == 0 else 1
+            x = torch.randn(1, S, dim, device=dev)
+            pos = rope3d(ppf=S, pph=1, ppw=1, patch_start_idx=0, device=dev, f_start=f, f_end=f + S)
+            y, y_ref = x, x
+            for b, mod in enumerate(mods):
+                y = mod(y, pos=pos, enable_3d_rope=True, kv_cache=m, global_idx=b, num_frames=S)
+                q, k, v = mod.attn_pre(y_ref, pos=pos, enable_3d_rope=True)      # [S, H, D]
+                seen_k[b].append(k.double()); seen_v[b].append(v.double())
+                K, V = torch.cat(seen_k[b]), torch.cat(seen_v[b])
+                s = torch.einsum("qhd,khd->hqk", q.double(), K) / D ** 0.5
+                a = torch.einsum("hqk,khd->qhd", torch.softmax(s, -1), V).reshape(1, S, dim).float()
+                y_ref = mod.ffn_residual(y_ref + mod.ls1(mod.attn.proj(a)))
+            err = (y - y_ref).abs().max().item()
+            assert err <= 2e-5, (f, err)
+            f += S
+    assert m.frame_count == [frames] * blocks and m.device_header()["error"] == 0
+
+
+@pytest.mark.parametrize("reference_calls", [False, True])
+def test_anchor_pass_over_several_frames_then_streaming(reference_calls):
+    """Phase 1 of the streaming model (attention.py:475-511): the anchor frames arrive in one call,
+    attend to one another densely, and are appended frame by frame, each block in turn, so block 0
+    is several frames ahead of the others while they write.  Later frames stream one at a time
+    and must see exactly the anchor frames and the window."""
+    from lingbot_map_amd import HipPagedBlock, HipPagedKVCacheManager, keyframe_flags, set_skip_append
+    from oracle.sdpa_cache import DictCacheOracle
+    torch.manual_seed(11)
+    dev = torch.device("cuda:0")
+    dim, H, T, n_sp, scale, window, blocks = 256, 4, 37, 5, 3, 2, 3
+    mods = [HipPagedBlock(dim, H, init_values=0.1, qk_norm=True, kv_cache_sliding_window=window,
+                          kv_cache_scale_frames=scale).to(dev, torch.bfloat16).eval() for _ in range(blocks)]
+    m = HipPagedKVCacheManager(blocks, scale + window + 16, T, H, 64, torch.bfloat16, dev, num_special_tokens=n_sp,
+                               scale_frames=scale, sliding_window=window, max_total_frames=64, page_size=16,
+                               layout="two_stream")
+    cache = ReferenceSurfaceOnly(m) if reference_calls else m
+    dense = [DictCacheOracle(scale, window, n_sp) for _ in range(blocks)]
+    sdpa = lambda q, k, v: torch.nn.functional.scaled_dot_product_attention(
+        q.float().permute(1, 0, 2)[None], k.float().permute(1, 0, 2)[None], v.float().permute(1, 0, 2)[None])[0].permute(1, 0, 2)
+    flags = [True] * scale + keyframe_flags(9, 0, 2)
+    with torch.no_grad():
+        f = 0
+        while f < len(flags):
+            S = scale if f == 0 else 1
+            kf = flags[f]
+            x = torch.randn(1, S * T, dim, device=dev).to(torch.bfloat16)
+            set_skip_append(cache, not kf)
+            y, y_ref = x, x
+            for b, mod in enumerate(mods):
+                y = mod(y, kv_cache=cache, global_idx=b, num_frames=S)
+                q, k, v = mod.attn_pre(y_ref)                                      # [S * T, H, D]
+                if S > 1:
+                    a = sdpa(q, k, v)
+                    for i in range(S):
+                        dense[b].visible(k[i * T:(i + 1) * T], v[i * T:(i + 1) * T], keyframe=True)
+                else:
+                    a = sdpa(q, *dense[b].visible(k, v, keyframe=kf))
+                a = a.reshape(1, S * T, dim).to(torch.bfloat16)
+                y_ref = mod.ffn_residual(y_ref + mod.ls1(mod.attn.proj(a)))
+            set_skip_append(cache, False)
+            err = (y.float() - y_ref.float()).abs()
+            assert err.max().item() <= 3e-2 and err.mean().item() <= 2e-3, (f, err.max().item(), err.mean().item())
+            f += S
+    assert m.frame_count == [sum(flags)] * blocks and m.device_header()["error"] == 0 and not m._rows_log
+
+
+def test_blocks_out_of_step_raise_with_shared_tables():
+    """With one page table for all blocks a block may lag only while appending (the anchor pass);
+    anything else out of step raises instead of reading or writing another frame's rows."""
+    from lingbot_map_amd import HipPagedKVCacheManager
+    dev = torch.device("cuda:0")
+    H, D, T = 2, 64, 9
+    mk = lambda **kw: HipPagedKVCacheManager(2, 24, T, H, D, torch.bfloat16, dev, num_special_tokens=1, scale_frames=1,
+                                             sliding_window=2, max_total_frames=32, page_size=4, **kw)
+    t = lambda: torch.randn(T, H, D, device=dev).to(torch.bfloat16)
+    m = mk()
+    with pytest.raises(RuntimeError, match="block 0 goes first"):
+        m.append_frame(1, t(), t())
+    m.append_frame(0, t(), t())
+    assert m.compute_attention(1, t()).abs().max().item() == 0      # an empty block attends to nothing
+    m.append_frame(0, t(), t())          # block 0 two frames ahead: allowed, rows of frame 0 are kept
+    m.append_frame(1, t(), t())
+    with pytest.raises(RuntimeError, match="compute_attention"):
+        m.compute_attention(1, t())
+    m.append_frame(1, t(), t())
+    m.compute_attention(1, t())
+    m.append_frame(0, t(), t())
+    with pytest.raises(RuntimeError, match="block 0 starts a frame"):
+        m.step(0, t(), t(), t())
+    m.append_frame(1, t(), t())
+    m.step(0, t(), t(), t())
+    with pytest.raises(RuntimeError, match="block 0 goes first|no longer known"):
+        m.append_frame(1, t(), t()); m.append_frame(1, t(), t())
+    # per-block tables: any order
+    p = mk(per_block_tables=True)
+    p.append_frame(1, t(), t()); p.compute_attention(1, t()); p.append_frame(0, t(), t())
+    assert p.device_header(0)["error"] == 0 and p.device_header(1)["error"] == 0
