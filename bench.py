@@ -102,7 +102,7 @@ def cpu_baseline(torch, kv_tokens: int, blocks: int) -> dict:
     }
 
 
-def aggregator_step(torch, blocks: int, steps: int, warmup: int) -> dict:
+def aggregator_step(torch, blocks: int, steps: int, warmup: int, windows=(WINDOW,)) -> dict:
     """One streamed frame (a 3 x 378 x 518 image) through the image encoder's ViT-L trunk (patch
     embedding, 24 blocks; lingbot_map/layers/vision_transformer.py:383-394) and through `blocks`
     groups of (frame block, global block) of the aggregator (lingbot_map/aggregator/stream.py:
@@ -110,7 +110,9 @@ def aggregator_step(torch, blocks: int, steps: int, warmup: int) -> dict:
     rotary embedding in the aggregator blocks), random init, bf16.  The global blocks run the HIP
     cache path, every block's pre-attention producer and cache-less attention are HIP kernels
     too; linears, LayerNorm, GELU and the patch-embedding convolution are PyTorch-ROCm library
-    calls.  The prediction heads are not part of the step."""
+    calls.  The prediction heads are not part of the step.  `windows` holds one sliding window
+    per stream: more than one entry runs that many independent streams as one ragged batch (a
+    step is then one frame of every stream)."""
     from lingbot_map_amd import (HipPagedBlock, HipPagedKVCacheManager, PositionGetter, RotaryPositionEmbedding2D,
                                  RotaryPositionEmbedding3D)
     dev = torch.device("cuda:0")
@@ -126,24 +128,26 @@ def aggregator_step(torch, blocks: int, steps: int, warmup: int) -> dict:
     encoder_blocks = [HipPagedBlock(dim=dim, num_heads=H, mlp_ratio=4.0, init_values=1.0).to(dev, torch.bfloat16).eval()
                       for _ in range(24)]
     patch_embed = torch.nn.Conv2d(3, dim, kernel_size=14, stride=14).to(dev, torch.bfloat16).eval()
-    special = torch.randn(1, N_SPECIAL, dim, device=dev).to(torch.bfloat16)      # class + register tokens
-    m = HipPagedKVCacheManager(blocks, ANCHOR + WINDOW + 16, T, H, D, torch.bfloat16, dev,
-                               num_special_tokens=N_SPECIAL, scale_frames=ANCHOR, sliding_window=WINDOW,
-                               max_total_frames=256, page_size=PAGE, layout="frame_pages")
+    B = len(windows)
+    special = torch.randn(1, N_SPECIAL, dim, device=dev).to(torch.bfloat16).expand(B, -1, -1)   # class + register tokens
+    m = HipPagedKVCacheManager(blocks, ANCHOR + max(windows) + 16, T, H, D, torch.bfloat16, dev,
+                               num_special_tokens=N_SPECIAL, scale_frames=ANCHOR,
+                               sliding_window=list(windows) if B > 1 else windows[0],
+                               max_total_frames=256, page_size=PAGE, layout="frame_pages", num_streams=B)
     g = torch.Generator(device=dev).manual_seed(4)
     # rotary table of the global blocks for frame 40 of a stream (frame / row / column pairs 10 / 11 / 11)
     rope3d = RotaryPositionEmbedding3D(attention_head_dim=D, patch_size=(1, 14, 14), max_seq_len=1024)
     freqs = rope3d(ppf=1, pph=27, ppw=37, patch_start_idx=N_SPECIAL, device=dev, f_start=40, f_end=41)
     assert freqs.shape == (1, 1, T, D // 2)
-    xs = [torch.rand(1, 3, 378, 518, generator=g, device=dev, dtype=torch.float32).to(torch.bfloat16) for _ in range(4)]
+    xs = [torch.rand(B, 3, 378, 518, generator=g, device=dev, dtype=torch.float32).to(torch.bfloat16) for _ in range(4)]
     # (y, x) of every token: specials at (0, 0), patches on the grid shifted by one (lingbot_map/aggregator/base.py:434-440)
     grid = PositionGetter()(1, 27, 37, dev)[0] + 1
-    pos2d = torch.cat([torch.zeros(N_SPECIAL, 2, dtype=grid.dtype, device=dev), grid])[None].contiguous()
-    assert pos2d.shape == (1, T, 2)
+    pos2d = torch.cat([torch.zeros(N_SPECIAL, 2, dtype=grid.dtype, device=dev), grid])[None].expand(B, -1, -1).contiguous()
+    assert pos2d.shape == (B, T, 2)
 
     @torch.no_grad()
     def frame_x(image):
-        x = torch.cat([special, patch_embed(image).flatten(2).transpose(1, 2)], dim=1)   # [1, 1004, 1024]
+        x = torch.cat([special, patch_embed(image).flatten(2).transpose(1, 2)], dim=1)   # [B, 1004, 1024]
         for blk in encoder_blocks:
             x = blk(x)
         for b in range(blocks):
@@ -154,7 +158,7 @@ def aggregator_step(torch, blocks: int, steps: int, warmup: int) -> dict:
     def frame(i: int):
         return frame_x(xs[i % len(xs)])
 
-    for i in range(ANCHOR + WINDOW + warmup):
+    for i in range(ANCHOR + max(windows) + warmup):
         frame(i)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
@@ -175,10 +179,11 @@ def aggregator_step(torch, blocks: int, steps: int, warmup: int) -> dict:
     torch.cuda.synchronize()
     dt_graph = (time.perf_counter() - t0) / steps
     assert torch.isfinite(out.float()).all() and m.device_header()["error"] == 0
-    return {"value": 1.0 / dt, "unit": "frames/s", "ms_per_step": dt * 1e3, "steps": steps,
-            "hip_graph": {"value": 1.0 / dt_graph, "unit": "frames/s", "ms_per_step": dt_graph * 1e3},
+    kv = " / ".join(str((ANCHOR + w) * T) for w in windows)
+    return {"value": B / dt, "unit": "frames/s", "ms_per_step": dt * 1e3, "steps": steps, "streams": B,
+            "hip_graph": {"value": B / dt_graph, "unit": "frames/s", "ms_per_step": dt_graph * 1e3},
             "what": f"patch embedding + 24 encoder blocks + {blocks} x (frame block + global block), dim {dim}, {H} heads, "
-                    f"MLP {4 * dim}, 1 stream, {T} tokens/frame, steady-state cache of {(ANCHOR + WINDOW) * T} KV tokens; "
+                    f"MLP {4 * dim}, {B} stream(s), {T} tokens/frame, steady-state cache of {kv} KV tokens; "
                     f"PyTorch-ROCm for linears / LayerNorm / GELU / convolution, HIP kernels for q/k norm + rotary + "
                     f"append, the cache path and every block's cache-less attention; prediction heads excluded"}
 
@@ -270,7 +275,7 @@ def main() -> None:
         assert m._plan_tokens[0][0] == kv_tokens == 17068
         ops = m._ops([{"ops": 16, "expect_kv_tokens": kv_tokens}])
         fn = {"attention": lambda: m._attend_planned(1, qs[0], None, None),
-              "append": lambda: m._scatter(1, 0, ks[0], vs[0]),
+              "append": lambda: m._scatter(1, m._append_rows[0], ks[0], vs[0]),
               "prepare": lambda: prepare(1),
               "residual": residual,
               "tables": lambda: m._tables_step(0, ops, kv_rows=True)}[args.mode]
@@ -297,7 +302,7 @@ def main() -> None:
     # ---- per-kernel timings with HIP events on the launch stream
     flops = 4.0 * T * kv_tokens * H * D
     attn_ms = event_time_ms(lambda: m._attend_planned(1, qs[0], None, None), 500, torch)
-    append_ms = kernel_time_ms(lambda: m._scatter(1, 0, ks[0], vs[0]), 100, torch)
+    append_ms = kernel_time_ms(lambda: m._scatter(1, m._append_rows[0], ks[0], vs[0]), 100, torch)
     ops = m._ops([{"ops": 16, "expect_kv_tokens": kv_tokens}])
     tables_ms = kernel_time_ms(lambda: m._tables_step(0, ops, kv_rows=True), 100, torch)
     attn_tflops = flops / (attn_ms * 1e-3) * 1e-12
@@ -340,6 +345,9 @@ def main() -> None:
     if not args.no_aggregator:
         del m
         line["aggregator_step"] = aggregator_step(torch, blocks, 20, 3)
+        torch.cuda.empty_cache()
+        # config 5: four independent streams with windows 4 / 8 / 16 / 16 as one ragged batch
+        line["aggregator_step_4_streams"] = aggregator_step(torch, blocks, 10, 2, windows=(4, 8, 16, 16))
     if not args.no_cpu_baseline:
         line["cpu_baseline"] = cpu_baseline(torch, kv_tokens, blocks)
     print(json.dumps(line))
