@@ -68,6 +68,53 @@ def event_time_ms(fn, iters: int, torch) -> float:
     return start.elapsed_time(stop) / iters
 
 
+def config1(torch) -> dict:
+    """Config 1, the CPU-runnable parity case: fp32, 8 frames of 1004 tokens, Q, K, V =
+    randn / 8 with seed 0, frame i attends to frames 0..i (148.6 GFLOP in all).  The oracle's
+    SDPA on the host cores beside the fp32 HIP kernel on the same inputs, and their largest
+    difference."""
+    from lingbot_map_amd import HipPagedKVCacheManager
+    from oracle.sdpa_cache import sdpa_nhd
+    torch.manual_seed(0)
+    frames = 8
+    qkv = [[torch.randn(T, H, D) / 8 for _ in range(3)] for _ in range(frames)]
+    dev = torch.device("cuda:0")
+    dq = [[t.to(dev) for t in f] for f in qkv]
+
+    def cpu():
+        outs = []
+        for i in range(frames):
+            k = torch.cat([f[1] for f in qkv[:i + 1]])
+            v = torch.cat([f[2] for f in qkv[:i + 1]])
+            outs.append(sdpa_nhd(qkv[i][0], k, v))
+        return outs
+
+    def gpu():
+        m.reset()
+        outs = []
+        for i in range(frames):
+            outs.append(m.step(0, dq[i][0], dq[i][1], dq[i][2], keyframe=[True]))
+        return outs
+
+    m = HipPagedKVCacheManager(1, 32, T, H, D, torch.float32, dev, num_special_tokens=N_SPECIAL, scale_frames=1,
+                               sliding_window=16, max_total_frames=32, force_fp32=True, page_size=PAGE, layout="frame_pages")
+    cpu()
+    t0 = time.perf_counter()
+    ref = cpu()
+    t_cpu = time.perf_counter() - t0
+    gpu()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    got = gpu()
+    torch.cuda.synchronize()
+    t_gpu = time.perf_counter() - t0
+    err = max((a.cpu() - b).abs().max().item() for a, b in zip(got, ref))
+    flops = sum(4.0 * T * (i + 1) * T * H * D for i in range(frames))
+    return {"cpu_ms": t_cpu * 1e3, "cpu_gflops": flops / t_cpu * 1e-9, "gpu_ms": t_gpu * 1e3,
+            "gpu_gflops": flops / t_gpu * 1e-9, "max_abs_diff": err, "tolerance": 1e-5,
+            "what": "8 frames, fp32, every frame attends to all frames so far (tables step + append + fp32 MFMA attention per frame, wall clock)"}
+
+
 def cpu_baseline(torch, kv_tokens: int, blocks: int) -> dict:
     """The reference SDPA arithmetic (dense gather of the visible pages, then
     F.scaled_dot_product_attention) as restated by the oracle, on the host cores."""
@@ -94,7 +141,9 @@ def cpu_baseline(torch, kv_tokens: int, blocks: int) -> dict:
         times.append(time.perf_counter() - t0)
     t = sorted(times)[len(times) // 2]
     flops = 4.0 * T * kv_tokens * H * D
+    c1 = config1(torch)
     return {
+        "config1_fp32": c1,
         "value": 1.0 / (t * blocks), "unit": "frames/s", "cores": torch.get_num_threads(), "kind": "port",
         "sample": f"2 warm-up + 15 timed layer-steps of gather + SDPA (q {T} x kv {kv_tokens}, {H} heads, "
                   f"bf16 storage, fp32 math), median {t * 1e3:.1f} ms = {flops / t * 1e-9:.0f} GFLOP/s; "

@@ -591,11 +591,22 @@ __global__ __launch_bounds__(256) void lbm_attn_combine_bf16_kernel(AttnArgs a) 
 
 // ---------------------------------------------------------------------------- fp32 path
 // Same contract as the bf16 kernel for pools kept in fp32 (the reference's force_fp32 mode,
-// lingbot_map/layers/flashinfer_cache.py:118-127,372-383).  Accuracy path, not a speed path:
-// plain fp32 FMAs, one workgroup per (64 query rows, head), four threads per query row that
-// each own a quarter of the head dimensions; exact running maximum, no split-KV.  head_dim 64,
-// and 128 for the camera head's one-token-per-frame cache (lingbot_map/heads/camera_head.py:
-// 284-377: 16 heads of 128, fp32).
+// lingbot_map/layers/flashinfer_cache.py:118-127,372-383), head_dim 64, and 128 for the camera
+// head's one-token-per-frame cache (lingbot_map/heads/camera_head.py:284-377: 16 heads of 128).
+// Full fp32 products and sums on the matrix pipe (v_mfma_f32_16x16x4_f32), exact running
+// maximum, no split-KV.  One workgroup per (64 query rows, head), one wave per 16 query rows.
+//
+// A lane is (n = lane % 16, g = lane / 16).  Scores are kept transposed, S^T = K Q^T: the
+// 16x16x4 product takes K[kv = n][dim k_g] from every lane as A and Q[q = n][dim k_g] as B and
+// leaves S^T[kv = 4g + i][q = n] in element i of lane (n, g), so a lane's four elements
+// belong to ONE query row and the softmax statistics are per lane plus two cross-lane steps
+// over g.  Which head dimension lane group g contributes in step t is free as long as A and B
+// agree; dim = (D/4) g + t makes the K operand four consecutive floats per four steps (one
+// ds_read_b128) and the Q operand a contiguous quarter row held in registers.  For O^T = V^T P^T
+// the same freedom is used on the KV index: step (c, i) contracts kv = 16c + 4g + i over g,
+// which is exactly where element i of the score block c already sits - P goes from the
+// accumulator into the B operand without a shuffle.  O^T[dim = 16e + 4g + i][q = n] ends up
+// as four consecutive dims per lane: 16-byte stores.
 namespace {
 constexpr int kF32Rows = 64;
 struct AttnArgsF32 {
@@ -617,13 +628,18 @@ struct AttnArgsF32 {
 
 template <int D>
 __global__ __launch_bounds__(256) void lbm_attn_f32_kernel(AttnArgsF32 a) {
-  constexpr int kTile = D == 64 ? 64 : 32;     // KV tokens per tile: 32 KiB of LDS either way
+  constexpr int kTile = D == 64 ? 64 : 32;     // KV tokens per tile: 16 KiB each of K and V
   constexpr int kStageThreads = 256 / kTile;   // threads that stage one row: 16 floats each
-  constexpr int DQ = D / 4;                    // head dims per compute thread
+  constexpr int LD = D + 4;                    // LDS row stride: rows stay 16-byte aligned and shift by 4 banks
+  constexpr int NC = kTile / 16;               // 16-token score blocks per tile
+  constexpr int NE = D / 16;                   // 16-dim output blocks
+  constexpr int DG = D / 4;                    // head dims one lane group contributes to q.k
   static_assert(D / kStageThreads == 16, "staging moves 16 floats per thread");
-  __shared__ __attribute__((aligned(16))) float lds_k[kTile][D];
-  __shared__ __attribute__((aligned(16))) float lds_v[kTile][D];
+  __shared__ __attribute__((aligned(16))) float lds_k[kTile][LD];
+  __shared__ __attribute__((aligned(16))) float lds_v[kTile][LD];
   const int tid = threadIdx.x;
+  const int lane = tid & 63, wave = tid >> 6;
+  const int n16 = lane & 15, g = lane >> 4;
   int b = 0;
   for (int i = 1; i < a.n_streams; ++i)
     if ((int)blockIdx.x >= a.wg_begin[i]) b = i;
@@ -632,26 +648,31 @@ __global__ __launch_bounds__(256) void lbm_attn_f32_kernel(AttnArgsF32 a) {
   const int H = a.num_heads;
   const int local = (int)blockIdx.x - a.wg_begin[b];
   const int head = local % H, qt = local / H;
-  const int r = qt * kF32Rows + (tid >> 2), c = tid & 3;  // query row, quarter of the head dim
+  const int r = qt * kF32Rows + wave * 16 + n16;   // this lane's query row
   const size_t row_elems = (size_t)H * D;
   const bool row_ok = r < sp.q_rows;
 
-  float q[DQ], o[DQ];
+  // Q[r][DG g .. DG g + DG - 1], pre-multiplied by scale * log2(e)
+  float q[DG];
   {
-    const float* qp = a.q + ((size_t)(sp.q_begin + (row_ok ? r : 0)) * H + head) * D + c * DQ;
+    const float* qp = a.q + ((size_t)(sp.q_begin + (row_ok ? r : 0)) * H + head) * D + DG * g;
 #pragma unroll
-    for (int d = 0; d < DQ; ++d) {
-      q[d] = row_ok ? qp[d] * a.scale_log2 : 0.f;
-      o[d] = 0.f;
+    for (int d4 = 0; d4 < DG / 4; ++d4) {
+      const f32x4 x = row_ok ? ((const f32x4*)qp)[d4] : f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int j = 0; j < 4; ++j) q[4 * d4 + j] = x[j] * a.scale_log2;
     }
   }
-  float m = -INFINITY, l = 0.f;
+  f32x4 o[NE];
+#pragma unroll
+  for (int e = 0; e < NE; ++e) o[e] = f32x4{0.f, 0.f, 0.f, 0.f};
+  float m = -INFINITY, l = 0.f;   // running maximum of the row; this lane's share of the row sum
 
   const int ld_r = tid / kStageThreads, ld_c = (tid % kStageThreads) * 16;
   const int n_tiles = (sp.kv_tokens + kTile - 1) / kTile;
-  for (int t = 0; t < n_tiles; ++t) {
+  f32x4 kk[4], vv[4];
+  auto fetch = [&](int t) {
     const int kvi = t * kTile + ld_r;
-    f32x4 kk[4], vv[4];
 #pragma unroll
     for (int i = 0; i < 4; ++i) kk[i] = vv[i] = f32x4{0.f, 0.f, 0.f, 0.f};
     if (kvi < sp.kv_tokens) {
@@ -671,6 +692,9 @@ __global__ __launch_bounds__(256) void lbm_attn_f32_kernel(AttnArgsF32 a) {
         vv[i] = ((const f32x4*)vp)[i];
       }
     }
+  };
+  if (n_tiles > 0) fetch(0);
+  for (int t = 0; t < n_tiles; ++t) {
     __syncthreads();  // the previous tile is no longer being read
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
@@ -678,42 +702,68 @@ __global__ __launch_bounds__(256) void lbm_attn_f32_kernel(AttnArgsF32 a) {
       *(f32x4*)&lds_v[ld_r][ld_c + 4 * i] = vv[i];
     }
     __syncthreads();
-    const int n_valid = min(kTile, sp.kv_tokens - t * kTile);
-    for (int j0 = 0; j0 < n_valid; j0 += 8) {
-      float sc[8];
+    if (t + 1 < n_tiles) fetch(t + 1);   // in flight while this tile is computed
+
+    // S^T blocks: sc[c][i] = score of kv token 16c + 4g + i for query row n16
+    f32x4 sc[NC];
 #pragma unroll
-      for (int jj = 0; jj < 8; ++jj) {
-        const int j = j0 + jj;
-        float acc = 0.f;
+    for (int c = 0; c < NC; ++c) sc[c] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-        for (int d = 0; d < DQ; ++d) acc = __builtin_fmaf(q[d], lds_k[j][c * DQ + d], acc);
-        acc += __shfl_xor(acc, 1);
-        acc += __shfl_xor(acc, 2);
-        sc[jj] = j < n_valid ? acc : -INFINITY;
-      }
-      float mx = m;
+    for (int d4 = 0; d4 < DG / 4; ++d4) {
+      f32x4 kf[NC];
 #pragma unroll
-      for (int jj = 0; jj < 8; ++jj) mx = fmaxf(mx, sc[jj]);
-      const float alpha = exp2f(m - mx);  // m = -inf on the first step gives 0
-      m = mx;
-      l *= alpha;
+      for (int c = 0; c < NC; ++c) kf[c] = *(const f32x4*)&lds_k[16 * c + n16][DG * g + 4 * d4];
 #pragma unroll
-      for (int d = 0; d < DQ; ++d) o[d] *= alpha;
+      for (int j = 0; j < 4; ++j)
 #pragma unroll
-      for (int jj = 0; jj < 8; ++jj) {
-        const float p = exp2f(sc[jj] - m);
-        l += p;
-        const int j = min(j0 + jj, kTile - 1);
-#pragma unroll
-        for (int d = 0; d < DQ; ++d) o[d] = __builtin_fmaf(p, lds_v[j][c * DQ + d], o[d]);
-      }
+        for (int c = 0; c < NC; ++c)
+          sc[c] = __builtin_amdgcn_mfma_f32_16x16x4f32(kf[c][j], q[4 * d4 + j], sc[c], 0, 0, 0);
     }
+    const int n_valid = sp.kv_tokens - t * kTile;
+    if (n_valid < kTile) {
+#pragma unroll
+      for (int c = 0; c < NC; ++c)
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          if (16 * c + 4 * g + i >= n_valid) sc[c][i] = -INFINITY;
+    }
+    float mx = sc[0][0];
+#pragma unroll
+    for (int c = 0; c < NC; ++c)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) mx = fmaxf(mx, sc[c][i]);
+    mx = fmaxf(mx, __shfl_xor(mx, 16));
+    mx = fmaxf(mx, __shfl_xor(mx, 32));
+    mx = fmaxf(mx, m);                      // finite: token 0 of every tile is valid
+    const float alpha = exp2f(m - mx);      // m = -inf on the first tile gives 0
+    m = mx;
+    l *= alpha;
+#pragma unroll
+    for (int e = 0; e < NE; ++e) o[e] *= alpha;
+#pragma unroll
+    for (int c = 0; c < NC; ++c)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const float p = exp2f(sc[c][i] - m);
+        sc[c][i] = p;
+        l += p;
+      }
+    // O^T += V^T P^T, contraction step (c, i) over kv = 16c + 4g + i
+#pragma unroll
+    for (int c = 0; c < NC; ++c)
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int e = 0; e < NE; ++e)
+          o[e] = __builtin_amdgcn_mfma_f32_16x16x4f32(lds_v[16 * c + 4 * g + i][16 * e + n16], sc[c][i], o[e], 0, 0, 0);
   }
+  l += __shfl_xor(l, 16);
+  l += __shfl_xor(l, 32);
   if (row_ok) {
     const float inv = l > 0.f ? 1.0f / l : 0.f;
-    float* op = a.out + ((size_t)(sp.q_begin + r) * H + head) * D + c * DQ;
+    float* op = a.out + ((size_t)(sp.q_begin + r) * H + head) * D + 4 * g;
 #pragma unroll
-    for (int d = 0; d < DQ; ++d) op[d] = o[d] * inv;
+    for (int e = 0; e < NE; ++e) *(f32x4*)(op + 16 * e) = o[e] * inv;
   }
 }
 
