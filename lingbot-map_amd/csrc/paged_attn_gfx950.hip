@@ -594,7 +594,8 @@ __global__ __launch_bounds__(256) void lbm_attn_combine_bf16_kernel(AttnArgs a) 
 // lingbot_map/layers/flashinfer_cache.py:118-127,372-383), head_dim 64, and 128 for the camera
 // head's one-token-per-frame cache (lingbot_map/heads/camera_head.py:284-377: 16 heads of 128).
 // Full fp32 products and sums on the matrix pipe (v_mfma_f32_16x16x4_f32), exact running
-// maximum, no split-KV.  One workgroup per (64 query rows, head), one wave per 16 query rows.
+// maximum, no split-KV across workgroups.  One workgroup per (64 query rows, head), two waves
+// per 16 query rows.
 //
 // A lane is (n = lane % 16, g = lane / 16).  Scores are kept transposed, S^T = K Q^T: the
 // 16x16x4 product takes K[kv = n][dim k_g] from every lane as A and Q[q = n][dim k_g] as B and
@@ -627,18 +628,25 @@ struct AttnArgsF32 {
 }  // namespace
 
 template <int D>
-__global__ __launch_bounds__(256) void lbm_attn_f32_kernel(AttnArgsF32 a) {
-  constexpr int kTile = D == 64 ? 64 : 32;     // KV tokens per tile: 16 KiB each of K and V
-  constexpr int kStageThreads = 256 / kTile;   // threads that stage one row: 16 floats each
+__global__ __launch_bounds__(512) void lbm_attn_f32_kernel(AttnArgsF32 a) {
+  // Eight waves: wave w and wave w + 4 own the same 16 query rows and take alternate KV tiles
+  // (two waves per SIMD, so one's softmax and LDS waits overlap the other's matrix work); the
+  // two partial results are merged through LDS at the end.
+  constexpr int kTile = D == 64 ? 32 : 16;     // KV tokens per tile; two tiles are staged per iteration
+  constexpr int kRowThreads = D / 8;           // threads that stage one row: 8 floats of K and of V each
   constexpr int LD = D + 4;                    // LDS row stride: rows stay 16-byte aligned and shift by 4 banks
   constexpr int NC = kTile / 16;               // 16-token score blocks per tile
   constexpr int NE = D / 16;                   // 16-dim output blocks
   constexpr int DG = D / 4;                    // head dims one lane group contributes to q.k
-  static_assert(D / kStageThreads == 16, "staging moves 16 floats per thread");
-  __shared__ __attribute__((aligned(16))) float lds_k[kTile][LD];
-  __shared__ __attribute__((aligned(16))) float lds_v[kTile][LD];
+  static_assert(512 / kRowThreads == 2 * kTile, "512 threads stage two tiles");
+  constexpr int kTileFloats = 2 * kTile * LD;   // two K tiles (and as many again for V)
+  constexpr int kMergeFloats = (NE * 4 + 2) * 256;
+  constexpr int kLdsFloats = 2 * kTileFloats > kMergeFloats ? 2 * kTileFloats : kMergeFloats;
+  __shared__ __attribute__((aligned(16))) float lds_raw[kLdsFloats];
+  float (*lds_k)[LD] = (float (*)[LD])lds_raw;
+  float (*lds_v)[LD] = (float (*)[LD])(lds_raw + kTileFloats);
   const int tid = threadIdx.x;
-  const int lane = tid & 63, wave = tid >> 6;
+  const int lane = tid & 63, wave = (tid >> 6) & 3, half = tid >> 8;
   const int n16 = lane & 15, g = lane >> 4;
   int b = 0;
   for (int i = 1; i < a.n_streams; ++i)
@@ -668,13 +676,13 @@ __global__ __launch_bounds__(256) void lbm_attn_f32_kernel(AttnArgsF32 a) {
   for (int e = 0; e < NE; ++e) o[e] = f32x4{0.f, 0.f, 0.f, 0.f};
   float m = -INFINITY, l = 0.f;   // running maximum of the row; this lane's share of the row sum
 
-  const int ld_r = tid / kStageThreads, ld_c = (tid % kStageThreads) * 16;
+  const int ld_r = tid / kRowThreads, ld_c = (tid % kRowThreads) * 8;
   const int n_tiles = (sp.kv_tokens + kTile - 1) / kTile;
-  f32x4 kk[4], vv[4];
-  auto fetch = [&](int t) {
-    const int kvi = t * kTile + ld_r;
-#pragma unroll
-    for (int i = 0; i < 4; ++i) kk[i] = vv[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+  const int n_iters = (n_tiles + 1) / 2;
+  f32x4 kk[2], vv[2];
+  auto fetch = [&](int it) {
+    const int kvi = it * 2 * kTile + ld_r;
+    kk[0] = kk[1] = vv[0] = vv[1] = f32x4{0.f, 0.f, 0.f, 0.f};
     if (kvi < sp.kv_tokens) {
       const int e = a.kv_rows[sp.kv_row_begin + kvi];
       const float *kp, *vp;
@@ -686,25 +694,26 @@ __global__ __launch_bounds__(256) void lbm_attn_f32_kernel(AttnArgsF32 a) {
         kp = a.self_k + off;
         vp = a.self_v + off;
       }
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        kk[i] = ((const f32x4*)kp)[i];
-        vv[i] = ((const f32x4*)vp)[i];
-      }
+      kk[0] = ((const f32x4*)kp)[0];
+      kk[1] = ((const f32x4*)kp)[1];
+      vv[0] = ((const f32x4*)vp)[0];
+      vv[1] = ((const f32x4*)vp)[1];
     }
   };
-  if (n_tiles > 0) fetch(0);
-  for (int t = 0; t < n_tiles; ++t) {
-    __syncthreads();  // the previous tile is no longer being read
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      *(f32x4*)&lds_k[ld_r][ld_c + 4 * i] = kk[i];
-      *(f32x4*)&lds_v[ld_r][ld_c + 4 * i] = vv[i];
-    }
+  if (n_iters > 0) fetch(0);
+  for (int it = 0; it < n_iters; ++it) {
+    __syncthreads();  // the previous pair of tiles is no longer being read
+    *(f32x4*)&lds_k[ld_r][ld_c] = kk[0];
+    *(f32x4*)&lds_k[ld_r][ld_c + 4] = kk[1];
+    *(f32x4*)&lds_v[ld_r][ld_c] = vv[0];
+    *(f32x4*)&lds_v[ld_r][ld_c + 4] = vv[1];
     __syncthreads();
-    if (t + 1 < n_tiles) fetch(t + 1);   // in flight while this tile is computed
+    if (it + 1 < n_iters) fetch(it + 1);   // in flight while this pair is computed
+    const int t = 2 * it + half;           // this wave's tile
+    if (t >= n_tiles) continue;            // odd tile count: the second half sits out the last pair
+    const int row0 = half * kTile;
 
-    // S^T blocks: sc[c][i] = score of kv token 16c + 4g + i for query row n16
+    // S^T blocks: sc[c][i] = score of kv token 16c + 4g + i of the tile for query row n16
     f32x4 sc[NC];
 #pragma unroll
     for (int c = 0; c < NC; ++c) sc[c] = f32x4{0.f, 0.f, 0.f, 0.f};
@@ -712,7 +721,7 @@ __global__ __launch_bounds__(256) void lbm_attn_f32_kernel(AttnArgsF32 a) {
     for (int d4 = 0; d4 < DG / 4; ++d4) {
       f32x4 kf[NC];
 #pragma unroll
-      for (int c = 0; c < NC; ++c) kf[c] = *(const f32x4*)&lds_k[16 * c + n16][DG * g + 4 * d4];
+      for (int c = 0; c < NC; ++c) kf[c] = *(const f32x4*)&lds_k[row0 + 16 * c + n16][DG * g + 4 * d4];
 #pragma unroll
       for (int j = 0; j < 4; ++j)
 #pragma unroll
@@ -755,15 +764,40 @@ __global__ __launch_bounds__(256) void lbm_attn_f32_kernel(AttnArgsF32 a) {
       for (int i = 0; i < 4; ++i)
 #pragma unroll
         for (int e = 0; e < NE; ++e)
-          o[e] = __builtin_amdgcn_mfma_f32_16x16x4f32(lds_v[16 * c + 4 * g + i][16 * e + n16], sc[c][i], o[e], 0, 0, 0);
+          o[e] = __builtin_amdgcn_mfma_f32_16x16x4f32(lds_v[row0 + 16 * c + 4 * g + i][16 * e + n16], sc[c][i], o[e], 0, 0, 0);
   }
   l += __shfl_xor(l, 16);
   l += __shfl_xor(l, 32);
-  if (row_ok) {
-    const float inv = l > 0.f ? 1.0f / l : 0.f;
+
+  // merge the two halves: the second writes (o, m, l) per lane, the first rescales and adds
+  float* merge = lds_raw;
+  const int slot = tid & 255;
+  __syncthreads();
+  if (half == 1) {
+#pragma unroll
+    for (int e = 0; e < NE; ++e)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) merge[(4 * e + i) * 256 + slot] = o[e][i];
+    merge[(4 * NE) * 256 + slot] = m;
+    merge[(4 * NE + 1) * 256 + slot] = l;
+  }
+  __syncthreads();
+  if (half == 0 && row_ok) {
+    const float m1 = merge[(4 * NE) * 256 + slot], l1 = merge[(4 * NE + 1) * 256 + slot];
+    const float mt = fmaxf(m, m1);
+    // a half that saw no tile has m = -inf and contributes nothing; no KV at all leaves zeros
+    const float w0 = m > -INFINITY ? exp2f(m - mt) : 0.f;
+    const float w1 = m1 > -INFINITY ? exp2f(m1 - mt) : 0.f;
+    const float lt = l * w0 + l1 * w1;
+    const float inv = lt > 0.f ? 1.0f / lt : 0.f;
     float* op = a.out + ((size_t)(sp.q_begin + r) * H + head) * D + 4 * g;
 #pragma unroll
-    for (int e = 0; e < NE; ++e) *(f32x4*)(op + 16 * e) = o[e] * inv;
+    for (int e = 0; e < NE; ++e) {
+      f32x4 x;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) x[i] = (o[e][i] * w0 + merge[(4 * e + i) * 256 + slot] * w1) * inv;
+      *(f32x4*)(op + 16 * e) = x;
+    }
   }
 }
 
@@ -943,8 +977,8 @@ int lbm_launch_attention(const void* q, const void* pool, void* out, const void*
     }
     f.wg_begin[LBM_MAX_STREAMS] = wg;
     if (wg == 0) return LBM_OK;
-    if (head_dim == 64) hipLaunchKernelGGL(lbm_attn_f32_kernel<64>, dim3(wg), dim3(256), 0, stream, f);
-    else hipLaunchKernelGGL(lbm_attn_f32_kernel<128>, dim3(wg), dim3(256), 0, stream, f);
+    if (head_dim == 64) hipLaunchKernelGGL(lbm_attn_f32_kernel<64>, dim3(wg), dim3(512), 0, stream, f);
+    else hipLaunchKernelGGL(lbm_attn_f32_kernel<128>, dim3(wg), dim3(512), 0, stream, f);
     return lbm_check_launch("lbm_attn_f32_kernel");
   }
   if (dtype != LBM_DTYPE_BF16) return lbm_fail(LBM_ERR_INVALID, "unknown dtype %d", dtype);
