@@ -12,6 +12,7 @@ from __future__ import annotations
 
 import argparse
 import json
+import math
 import os
 import sys
 import time
@@ -66,6 +67,61 @@ def event_time_ms(fn, iters: int, torch) -> float:
     stop.record()
     stop.synchronize()
     return start.elapsed_time(stop) / iters
+
+
+def attention_shapes(torch) -> list:
+    """One lbm_attn_run at the attention shapes of the other configurations (synthetic bf16 pools and
+    row tables built here; HIP events around 100 launches after 100 warm-up launches)."""
+    import ctypes as C
+    from lingbot_map_amd import _native as N
+    dev = torch.device("cuda:0")
+
+    def run(name, kvs, tail=False, shuffle_seed=None):
+        ns = len(kvs)
+        g = torch.Generator(device=dev).manual_seed(0)
+        q = torch.randn(ns * T, H, D, generator=g, device=dev, dtype=torch.float32).to(torch.bfloat16)
+        n_pages = sum(-(-kv // PAGE) for kv in kvs)
+        pool = torch.randn(n_pages, 2, PAGE, H, D, generator=g, device=dev, dtype=torch.float32).to(torch.bfloat16)
+        order = torch.arange(n_pages)
+        if shuffle_seed is not None:   # cached pages scattered over the pool
+            order = torch.randperm(n_pages, generator=torch.Generator().manual_seed(shuffle_seed))
+        rows, begin, off, base = [], [], 0, 0
+        for b, kv in enumerate(kvs):
+            begin.append(off)
+            r = torch.arange(kv)
+            rr = order[r // PAGE + base] * 2 * PAGE + r % PAGE
+            if tail:   # the frame's own K/V, not in the pool (entry -1 - row)
+                rr[-T:] = -1 - (b * T + torch.arange(T))
+            rows.append(rr.to(torch.int32))
+            off += kv
+            base += -(-kv // PAGE)
+        kv_rows = torch.cat(rows).to(dev)
+        streams = (N.AttnStream * ns)(*[N.AttnStream(b * T, T, begin[b], kvs[b]) for b in range(ns)])
+        need = int(N.lib.lbm_attn_workspace_bytes(streams, ns, H, D))
+        ws = torch.empty(max(need, 16), dtype=torch.uint8, device=dev)
+        out = torch.empty_like(q)
+        own = q if tail else None
+        vp = lambda t: None if t is None else C.c_void_p(t.data_ptr())
+        stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+        def launch():
+            N.check(N.lib.lbm_attn_run(vp(q), vp(pool), vp(out), vp(own), vp(own), vp(kv_rows), streams, ns, H, D, PAGE,
+                                       N.DTYPE_BF16, 1.0 / math.sqrt(D), vp(ws), ws.numel(), stream))
+
+        for _ in range(100):
+            launch()
+        ms = event_time_ms(launch, 100, torch)
+        flop = 4.0 * T * sum(kvs) * H * D
+        assert torch.isfinite(out.float()).all()
+        return {"shape": name, "kv_tokens": kvs, "avg_launch_us": ms * 1e3, "tflops": flop / (ms * 1e-3) * 1e-12,
+                "frac": flop / (ms * 1e-3) * 1e-12 / PEAK_BF16_TFLOPS}
+
+    return [
+        run("config 3: 67,068 tokens, pages in shuffled order", [67068], shuffle_seed=2),
+        run("config 4 non-keyframe: 17,068 cached + the frame's own 1,004", [18072], tail=True),
+        run("config 5: four streams, 5,020 / 9,036 / 17,068 / 17,068", [5020, 9036, 17068, 17068]),
+        run("frame block: 1,004 x 1,004, no cache", [1004], tail=True),
+    ]
 
 
 def config1(torch) -> dict:
@@ -397,6 +453,7 @@ def main() -> None:
                           "avg_launch_us": residual_ms * 1e3,
                           "what": "x + ls(y) fused with the following LayerNorm, 1004 x 1024 bf16 (not in `value`'s timed loop)"},
         "tables_step_us": tables_ms * 1e3,
+        "attention_shapes": attention_shapes(torch),
     }
     if not args.no_aggregator:
         del m
