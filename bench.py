@@ -167,14 +167,17 @@ def config1(torch) -> dict:
     err = max((a.cpu() - b).abs().max().item() for a, b in zip(got, ref))
     flops = sum(4.0 * T * (i + 1) * T * H * D for i in range(frames))
     # the attention launch of the last frame alone (1004 queries x 8032 cached tokens)
-    k_ms = event_time_ms(lambda: m.compute_attention(0, dq[-1][0]), 20, torch)
+    m._plan(0, [False])
+    for _ in range(20):
+        m._attend_planned(0, dq[-1][0], None, None)
+    k_ms = event_time_ms(lambda: m._attend_planned(0, dq[-1][0], None, None), 50, torch)
     k_flops = 4.0 * T * frames * T * H * D
     return {"cpu_ms": t_cpu * 1e3, "cpu_gflops": flops / t_cpu * 1e-9, "gpu_ms": t_gpu * 1e3,
             "gpu_gflops": flops / t_gpu * 1e-9, "max_abs_diff": err, "tolerance": 1e-5,
             "kernel": {"name": "lbm_attn_f32_kernel<64>", "bound": "mfma", "achieved": k_flops / (k_ms * 1e-3) * 1e-12,
                        "peak": 157.3, "unit": "TFLOP/s", "frac": k_flops / (k_ms * 1e-3) * 1e-12 / 157.3,
                        "avg_launch_us": k_ms * 1e3, "flop_per_launch": k_flops,
-                       "what": "plan + attention of frame 8 (1004 x 8032 tokens), HIP events around 20 calls"},
+                       "what": "attention of frame 8 (1004 x 8032 tokens), HIP events around 50 launches after 20 warm-up launches"},
             "what": "8 frames, fp32, every frame attends to all frames so far (tables step + append + fp32 MFMA attention per frame, wall clock)"}
 
 
@@ -309,8 +312,8 @@ def main() -> None:
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-aggregator", action="store_true",
                     help="skip the full aggregator-trunk step (frame + global blocks) timed after the hot path")
-    ap.add_argument("--mode", choices=["full", "attention", "append", "prepare", "residual", "tables", "copy"], default="full",
-                    help="full = the benchmark line; attention/append/prepare/residual/tables launch one kernel --steps "
+    ap.add_argument("--mode", choices=["full", "attention", "attention_f32", "append", "prepare", "residual", "tables", "copy"], default="full",
+                    help="full = the benchmark line; attention/attention_f32/append/prepare/residual/tables launch one kernel --steps "
                          "times on the steady-state cache (for rocprofv3 runs); copy = a plain 256 MiB "
                          "device copy, the known-size kernel the HBM counters are calibrated on")
     args = ap.parse_args()
@@ -376,6 +379,23 @@ def main() -> None:
             m.step(b, qs[j], ks[j], vs[j], keyframe=[True], cross_frame_special=False)
 
     kv_tokens = (ANCHOR + WINDOW) * T
+    if args.mode == "attention_f32":
+        # config 1's last frame: 1004 fp32 queries over 8 cached frames (8032 tokens)
+        m32 = HipPagedKVCacheManager(1, 32, T, H, D, torch.float32, dev, num_special_tokens=N_SPECIAL, scale_frames=1,
+                                     sliding_window=16, max_total_frames=32, force_fp32=True, page_size=PAGE,
+                                     layout="frame_pages")
+        torch.manual_seed(0)
+        for _ in range(8):
+            m32.append_frame(0, torch.randn(T, H, D, device=dev) / 8, torch.randn(T, H, D, device=dev) / 8)
+        q32 = torch.randn(T, H, D, device=dev) / 8
+        m32._plan(0, [False])
+        fn = lambda: m32._attend_planned(0, q32, None, None)
+        for _ in range(args.warmup):
+            fn()
+        ms = event_time_ms(fn, args.steps, torch)
+        print(json.dumps({"mode": args.mode, "launches": args.steps, "avg_launch_us": ms * 1e3,
+                          "tflops": 4.0 * T * 8 * T * H * D / (ms * 1e-3) * 1e-12}))
+        return
     if args.mode != "full":
         # fill the anchor and the window with appends only, so that a profiler sees nothing
         # but --steps + --warmup launches of the one kernel at the steady-state shape

@@ -594,8 +594,8 @@ __global__ __launch_bounds__(256) void lbm_attn_combine_bf16_kernel(AttnArgs a) 
 // lingbot_map/layers/flashinfer_cache.py:118-127,372-383), head_dim 64, and 128 for the camera
 // head's one-token-per-frame cache (lingbot_map/heads/camera_head.py:284-377: 16 heads of 128).
 // Full fp32 products and sums on the matrix pipe (v_mfma_f32_16x16x4_f32), exact running
-// maximum, no split-KV across workgroups.  One workgroup per (64 query rows, head), two waves
-// per 16 query rows.
+// maximum, no split-KV across workgroups.  One workgroup per (64 query rows, head), four waves
+// (head_dim 64) or two (128) per 16 query rows.
 //
 // A lane is (n = lane % 16, g = lane / 16).  Scores are kept transposed, S^T = K Q^T: the
 // 16x16x4 product takes K[kv = n][dim k_g] from every lane as A and Q[q = n][dim k_g] as B and
@@ -627,26 +627,41 @@ struct AttnArgsF32 {
 };
 }  // namespace
 
+// Maximum over the four lanes n, n + 16, n + 32, n + 48 that share a query row, on the vector
+// ALU: v_permlane16_swap exchanges the odd 16-lane rows of one operand with the even rows of
+// the other, v_permlane32_swap the upper half of one with the lower half of the other; with
+// both operands equal to x the two results together hold x of the lane and of its partner.
+__device__ __forceinline__ float max_over_lane_groups(float x) {
+  const unsigned a = __builtin_bit_cast(unsigned, x);
+  const auto r = __builtin_amdgcn_permlane16_swap(a, a, false, false);
+  const float y = fmaxf(__builtin_bit_cast(float, r[0]), __builtin_bit_cast(float, r[1]));
+  const unsigned b = __builtin_bit_cast(unsigned, y);
+  const auto t = __builtin_amdgcn_permlane32_swap(b, b, false, false);
+  return fmaxf(__builtin_bit_cast(float, t[0]), __builtin_bit_cast(float, t[1]));
+}
+
 template <int D>
-__global__ __launch_bounds__(512) void lbm_attn_f32_kernel(AttnArgsF32 a) {
-  // Eight waves: wave w and wave w + 4 own the same 16 query rows and take alternate KV tiles
-  // (two waves per SIMD, so one's softmax and LDS waits overlap the other's matrix work); the
-  // two partial results are merged through LDS at the end.
-  constexpr int kTile = D == 64 ? 32 : 16;     // KV tokens per tile; two tiles are staged per iteration
-  constexpr int kRowThreads = D / 8;           // threads that stage one row: 8 floats of K and of V each
+__global__ __launch_bounds__(D == 64 ? 1024 : 512) void lbm_attn_f32_kernel(AttnArgsF32 a) {
+  // NG groups of four waves: wave w of every group owns the same 16 query rows, group j takes
+  // KV tiles j, j + NG, ... (NG waves per SIMD, so one wave's softmax, LDS waits and barriers
+  // overlap the others' matrix work); the partial results are merged through LDS at the end.
+  constexpr int NG = D == 64 ? 4 : 2;          // wave groups = tiles staged per iteration
+  constexpr int kThreadsF32 = 256 * NG;
+  constexpr int kTile = 16;                    // KV tokens per tile = one 16-token score block
+  constexpr int kStage = kTile * D / 256;      // floats of K (and of V) a thread stages per iteration
+  constexpr int kRowThreads = D / kStage;      // threads that stage one row
   constexpr int LD = D + 4;                    // LDS row stride: rows stay 16-byte aligned and shift by 4 banks
-  constexpr int NC = kTile / 16;               // 16-token score blocks per tile
   constexpr int NE = D / 16;                   // 16-dim output blocks
   constexpr int DG = D / 4;                    // head dims one lane group contributes to q.k
-  static_assert(512 / kRowThreads == 2 * kTile, "512 threads stage two tiles");
-  constexpr int kTileFloats = 2 * kTile * LD;   // two K tiles (and as many again for V)
-  constexpr int kMergeFloats = (NE * 4 + 2) * 256;
+  static_assert(kThreadsF32 / kRowThreads == NG * kTile && kStage % 4 == 0, "the threads stage NG tiles");
+  constexpr int kTileFloats = NG * kTile * LD;  // NG tiles of K (and as many again of V)
+  constexpr int kMergeFloats = (NE * 4 + 2) * 256 * (NG / 2);
   constexpr int kLdsFloats = 2 * kTileFloats > kMergeFloats ? 2 * kTileFloats : kMergeFloats;
   __shared__ __attribute__((aligned(16))) float lds_raw[kLdsFloats];
   float (*lds_k)[LD] = (float (*)[LD])lds_raw;
   float (*lds_v)[LD] = (float (*)[LD])(lds_raw + kTileFloats);
   const int tid = threadIdx.x;
-  const int lane = tid & 63, wave = (tid >> 6) & 3, half = tid >> 8;
+  const int lane = tid & 63, wave = (tid >> 6) & 3, grp = tid >> 8;
   const int n16 = lane & 15, g = lane >> 4;
   int b = 0;
   for (int i = 1; i < a.n_streams; ++i)
@@ -676,15 +691,21 @@ __global__ __launch_bounds__(512) void lbm_attn_f32_kernel(AttnArgsF32 a) {
   for (int e = 0; e < NE; ++e) o[e] = f32x4{0.f, 0.f, 0.f, 0.f};
   float m = -INFINITY, l = 0.f;   // running maximum of the row; this lane's share of the row sum
 
-  const int ld_r = tid / kRowThreads, ld_c = (tid % kRowThreads) * 8;
+  const int ld_r = tid / kRowThreads, ld_c = (tid % kRowThreads) * kStage;
   const int n_tiles = (sp.kv_tokens + kTile - 1) / kTile;
-  const int n_iters = (n_tiles + 1) / 2;
-  f32x4 kk[2], vv[2];
-  auto fetch = [&](int it) {
-    const int kvi = it * 2 * kTile + ld_r;
-    kk[0] = kk[1] = vv[0] = vv[1] = f32x4{0.f, 0.f, 0.f, 0.f};
-    if (kvi < sp.kv_tokens) {
-      const int e = a.kv_rows[sp.kv_row_begin + kvi];
+  const int n_iters = (n_tiles + NG - 1) / NG;
+  // Two-deep prefetch: the row-table entry of iteration it + 2 is requested while iteration it
+  // is computed, so the K/V loads of iteration it + 1 can be issued without waiting for it.
+  f32x4 kk[kStage / 4], vv[kStage / 4];
+  constexpr int kNoRow = INT32_MIN;   // not a row: past the end of the stream's KV
+  auto entry = [&](int it) -> int {
+    const int kvi = it * NG * kTile + ld_r;
+    return kvi < sp.kv_tokens ? a.kv_rows[sp.kv_row_begin + kvi] : kNoRow;
+  };
+  auto fetch = [&](int e) {
+#pragma unroll
+    for (int i = 0; i < kStage / 4; ++i) kk[i] = vv[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+    if (e != kNoRow) {
       const float *kp, *vp;
       if (e >= 0) {
         kp = a.pool + ((size_t)e * H + head) * D + ld_c;
@@ -694,110 +715,116 @@ __global__ __launch_bounds__(512) void lbm_attn_f32_kernel(AttnArgsF32 a) {
         kp = a.self_k + off;
         vp = a.self_v + off;
       }
-      kk[0] = ((const f32x4*)kp)[0];
-      kk[1] = ((const f32x4*)kp)[1];
-      vv[0] = ((const f32x4*)vp)[0];
-      vv[1] = ((const f32x4*)vp)[1];
+#pragma unroll
+      for (int i = 0; i < kStage / 4; ++i) {
+        kk[i] = ((const f32x4*)kp)[i];
+        vv[i] = ((const f32x4*)vp)[i];
+      }
     }
   };
-  if (n_iters > 0) fetch(0);
+  int e_next = kNoRow;
+  if (n_iters > 0) {
+    fetch(entry(0));
+    if (n_iters > 1) e_next = entry(1);
+  }
   for (int it = 0; it < n_iters; ++it) {
-    __syncthreads();  // the previous pair of tiles is no longer being read
-    *(f32x4*)&lds_k[ld_r][ld_c] = kk[0];
-    *(f32x4*)&lds_k[ld_r][ld_c + 4] = kk[1];
-    *(f32x4*)&lds_v[ld_r][ld_c] = vv[0];
-    *(f32x4*)&lds_v[ld_r][ld_c + 4] = vv[1];
-    __syncthreads();
-    if (it + 1 < n_iters) fetch(it + 1);   // in flight while this pair is computed
-    const int t = 2 * it + half;           // this wave's tile
-    if (t >= n_tiles) continue;            // odd tile count: the second half sits out the last pair
-    const int row0 = half * kTile;
-
-    // S^T blocks: sc[c][i] = score of kv token 16c + 4g + i of the tile for query row n16
-    f32x4 sc[NC];
+    __syncthreads();  // the previous tiles are no longer being read
 #pragma unroll
-    for (int c = 0; c < NC; ++c) sc[c] = f32x4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-    for (int d4 = 0; d4 < DG / 4; ++d4) {
-      f32x4 kf[NC];
-#pragma unroll
-      for (int c = 0; c < NC; ++c) kf[c] = *(const f32x4*)&lds_k[row0 + 16 * c + n16][DG * g + 4 * d4];
-#pragma unroll
-      for (int j = 0; j < 4; ++j)
-#pragma unroll
-        for (int c = 0; c < NC; ++c)
-          sc[c] = __builtin_amdgcn_mfma_f32_16x16x4f32(kf[c][j], q[4 * d4 + j], sc[c], 0, 0, 0);
+    for (int i = 0; i < kStage / 4; ++i) {
+      *(f32x4*)&lds_k[ld_r][ld_c + 4 * i] = kk[i];
+      *(f32x4*)&lds_v[ld_r][ld_c + 4 * i] = vv[i];
     }
+    __syncthreads();
+    if (it + 1 < n_iters) {                // in flight while these tiles are computed
+      fetch(e_next);
+      e_next = it + 2 < n_iters ? entry(it + 2) : kNoRow;
+    }
+    const int t = NG * it + grp;           // this wave's tile
+    if (t >= n_tiles) continue;            // the last iteration may not have a tile for every group
+    const int row0 = grp * kTile;
+
+    // S^T block: sc[i] = score of kv token 4g + i of the tile for query row n16
+    // every LDS operand of the tile is requested up front: the V reads complete under the
+    // score MFMAs instead of stalling each output MFMA
+    f32x4 kf[DG / 4];
+#pragma unroll
+    for (int d4 = 0; d4 < DG / 4; ++d4) kf[d4] = *(const f32x4*)&lds_k[row0 + n16][DG * g + 4 * d4];
+    float vf[4][NE];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int e = 0; e < NE; ++e) vf[i][e] = lds_v[row0 + 4 * g + i][16 * e + n16];
+    f32x4 sc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int d4 = 0; d4 < DG / 4; ++d4)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) sc = __builtin_amdgcn_mfma_f32_16x16x4f32(kf[d4][j], q[4 * d4 + j], sc, 0, 0, 0);
     const int n_valid = sp.kv_tokens - t * kTile;
     if (n_valid < kTile) {
 #pragma unroll
-      for (int c = 0; c < NC; ++c)
-#pragma unroll
-        for (int i = 0; i < 4; ++i)
-          if (16 * c + 4 * g + i >= n_valid) sc[c][i] = -INFINITY;
+      for (int i = 0; i < 4; ++i)
+        if (4 * g + i >= n_valid) sc[i] = -INFINITY;
     }
-    float mx = sc[0][0];
-#pragma unroll
-    for (int c = 0; c < NC; ++c)
-#pragma unroll
-      for (int i = 0; i < 4; ++i) mx = fmaxf(mx, sc[c][i]);
-    mx = fmaxf(mx, __shfl_xor(mx, 16));
-    mx = fmaxf(mx, __shfl_xor(mx, 32));
-    mx = fmaxf(mx, m);                      // finite: token 0 of every tile is valid
-    const float alpha = exp2f(m - mx);      // m = -inf on the first tile gives 0
+    float mx = fmaxf(fmaxf(sc[0], sc[1]), fmaxf(sc[2], sc[3]));
+    mx = max_over_lane_groups(mx);
+    mx = fmaxf(mx, m);                                    // finite: token 0 of every tile is valid
+    const float alpha = __builtin_amdgcn_exp2f(m - mx);   // m = -inf on the first tile gives 0
     m = mx;
     l *= alpha;
 #pragma unroll
     for (int e = 0; e < NE; ++e) o[e] *= alpha;
 #pragma unroll
-    for (int c = 0; c < NC; ++c)
+    for (int i = 0; i < 4; ++i) {
+      sc[i] = __builtin_amdgcn_exp2f(sc[i] - m);
+      l += sc[i];
+    }
+    // O^T += V^T P^T, contraction step i over kv = 4g + i
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const float p = exp2f(sc[c][i] - m);
-        sc[c][i] = p;
-        l += p;
-      }
-    // O^T += V^T P^T, contraction step (c, i) over kv = 16c + 4g + i
+    for (int i = 0; i < 4; ++i)
 #pragma unroll
-    for (int c = 0; c < NC; ++c)
-#pragma unroll
-      for (int i = 0; i < 4; ++i)
-#pragma unroll
-        for (int e = 0; e < NE; ++e)
-          o[e] = __builtin_amdgcn_mfma_f32_16x16x4f32(lds_v[row0 + 16 * c + 4 * g + i][16 * e + n16], sc[c][i], o[e], 0, 0, 0);
+      for (int e = 0; e < NE; ++e)
+        o[e] = __builtin_amdgcn_mfma_f32_16x16x4f32(vf[i][e], sc[i], o[e], 0, 0, 0);
   }
   l += __shfl_xor(l, 16);
   l += __shfl_xor(l, 32);
 
-  // merge the two halves: the second writes (o, m, l) per lane, the first rescales and adds
+  // merge the groups pairwise: the upper half of the remaining groups writes (o, m, l) per
+  // lane, the lower half rescales and adds; the last round normalises and stores
   float* merge = lds_raw;
   const int slot = tid & 255;
-  __syncthreads();
-  if (half == 1) {
 #pragma unroll
-    for (int e = 0; e < NE; ++e)
+  for (int stride = NG / 2; stride >= 1; stride /= 2) {
+    __syncthreads();
+    if (grp >= stride && grp < 2 * stride) {
+      float* mb = merge + (size_t)(grp - stride) * (NE * 4 + 2) * 256;
 #pragma unroll
-      for (int i = 0; i < 4; ++i) merge[(4 * e + i) * 256 + slot] = o[e][i];
-    merge[(4 * NE) * 256 + slot] = m;
-    merge[(4 * NE + 1) * 256 + slot] = l;
+      for (int e = 0; e < NE; ++e)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) mb[(4 * e + i) * 256 + slot] = o[e][i];
+      mb[(4 * NE) * 256 + slot] = m;
+      mb[(4 * NE + 1) * 256 + slot] = l;
+    }
+    __syncthreads();
+    if (grp < stride) {
+      const float* mb = merge + (size_t)grp * (NE * 4 + 2) * 256;
+      const float m1 = mb[(4 * NE) * 256 + slot], l1 = mb[(4 * NE + 1) * 256 + slot];
+      const float mt = fmaxf(m, m1);
+      // a group that saw no tile has m = -inf and contributes nothing
+      const float w0 = m > -INFINITY ? exp2f(m - mt) : 0.f;
+      const float w1 = m1 > -INFINITY ? exp2f(m1 - mt) : 0.f;
+      l = l * w0 + l1 * w1;
+      m = mt;
+#pragma unroll
+      for (int e = 0; e < NE; ++e)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) o[e][i] = o[e][i] * w0 + mb[(4 * e + i) * 256 + slot] * w1;
+    }
   }
-  __syncthreads();
-  if (half == 0 && row_ok) {
-    const float m1 = merge[(4 * NE) * 256 + slot], l1 = merge[(4 * NE + 1) * 256 + slot];
-    const float mt = fmaxf(m, m1);
-    // a half that saw no tile has m = -inf and contributes nothing; no KV at all leaves zeros
-    const float w0 = m > -INFINITY ? exp2f(m - mt) : 0.f;
-    const float w1 = m1 > -INFINITY ? exp2f(m1 - mt) : 0.f;
-    const float lt = l * w0 + l1 * w1;
-    const float inv = lt > 0.f ? 1.0f / lt : 0.f;
+  if (grp == 0 && row_ok) {
+    const float inv = l > 0.f ? 1.0f / l : 0.f;   // no KV at all leaves zeros
     float* op = a.out + ((size_t)(sp.q_begin + r) * H + head) * D + 4 * g;
 #pragma unroll
-    for (int e = 0; e < NE; ++e) {
-      f32x4 x;
-#pragma unroll
-      for (int i = 0; i < 4; ++i) x[i] = (o[e][i] * w0 + merge[(4 * e + i) * 256 + slot] * w1) * inv;
-      *(f32x4*)(op + 16 * e) = x;
-    }
+    for (int e = 0; e < NE; ++e) *(f32x4*)(op + 16 * e) = o[e] * inv;
   }
 }
 
@@ -977,7 +1004,7 @@ int lbm_launch_attention(const void* q, const void* pool, void* out, const void*
     }
     f.wg_begin[LBM_MAX_STREAMS] = wg;
     if (wg == 0) return LBM_OK;
-    if (head_dim == 64) hipLaunchKernelGGL(lbm_attn_f32_kernel<64>, dim3(wg), dim3(512), 0, stream, f);
+    if (head_dim == 64) hipLaunchKernelGGL(lbm_attn_f32_kernel<64>, dim3(wg), dim3(1024), 0, stream, f);
     else hipLaunchKernelGGL(lbm_attn_f32_kernel<128>, dim3(wg), dim3(512), 0, stream, f);
     return lbm_check_launch("lbm_attn_f32_kernel");
   }
