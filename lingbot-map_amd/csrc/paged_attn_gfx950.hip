@@ -606,8 +606,10 @@ __global__ __launch_bounds__(256) void lbm_attn_combine_bf16_kernel(AttnArgs a) 
 // ds_read_b128) and the Q operand a contiguous quarter row held in registers.  For O^T = V^T P^T
 // the same freedom is used on the KV index: step (c, i) contracts kv = 16c + 4g + i over g,
 // which is exactly where element i of the score block c already sits - P goes from the
-// accumulator into the B operand without a shuffle.  O^T[dim = 16e + 4g + i][q = n] ends up
-// as four consecutive dims per lane: 16-byte stores.
+// accumulator into the B operand without a shuffle.  Output block e takes head dimension
+// (D/16) n + e from lane n as its A operand (one ds_read_b128 of V per lane and KV row covers
+// four blocks), which leaves O^T[dim = (D/16)(4g + i) + e][q = n] in element i of block e:
+// consecutive dims across the blocks, 16-byte stores.
 namespace {
 constexpr int kF32Rows = 64;
 struct AttnArgsF32 {
@@ -749,11 +751,11 @@ __global__ __launch_bounds__(D == 64 ? 1024 : 512) void lbm_attn_f32_kernel(Attn
     f32x4 kf[DG / 4];
 #pragma unroll
     for (int d4 = 0; d4 < DG / 4; ++d4) kf[d4] = *(const f32x4*)&lds_k[row0 + n16][DG * g + 4 * d4];
-    float vf[4][NE];
+    f32x4 vf[4][NE / 4];
 #pragma unroll
     for (int i = 0; i < 4; ++i)
 #pragma unroll
-      for (int e = 0; e < NE; ++e) vf[i][e] = lds_v[row0 + 4 * g + i][16 * e + n16];
+      for (int h = 0; h < NE / 4; ++h) vf[i][h] = *(const f32x4*)&lds_v[row0 + 4 * g + i][NE * n16 + 4 * h];
     f32x4 sc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int d4 = 0; d4 < DG / 4; ++d4)
@@ -778,12 +780,12 @@ __global__ __launch_bounds__(D == 64 ? 1024 : 512) void lbm_attn_f32_kernel(Attn
       sc[i] = __builtin_amdgcn_exp2f(sc[i] - m);
       l += sc[i];
     }
-    // O^T += V^T P^T, contraction step i over kv = 4g + i
+    // O^T += V^T P^T, contraction step i over kv = 4g + i; block e holds dims NE * m + e
 #pragma unroll
     for (int i = 0; i < 4; ++i)
 #pragma unroll
       for (int e = 0; e < NE; ++e)
-        o[e] = __builtin_amdgcn_mfma_f32_16x16x4f32(vf[i][e], sc[i], o[e], 0, 0, 0);
+        o[e] = __builtin_amdgcn_mfma_f32_16x16x4f32(vf[i][e / 4][e % 4], sc[i], o[e], 0, 0, 0);
   }
   l += __shfl_xor(l, 16);
   l += __shfl_xor(l, 32);
@@ -822,9 +824,13 @@ __global__ __launch_bounds__(D == 64 ? 1024 : 512) void lbm_attn_f32_kernel(Attn
   }
   if (grp == 0 && row_ok) {
     const float inv = l > 0.f ? 1.0f / l : 0.f;   // no KV at all leaves zeros
-    float* op = a.out + ((size_t)(sp.q_begin + r) * H + head) * D + 4 * g;
+    float* op = a.out + ((size_t)(sp.q_begin + r) * H + head) * D + NE * 4 * g;
 #pragma unroll
-    for (int e = 0; e < NE; ++e) *(f32x4*)(op + 16 * e) = o[e] * inv;
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int h = 0; h < NE / 4; ++h)
+        *(f32x4*)(op + NE * i + 4 * h) =
+            f32x4{o[4 * h][i], o[4 * h + 1][i], o[4 * h + 2][i], o[4 * h + 3][i]} * inv;
   }
 }
 
