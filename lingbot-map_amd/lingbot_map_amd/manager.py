@@ -330,7 +330,8 @@ class HipPagedKVCacheManager:
                 rows = self._rows_log.get(n)
                 if rows is None:
                     raise RuntimeError(f"block {block_idx} has made {n} appends, block 0 {lead}, and the rows of "
-                                       "that frame are no longer known (evicted or rolled back in between)")
+                                       "that frame are no longer known (block 0 evicted or rolled back in between); blocks that "
+                                       "run that far apart need per_block_tables=True")
         self._scatter(block_idx, rows, k, v)
         self.frame_count[block_idx] += 1
         self._n_appends[block_idx] += 1
