@@ -124,6 +124,49 @@ def attention_shapes(torch) -> list:
     ]
 
 
+def hbm_kernels_4_streams(torch) -> dict:
+    """The three HBM-bound kernels at config 5's batch (four streams in one launch, 4,016 rows):
+    the single-stream launches of 8-13 MB are as much launch ramp as stream."""
+    import ctypes as C
+    from lingbot_map_amd import HipPagedKVCacheManager
+    from lingbot_map_amd import _native as N
+    dev = torch.device("cuda:0")
+    B = 4
+    g = torch.Generator(device=dev).manual_seed(6)
+    rnd = lambda *shape: torch.randn(*shape, generator=g, device=dev, dtype=torch.float32).to(torch.bfloat16)
+    m = HipPagedKVCacheManager(1, 8, T, H, D, torch.bfloat16, dev, num_special_tokens=N_SPECIAL, scale_frames=1,
+                               sliding_window=2, max_total_frames=16, page_size=PAGE, layout="frame_pages", num_streams=B)
+    k, v, qkv = rnd(B * T, H, D), rnd(B * T, H, D), rnd(B * T, 3 * H * D)
+    m.append_frame(0, k, v)     # leaves the rows of one frame per stream in the append plan
+    vp = lambda t: C.c_void_p(t.data_ptr())
+    ln = [torch.rand(D, generator=g, device=dev) + 0.5 for _ in range(4)]
+    ang = torch.rand(B * T, D // 2, generator=g, device=dev) * 6.283185
+    cs = torch.stack([ang.cos(), ang.sin()], dim=-1).contiguous()
+    q_out = torch.empty(B * T, H, D, dtype=torch.bfloat16, device=dev)
+    x, y = rnd(B * T, H * D), rnd(B * T, H * D)
+    par = [torch.rand(H * D, generator=g, device=dev) + 0.5 for _ in range(3)]
+    outs = [torch.empty_like(x) for _ in range(2)]
+    stream = lambda: m._stream_handle()
+    fns = {
+        "append": (lambda: m._scatter(0, m._append_rows[0], k, v), 2 * 2 * B * T * H * D * 2),
+        "qkv_prepare": (lambda: N.check(N.lib.lbm_qkv_prepare(
+            vp(qkv), N.DTYPE_BF16, vp(ln[0]), vp(ln[1]), vp(ln[2]), vp(ln[3]), 1e-5, vp(cs), N.ROPE_INTERLEAVED, vp(q_out),
+            None, None, N.DTYPE_BF16, vp(m.kv_caches[0]), vp(m._append_rows[0]), B * T, H, D, PAGE, stream())),
+            6 * B * T * H * D * 2 + cs.numel() * 4),
+        "residual_norm": (lambda: N.check(N.lib.lbm_residual_norm(
+            vp(x), vp(y), N.DTYPE_BF16, vp(par[0]), vp(par[1]), vp(par[2]), 1e-5, vp(outs[0]), vp(outs[1]), B * T, H * D,
+            stream())), 4 * B * T * H * D * 2),
+    }
+    res = {}
+    for name, (fn, nbytes) in fns.items():
+        ms = kernel_time_ms(fn, 100, torch)
+        gbps = nbytes / (ms * 1e-3) * 1e-9
+        res[name] = {"bytes_per_launch": nbytes, "avg_launch_us": ms * 1e3, "achieved": gbps, "unit": "GB/s",
+                     "frac": gbps / PEAK_HBM_GBPS}
+    assert m.device_header()["error"] == 0
+    return res
+
+
 def config1(torch) -> dict:
     """Config 1, the CPU-runnable parity case: fp32, 8 frames of 1004 tokens, Q, K, V =
     randn / 8 with seed 0, frame i attends to frames 0..i (148.6 GFLOP in all).  The oracle's
@@ -474,6 +517,7 @@ def main() -> None:
                           "what": "x + ls(y) fused with the following LayerNorm, 1004 x 1024 bf16 (not in `value`'s timed loop)"},
         "tables_step_us": tables_ms * 1e3,
         "attention_shapes": attention_shapes(torch),
+        "hbm_kernels_4_streams": hbm_kernels_4_streams(torch),
     }
     if not args.no_aggregator:
         del m
