@@ -28,8 +28,8 @@ PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA
 PEAK_HBM_GBPS = 8000.0
 # HBM bytes of one lbm_attn_bf16_d64_kernel launch at this workload, from rocprofv3 --pmc
 # FETCH_SIZE (x2.0, the factor a 256 MiB plain copy gives) and WRITE_SIZE (x1.0), in KiB:
-# 35,492 * 2 + 20,082 KiB  (profiles/attention_config2_hbm_traffic.md)
-ATTN_TRAFFIC_BYTES = (35492.0 * 2.0 + 20082.0) * 1024.0
+# 35,738 * 2 + 20,592 KiB  (profiles/attention_config2_hbm_traffic.md)
+ATTN_TRAFFIC_BYTES = (35738.0 * 2.0 + 20592.0) * 1024.0
 METRIC = "frames/sec streaming @518x378 (1 GPU); attention TFLOPS & % bf16 MFMA peak"
 
 
