@@ -5,8 +5,9 @@
 // One pass over the rows instead of three elementwise / normalisation kernels.  HBM-bound:
 // reads x and y once, writes x_out and n_out once.
 //
-// One 128-thread workgroup per row; a thread owns 8 consecutive elements per 1024-element
-// chunk of the row (up to 8 chunks), kept in registers between the statistics and the output.
+// Rows of up to 2048 elements take one wavefront each (butterfly sums, no LDS); longer rows one
+// 128-thread workgroup: a thread owns 8 consecutive elements per 1024-element chunk of the row
+// (up to 8 chunks).  Either way the row stays in registers between the statistics and the output.
 // Rounding follows torch for bf16 activations: y * gamma rounded to bf16, the sum rounded to
 // bf16, the LayerNorm computed in fp32 on those bf16 values (two-pass mean / variance) and
 // rounded once.  For fp32 activations every step is a separately rounded fp32 operation.
@@ -80,16 +81,17 @@ struct ResidualNormArgs {
   int rows, cols;
 };
 
-template <int DT>
+// NCH = 1024-element chunks a row may have (1, 2, 4 or 8): sizes the register array
+template <int DT, int NCH>
 __global__ __launch_bounds__(kThreads) void lbm_residual_norm_kernel(ResidualNormArgs a) {
   __shared__ float lds2[2];
   const int row = blockIdx.x;
   const long long base = (long long)row * a.cols;
   const int n_chunks = (a.cols + 1023) >> 10;
-  float v[kMaxChunks][8];
+  float v[NCH][8];
   float sum = 0.f;
 #pragma unroll
-  for (int c = 0; c < kMaxChunks; ++c) {
+  for (int c = 0; c < NCH; ++c) {
     const int col = c * 1024 + threadIdx.x * 8;
     if (c < n_chunks && col < a.cols) {
       float x[8], y[8];
@@ -113,7 +115,7 @@ __global__ __launch_bounds__(kThreads) void lbm_residual_norm_kernel(ResidualNor
   const float mean = block_sum(sum, lds2) / (float)a.cols;
   float sq = 0.f;
 #pragma unroll
-  for (int c = 0; c < kMaxChunks; ++c) {
+  for (int c = 0; c < NCH; ++c) {
     const int col = c * 1024 + threadIdx.x * 8;
     if (c < n_chunks && col < a.cols) {
 #pragma unroll
@@ -122,9 +124,68 @@ __global__ __launch_bounds__(kThreads) void lbm_residual_norm_kernel(ResidualNor
   }
   const float rstd = __builtin_amdgcn_rsqf(block_sum(sq, lds2) / (float)a.cols + a.eps);
 #pragma unroll
-  for (int c = 0; c < kMaxChunks; ++c) {
+  for (int c = 0; c < NCH; ++c) {
     const int col = c * 1024 + threadIdx.x * 8;
     if (c < n_chunks && col < a.cols) {
+      float o[8];
+#pragma unroll
+      for (int i = 0; i < 8; ++i)
+        o[i] = __fadd_rn(__fmul_rn(__fmul_rn(v[c][i] - mean, rstd), a.norm_w[col + i]), a.norm_b[col + i]);
+      store8<DT>(a.n_out, base + col, o);
+    }
+  }
+}
+
+// Rows of up to 2048 elements: one wavefront per row, four rows per workgroup.  A lane owns 8
+// consecutive elements per 512-element chunk (NV chunks), the two statistics are butterfly
+// sums over the 64 lanes - no LDS, no barrier.
+template <int DT, int NV>
+__global__ __launch_bounds__(256) void lbm_residual_norm_wave_kernel(ResidualNormArgs a) {
+  const int lane = threadIdx.x & 63;
+  const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= a.rows) return;   // whole wavefronts leave; nothing below synchronises across them
+  const long long base = (long long)row * a.cols;
+  float v[NV][8];
+  float sum = 0.f;
+#pragma unroll
+  for (int c = 0; c < NV; ++c) {
+    const int col = (c * 64 + lane) * 8;
+    if (col < a.cols) {
+      float x[8], y[8];
+      load8<DT>(a.x, base + col, x);
+      load8<DT>(a.y, base + col, y);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        float t = y[i];
+        if (a.gamma) t = DT == 0 ? round_bf16(__fmul_rn(t, a.gamma[col + i])) : __fmul_rn(t, a.gamma[col + i]);
+        const float s = __fadd_rn(x[i], t);
+        v[c][i] = DT == 0 ? round_bf16(s) : s;
+        sum += v[c][i];
+      }
+      store8<DT>(a.x_out, base + col, v[c]);
+    } else {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) v[c][i] = 0.f;
+    }
+  }
+  if (!a.norm_w) return;  // uniform: a launch parameter
+#pragma unroll
+  for (int o = 32; o >= 1; o >>= 1) sum += __shfl_xor(sum, o);
+  const float mean = sum / (float)a.cols;
+  float sq = 0.f;
+#pragma unroll
+  for (int c = 0; c < NV; ++c)
+    if ((c * 64 + lane) * 8 < a.cols) {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) sq += (v[c][i] - mean) * (v[c][i] - mean);
+    }
+#pragma unroll
+  for (int o = 32; o >= 1; o >>= 1) sq += __shfl_xor(sq, o);
+  const float rstd = __builtin_amdgcn_rsqf(sq / (float)a.cols + a.eps);
+#pragma unroll
+  for (int c = 0; c < NV; ++c) {
+    const int col = (c * 64 + lane) * 8;
+    if (col < a.cols) {
       float o[8];
 #pragma unroll
       for (int i = 0; i < 8; ++i)
@@ -144,7 +205,35 @@ int lbm_launch_residual_norm(const void* x, const void* y, int dtype, const floa
     return lbm_fail(LBM_ERR_UNSUPPORTED, "lbm_residual_norm: cols must be a multiple of 8 and at most %d (got %d)",
                     1024 * kMaxChunks, cols);
   ResidualNormArgs a{x, y, gamma, norm_w, norm_b, x_out, n_out, eps, rows, cols};
-  if (dtype == LBM_DTYPE_BF16) hipLaunchKernelGGL(lbm_residual_norm_kernel<0>, dim3(rows), dim3(kThreads), 0, stream, a);
-  else hipLaunchKernelGGL(lbm_residual_norm_kernel<1>, dim3(rows), dim3(kThreads), 0, stream, a);
+  if (cols <= 2048) {
+    const int nv = (cols + 511) >> 9;
+    const dim3 grid((rows + 3) / 4);
+#define LBM_RN_WAVE(DT, NV) hipLaunchKernelGGL((lbm_residual_norm_wave_kernel<DT, NV>), grid, dim3(256), 0, stream, a)
+    if (dtype == LBM_DTYPE_BF16) {
+      if (nv <= 1) LBM_RN_WAVE(0, 1);
+      else if (nv <= 2) LBM_RN_WAVE(0, 2);
+      else LBM_RN_WAVE(0, 4);
+    } else {
+      if (nv <= 1) LBM_RN_WAVE(1, 1);
+      else if (nv <= 2) LBM_RN_WAVE(1, 2);
+      else LBM_RN_WAVE(1, 4);
+    }
+#undef LBM_RN_WAVE
+    return lbm_check_launch("lbm_residual_norm_wave_kernel");
+  }
+  const int n_chunks = (cols + 1023) >> 10;
+#define LBM_RN_LAUNCH(DT, NCH) hipLaunchKernelGGL((lbm_residual_norm_kernel<DT, NCH>), dim3(rows), dim3(kThreads), 0, stream, a)
+  if (dtype == LBM_DTYPE_BF16) {
+    if (n_chunks <= 1) LBM_RN_LAUNCH(0, 1);
+    else if (n_chunks <= 2) LBM_RN_LAUNCH(0, 2);
+    else if (n_chunks <= 4) LBM_RN_LAUNCH(0, 4);
+    else LBM_RN_LAUNCH(0, 8);
+  } else {
+    if (n_chunks <= 1) LBM_RN_LAUNCH(1, 1);
+    else if (n_chunks <= 2) LBM_RN_LAUNCH(1, 2);
+    else if (n_chunks <= 4) LBM_RN_LAUNCH(1, 4);
+    else LBM_RN_LAUNCH(1, 8);
+  }
+#undef LBM_RN_LAUNCH
   return lbm_check_launch("lbm_residual_norm_kernel");
 }

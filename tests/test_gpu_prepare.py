@@ -186,7 +186,7 @@ def test_prepare_half_split_rope_matches_oracle(dtype):
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
-@pytest.mark.parametrize("rows,C", [(3, 256), (1004, 1024), (17, 2048 + 8)])
+@pytest.mark.parametrize("rows,C", [(3, 256), (1004, 1024), (6, 1536), (5, 2048), (17, 2048 + 8), (2, 8192)])
 def test_residual_norm_matches_oracle(dtype, rows, C):
     """x + y * gamma and the LayerNorm of it in one kernel.  bf16: x_out bit-exact (products and
     sums rounded where torch rounds them), the LayerNorm within one bf16 ulp; fp32: 2e-6."""
