@@ -167,6 +167,59 @@ def hbm_kernels_4_streams(torch) -> dict:
     return res
 
 
+def camera_head_cache(torch) -> dict:
+    """The camera head's cache traffic of one streamed frame (lingbot_map/heads/camera_head.py:296-346,
+    lingbot_map/layers/attention.py:224-349): 4 refinement iterations x 4 trunk blocks, each with
+    its own cache of one 16 x 128 fp32 token per frame, nothing evicted.  One manager with 16
+    blocks holds them; a frame is 16 x (append + attend).  Beside it the reference's scheme in
+    plain PyTorch on the same GPU: concatenate the new token to the block's K and V, clone
+    both, SDPA with an all-true mask."""
+    from lingbot_map_amd import HipPagedKVCacheManager
+    dev = torch.device("cuda:0")
+    Hc, Dc, blocks, cached, timed = 16, 128, 16, 300, 50
+    m = HipPagedKVCacheManager(blocks, cached + timed + 8, 1, Hc, Dc, torch.float32, dev, num_special_tokens=0,
+                               scale_frames=8, sliding_window=cached + timed, max_total_frames=cached + timed + 8,
+                               force_fp32=True, page_size=16, layout="frame_pages")
+    g = torch.Generator(device=dev).manual_seed(8)
+    qkv = [torch.randn(1, Hc, Dc, generator=g, device=dev) for _ in range(3)]
+    dict_k = [torch.randn(1, Hc, cached, 1, Dc, generator=g, device=dev) for _ in range(blocks)]
+    dict_v = [torch.randn(1, Hc, cached, 1, Dc, generator=g, device=dev) for _ in range(blocks)]
+
+    def frame_hip():
+        for b in range(blocks):
+            out = m.step(b, qkv[0], qkv[1], qkv[2], keyframe=[True], cross_frame_special=False)
+        return out
+
+    def frame_dict():
+        q = qkv[0].permute(1, 0, 2)[None]                        # [1, H, 1, D]
+        for b in range(blocks):
+            dict_k[b] = torch.cat((dict_k[b], qkv[1].view(1, Hc, 1, 1, Dc)), dim=2)
+            dict_v[b] = torch.cat((dict_v[b], qkv[2].view(1, Hc, 1, 1, Dc)), dim=2)
+            k = dict_k[b].clone().reshape(1, Hc, -1, Dc)
+            v = dict_v[b].clone().reshape(1, Hc, -1, Dc)
+            mask = torch.ones(1, 1, 1, k.shape[2], dtype=torch.bool, device=dev)
+            out = torch.nn.functional.scaled_dot_product_attention(q, k, v, attn_mask=mask)
+        return out
+
+    for _ in range(cached):
+        frame_hip()
+    res = {}
+    for name, fn in (("hip_paged", frame_hip), ("torch_dict_cache", frame_dict)):
+        for _ in range(5):
+            fn()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(timed - 5):
+            out = fn()
+        torch.cuda.synchronize()
+        res[name + "_us_per_frame"] = (time.perf_counter() - t0) / (timed - 5) * 1e6
+        assert torch.isfinite(out).all()
+    assert m.device_header()["error"] == 0
+    res["what"] = (f"{blocks} caches x (append one token + attend to ~{cached + timed // 2} cached tokens), 16 heads of 128, fp32, "
+                   "wall clock per frame including the host's launches")
+    return res
+
+
 def config1(torch) -> dict:
     """Config 1, the CPU-runnable parity case: fp32, 8 frames of 1004 tokens, Q, K, V =
     randn / 8 with seed 0, frame i attends to frames 0..i (148.6 GFLOP in all).  The oracle's
@@ -518,6 +571,7 @@ def main() -> None:
         "tables_step_us": tables_ms * 1e3,
         "attention_shapes": attention_shapes(torch),
         "hbm_kernels_4_streams": hbm_kernels_4_streams(torch),
+        "camera_head_cache": camera_head_cache(torch),
     }
     if not args.no_aggregator:
         del m
