@@ -217,6 +217,23 @@ def camera_head_cache(torch) -> dict:
     assert m.device_header()["error"] == 0
     res["what"] = (f"{blocks} caches x (append one token + attend to ~{cached + timed // 2} cached tokens), 16 heads of 128, fp32, "
                    "wall clock per frame including the host's launches")
+    # the same attention after 10,000 frames (the head never evicts): one launch, K/V read once
+    del m
+    long_frames = 10000
+    ml = HipPagedKVCacheManager(1, long_frames + 16, 1, Hc, Dc, torch.float32, dev, num_special_tokens=0, scale_frames=8,
+                                sliding_window=long_frames + 8, max_total_frames=long_frames + 16, force_fp32=True,
+                                page_size=16, layout="frame_pages")
+    for _ in range(long_frames):
+        ml.append_frame(0, qkv[1], qkv[2])
+    ml._plan(0, [False])
+    for _ in range(10):
+        ml._attend_planned(0, qkv[0], None, None)
+    ms = event_time_ms(lambda: ml._attend_planned(0, qkv[0], None, None), 50, torch)
+    nbytes = long_frames * Hc * Dc * 4 * 2
+    res["attend_10000_frames"] = {"avg_launch_us": ms * 1e3, "bytes_per_launch": nbytes, "bound": "hbm",
+                                  "achieved": nbytes / (ms * 1e-3) * 1e-9, "unit": "GB/s",
+                                  "frac": nbytes / (ms * 1e-3) * 1e-9 / PEAK_HBM_GBPS,
+                                  "what": "one query token over 10,000 cached tokens (few-query fp32 kernels: chunked KV + merge)"}
     return res
 
 

@@ -209,7 +209,9 @@ int lbm_qkv_prepare(const void* qkv, int32_t src_dtype, const float* q_norm_w,
                     const int32_t* append_rows, int32_t n_tokens, int32_t num_heads,
                     int32_t head_dim, int32_t page_size, void* stream);
 
-/* Bytes of workspace lbm_attn_run needs for this batch (split-KV partial results). */
+/* Bytes of workspace lbm_attn_run needs for this batch: the split-KV partial results of the
+ * bf16 kernel or, when every stream has at most 8 query rows, the per-chunk partials of the
+ * fp32 few-query kernels, whichever is larger (the query does not take the dtype). */
 size_t lbm_attn_workspace_bytes(const lbm_attn_stream* streams, int32_t n_streams,
                                 int32_t num_heads, int32_t head_dim);
 

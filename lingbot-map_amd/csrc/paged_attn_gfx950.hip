@@ -88,6 +88,15 @@ __device__ __forceinline__ void swap_halves(float x, float& lo, float& hi) {
   lo = a;
   hi = b;
 }
+// The same for neighbouring rows of 16 lanes: v_permlane16_swap swaps the odd rows of its first
+// register with the even rows of its second; fed two copies of x it leaves rows {0, 0, 2, 2}
+// in the first and rows {1, 1, 3, 3} in the second.
+__device__ __forceinline__ void swap_rows(float x, float& even, float& odd) {
+  float a = x, b = x;
+  asm("s_nop 1\n\tv_permlane16_swap_b32 %0, %1" : "+v"(a), "+v"(b));
+  even = a;
+  odd = b;
+}
 // Built with -fno-honor-nans, fmaxf chains become v_max3_f32 without NaN-quieting moves.
 __device__ __forceinline__ float max3(float a, float b, float c) { return fmaxf(fmaxf(a, b), c); }
 __device__ __forceinline__ float max2(float a, float b) { return fmaxf(a, b); }
@@ -630,16 +639,13 @@ struct AttnArgsF32 {
 }  // namespace
 
 // Maximum over the four lanes n, n + 16, n + 32, n + 48 that share a query row, on the vector
-// ALU: v_permlane16_swap exchanges the odd 16-lane rows of one operand with the even rows of
-// the other, v_permlane32_swap the upper half of one with the lower half of the other; with
-// both operands equal to x the two results together hold x of the lane and of its partner.
+// ALU (no LDS round trip): rows of 16 lanes pairwise, then the two halves of the wavefront.
 __device__ __forceinline__ float max_over_lane_groups(float x) {
-  const unsigned a = __builtin_bit_cast(unsigned, x);
-  const auto r = __builtin_amdgcn_permlane16_swap(a, a, false, false);
-  const float y = fmaxf(__builtin_bit_cast(float, r[0]), __builtin_bit_cast(float, r[1]));
-  const unsigned b = __builtin_bit_cast(unsigned, y);
-  const auto t = __builtin_amdgcn_permlane32_swap(b, b, false, false);
-  return fmaxf(__builtin_bit_cast(float, t[0]), __builtin_bit_cast(float, t[1]));
+  float a, b;
+  swap_rows(x, a, b);
+  x = fmaxf(a, b);
+  swap_halves(x, a, b);
+  return fmaxf(a, b);
 }
 
 template <int D>
@@ -834,6 +840,186 @@ __global__ __launch_bounds__(D == 64 ? 1024 : 512) void lbm_attn_f32_kernel(Attn
   }
 }
 
+// ---------------------------------------------------------------------------- fp32, few queries
+// Streams with at most kDecQ query rows (the camera head: one token per frame attending to
+// every frame so far, lingbot_map/heads/camera_head.py:296-346) are bound by reading K and V
+// once, not by arithmetic, and have far too few rows for the matrix kernel's (64 rows, head)
+// workgroups to fill the chip.  Here the KV range of a (stream, head) is cut into n_chunks
+// pieces, one workgroup per piece and query row; a workgroup walks its piece in blocks of 256
+// tokens: scores by fp32 dot products (D/4 lanes per K row, 16 bytes each, summed with DPP
+// steps), block maximum and exp2 through LDS, then the V rows of the block weighted into the
+// output accumulator, with the usual running-maximum rescale between blocks.  Each workgroup
+// leaves one partial (maximum, sum, unnormalised output); a second small kernel merges them.
+namespace {
+constexpr int kDecQ = 8;         // query rows per stream this path takes
+constexpr int kDecBlock = 256;   // tokens a workgroup handles between two softmax updates
+constexpr int kDecMaxChunks = 64;
+
+struct DecodeArgs {
+  AttnArgsF32 f;
+  float* part;                           // [sum n_chunks][q_rows][H][D + 2]
+  int n_chunks[LBM_MAX_STREAMS];
+  int part_begin[LBM_MAX_STREAMS];       // in (chunk, query row) units
+  int max_q;                             // most query rows of any stream
+};
+
+__device__ __forceinline__ float block_reduce_256(float v, bool is_max, float* red) {
+#pragma unroll
+  for (int o = 32; o >= 1; o >>= 1) {
+    const float w = __shfl_xor(v, o);
+    v = is_max ? fmaxf(v, w) : v + w;
+  }
+  __syncthreads();   // red may still be read from the previous reduction
+  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
+  __syncthreads();
+  return is_max ? fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3])) : (red[0] + red[1]) + (red[2] + red[3]);
+}
+}  // namespace
+
+// sum over the LPR = D/4 lanes that share a K row, on the vector ALU: four DPP steps inside a
+// row of 16 lanes, and for 32-lane groups one exchange between neighbouring rows
+template <int LPR>
+__device__ __forceinline__ float row_group_sum(float v) {
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0xB1, 0xf, 0xf, false));   // quad_perm [1,0,3,2]
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x4E, 0xf, 0xf, false));   // quad_perm [2,3,0,1]
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x141, 0xf, 0xf, false));  // row_half_mirror
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x140, 0xf, 0xf, false));  // row_mirror
+  if (LPR == 32) {
+    float even, odd;
+    swap_rows(v, even, odd);
+    v = even + odd;
+  }
+  return v;
+}
+
+// grid: x = chunk of the KV axis, y = head, z = stream * max_q + query row
+template <int D>
+__global__ __launch_bounds__(256) void lbm_attn_f32_decode_kernel(DecodeArgs a) {
+  constexpr int LPR = D / 4;         // lanes per K/V row, 16 bytes each
+  constexpr int RPP = 256 / LPR;     // rows per pass of the workgroup
+  constexpr int NPASS = kDecBlock / RPP;
+  constexpr int kBatch = 8;          // rows per lane in flight
+  __shared__ float sc[kDecBlock];               // scores, then numerators, of the block
+  __shared__ __attribute__((aligned(16))) float acc_red[RPP][D];   // per row-group partial outputs
+  __shared__ float red[4];
+  const int tid = threadIdx.x;
+  const int b = blockIdx.z / a.max_q, qi = blockIdx.z % a.max_q, head = blockIdx.y, chunk = blockIdx.x;
+  lbm_attn_stream sp = a.f.s[b];
+  if (chunk >= a.n_chunks[b] || qi >= sp.q_rows) return;
+  if (a.f.live_kv_tokens) sp.kv_tokens = max(a.f.live_kv_tokens[sp.live_at], 0);
+  const int H = a.f.num_heads;
+  const size_t row_elems = (size_t)H * D;
+  // this workgroup's piece of the KV axis, a whole number of blocks
+  const int per = ((sp.kv_tokens + a.n_chunks[b] - 1) / a.n_chunks[b] + kDecBlock - 1) / kDecBlock * kDecBlock;
+  const int t_begin = chunk * per, t_end = min(t_begin + per, sp.kv_tokens);
+  const int grp = tid / LPR, ln = tid % LPR;   // row group of a pass, lane within the row
+
+  const f32x4 q4 = *(const f32x4*)(a.f.q + ((size_t)(sp.q_begin + qi) * H + head) * D + 4 * ln) * a.f.scale_log2;
+  f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+  float m_run = -INFINITY, l_run = 0.f;
+
+  auto row_ptr = [&](int token, bool want_v) -> const float* {
+    const int e = a.f.kv_rows[sp.kv_row_begin + token];
+    if (e >= 0) return a.f.pool + ((size_t)e * H + head) * D + 4 * ln + (want_v ? (size_t)a.f.page_size * row_elems : 0);
+    return (want_v ? a.f.self_v : a.f.self_k) + ((size_t)(-1 - e) * H + head) * D + 4 * ln;
+  };
+
+  for (int t0 = t_begin; t0 < t_end; t0 += kDecBlock) {
+    // ---- scores of the block, kBatch rows per lane in flight
+    __syncthreads();   // sc of the previous block is no longer read
+#pragma unroll 1
+    for (int pb = 0; pb < NPASS; pb += kBatch) {
+      f32x4 kx[kBatch];
+#pragma unroll
+      for (int p = 0; p < kBatch; ++p) {
+        const int token = t0 + (pb + p) * RPP + grp;
+        kx[p] = token < t_end ? *(const f32x4*)row_ptr(token, false) : f32x4{0.f, 0.f, 0.f, 0.f};
+      }
+#pragma unroll
+      for (int p = 0; p < kBatch; ++p) {
+        const int local = (pb + p) * RPP + grp;
+        const float d = row_group_sum<LPR>(kx[p][0] * q4[0] + kx[p][1] * q4[1] + kx[p][2] * q4[2] + kx[p][3] * q4[3]);
+        if (ln == 0) sc[local] = t0 + local < t_end ? d : -INFINITY;
+      }
+    }
+    __syncthreads();
+    // ---- running maximum, numerators, running sum (thread tid owns token tid of the block)
+    const float s = sc[tid];
+    const float m_new = fmaxf(m_run, block_reduce_256(s, true, red));   // finite: token t0 is valid
+    const float pr = exp2f(s - m_new);
+    sc[tid] = pr;
+    const float alpha = exp2f(m_run - m_new);   // 0 on the first block
+    l_run = l_run * alpha + block_reduce_256(pr, false, red);
+    m_run = m_new;
+    __syncthreads();
+    // ---- weighted V rows
+    acc *= alpha;
+#pragma unroll 1
+    for (int pb = 0; pb < NPASS; pb += kBatch) {
+      f32x4 vx[kBatch];
+#pragma unroll
+      for (int p = 0; p < kBatch; ++p) {
+        const int token = t0 + (pb + p) * RPP + grp;
+        vx[p] = token < t_end ? *(const f32x4*)row_ptr(token, true) : f32x4{0.f, 0.f, 0.f, 0.f};
+      }
+#pragma unroll
+      for (int p = 0; p < kBatch; ++p) acc += vx[p] * sc[(pb + p) * RPP + grp];
+    }
+  }
+  // ---- sum the row groups' accumulators, write the partial
+  *(f32x4*)&acc_red[grp][4 * ln] = acc;
+  __syncthreads();
+  if (tid < D) {
+    float o = 0.f;
+#pragma unroll
+    for (int r = 0; r < RPP; ++r) o += acc_red[r][tid];
+    float* pp = a.part + (((size_t)a.part_begin[b] + (size_t)chunk * sp.q_rows + qi) * H + head) * (D + 2);
+    pp[tid] = o;
+    if (tid == 0) {
+      pp[D] = m_run;       // identical in every thread
+      pp[D + 1] = l_run;
+    }
+  }
+}
+
+// one workgroup of D threads per (stream, query row, head): merge the chunks' partials
+template <int D>
+__global__ __launch_bounds__(D) void lbm_attn_f32_decode_merge_kernel(DecodeArgs a) {
+  const int b = blockIdx.z, head = blockIdx.y, qi = blockIdx.x, d = threadIdx.x;
+  const lbm_attn_stream sp = a.f.s[b];
+  if (qi >= sp.q_rows) return;
+  const int H = a.f.num_heads, nc = a.n_chunks[b];
+  float m = -INFINITY;
+  for (int c = 0; c < nc; ++c)
+    m = fmaxf(m, a.part[(((size_t)a.part_begin[b] + (size_t)c * sp.q_rows + qi) * H + head) * (D + 2) + D]);
+  float o = 0.f, l = 0.f;
+  for (int c = 0; c < nc; ++c) {
+    const float* pp = a.part + (((size_t)a.part_begin[b] + (size_t)c * sp.q_rows + qi) * H + head) * (D + 2);
+    const float w = pp[D] > -INFINITY ? exp2f(pp[D] - m) : 0.f;   // a chunk without tokens weighs nothing
+    o += pp[d] * w;
+    l += pp[D + 1] * w;
+  }
+  a.f.out[((size_t)(sp.q_begin + qi) * H + head) * D + d] = l > 0.f ? o / l : 0.f;
+}
+
+// Chunks per stream for the few-query path, and the floats of partials they need.  Depends on
+// row and token counts only (never on the dtype), so the workspace query can include it.
+static int lbm_decode_chunks(int kv_tokens) {
+  int n = (kv_tokens + kDecBlock - 1) / kDecBlock;
+  return n < 1 ? 1 : (n > kDecMaxChunks ? kDecMaxChunks : n);
+}
+static bool lbm_decode_applies(const LbmAttnSchedule& sch) {
+  for (int i = 0; i < sch.n_streams; ++i)
+    if (sch.s[i].q_rows > kDecQ) return false;
+  return sch.n_streams > 0;
+}
+static size_t lbm_decode_bytes(const LbmAttnSchedule& sch, int num_heads, int head_dim) {
+  if (!lbm_decode_applies(sch)) return 0;
+  size_t rows = 0;
+  for (int i = 0; i < sch.n_streams; ++i) rows += (size_t)lbm_decode_chunks(sch.s[i].kv_tokens) * sch.s[i].q_rows;
+  return rows * num_heads * (head_dim + 2) * sizeof(float);
+}
+
 // ---------------------------------------------------------------------------- schedule
 // How many KV splits each stream gets.  All workgroups of one launch compete for the 256 CUs
 // (one 8-wave workgroup per CU at a time, handed out in blockIdx order), so the choice is a
@@ -975,8 +1161,12 @@ void lbm_attn_schedule(const lbm_attn_stream* streams, int n_streams, int num_he
 }
 
 size_t lbm_attn_schedule_bytes(const LbmAttnSchedule& sch, int num_heads, int head_dim) {
-  // bf16 partial outputs followed by one float log-sum-exp per (row, head)
-  return (size_t)sch.part_rows * num_heads * (head_dim * 2 + 4);
+  // bf16 partial outputs followed by one float log-sum-exp per (row, head); or, when every
+  // stream has only a few query rows, the fp32 partials of the few-query path (the query does
+  // not know the dtype, so it covers both)
+  const size_t split_kv = (size_t)sch.part_rows * num_heads * (head_dim * 2 + 4);
+  const size_t few_q = lbm_decode_bytes(sch, num_heads, head_dim);
+  return split_kv > few_q ? split_kv : few_q;
 }
 
 int lbm_launch_attention(const void* q, const void* pool, void* out, const void* self_k,
@@ -1010,6 +1200,33 @@ int lbm_launch_attention(const void* q, const void* pool, void* out, const void*
     }
     f.wg_begin[LBM_MAX_STREAMS] = wg;
     if (wg == 0) return LBM_OK;
+    if (lbm_decode_applies(sch)) {
+      DecodeArgs d;
+      d.f = f;
+      d.part = (float*)workspace;
+      int max_chunks = 0, max_q = 0, part = 0;
+      for (int i = 0; i < LBM_MAX_STREAMS; ++i) {
+        d.n_chunks[i] = 0;
+        d.part_begin[i] = part;
+        if (i < sch.n_streams) {
+          d.n_chunks[i] = lbm_decode_chunks(sch.s[i].kv_tokens);
+          part += d.n_chunks[i] * sch.s[i].q_rows;
+          if (d.n_chunks[i] > max_chunks) max_chunks = d.n_chunks[i];
+          if (sch.s[i].q_rows > max_q) max_q = sch.s[i].q_rows;
+        }
+      }
+      if (max_q == 0) return LBM_OK;
+      d.max_q = max_q;
+      const dim3 grid(max_chunks, num_heads, sch.n_streams * max_q), mgrid(max_q, num_heads, sch.n_streams);
+      if (head_dim == 64) {
+        hipLaunchKernelGGL(lbm_attn_f32_decode_kernel<64>, grid, dim3(256), 0, stream, d);
+        hipLaunchKernelGGL(lbm_attn_f32_decode_merge_kernel<64>, mgrid, dim3(64), 0, stream, d);
+      } else {
+        hipLaunchKernelGGL(lbm_attn_f32_decode_kernel<128>, grid, dim3(256), 0, stream, d);
+        hipLaunchKernelGGL(lbm_attn_f32_decode_merge_kernel<128>, mgrid, dim3(128), 0, stream, d);
+      }
+      return lbm_check_launch("lbm_attn_f32_decode_kernel");
+    }
     if (head_dim == 64) hipLaunchKernelGGL(lbm_attn_f32_kernel<64>, dim3(wg), dim3(1024), 0, stream, f);
     else hipLaunchKernelGGL(lbm_attn_f32_kernel<128>, dim3(wg), dim3(512), 0, stream, f);
     return lbm_check_launch("lbm_attn_f32_kernel");

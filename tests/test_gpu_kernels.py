@@ -325,3 +325,85 @@ def test_append_is_exact_and_gated(src, dst):
             expect[p, 0, s] = k[t].to(dst)
             expect[p, 1, s] = v[t].to(dst)
     assert torch.equal(pool.cpu(), expect)
+
+
+@pytest.mark.parametrize("D", [64, 128])
+def test_fp32_few_query_rows_path(D):
+    """Streams of 1..8 query rows in fp32 take the few-query kernels (the KV axis cut into
+    chunks, one workgroup per chunk and query row, partials merged by a second kernel): two
+    ragged streams per launch over shuffled pool rows with the streams' own rows at the tail,
+    KV lengths around the 256-token block size, longer than 64 chunks, and empty.  Against
+    float64 softmax(q k^T / sqrt(D)) v: 1e-5."""
+    N = _native()
+    dev = torch.device("cuda:0")
+    H, S = 4, 16
+    g = torch.Generator().manual_seed(40 + D)
+    for (q0, kv0), (q1, kv1) in [((1, 1), (8, 255)), ((3, 256), (1, 257)), ((1, 5000), (2, 700)), ((1, 20000), (8, 300)),
+                                 ((4, 0), (1, 33))]:
+        nq = q0 + q1
+        q = torch.randn(nq, H, D, generator=g)
+        own_k, own_v = torch.randn(nq, H, D, generator=g), torch.randn(nq, H, D, generator=g)
+        n_pages = (kv0 + kv1) // S + 4
+        pool = torch.randn(n_pages, 2, S, H, D, generator=g)
+        flat_k, flat_v = pool[:, 0].reshape(-1, H, D), pool[:, 1].reshape(-1, H, D)
+        perm = torch.randperm(n_pages * S, generator=g)
+        rows, refs, begin, off = [], [], [], 0
+        for qb, qn, kv in ((0, q0, kv0), (q0, q1, kv1)):
+            begin.append(len(torch.cat(rows)) if rows else 0)
+            tail = min(qn, kv)                     # the stream's own rows close its KV list
+            slots = perm[off:off + kv - tail]
+            off += kv - tail
+            r = (slots // S) * 2 * S + slots % S
+            r = torch.cat([r, -1 - (qb + torch.arange(tail))])
+            rows.append(r.to(torch.int32))
+            K = torch.cat([flat_k[slots], own_k[qb:qb + tail]]).double()
+            V = torch.cat([flat_v[slots], own_v[qb:qb + tail]]).double()
+            if kv == 0:
+                refs.append(torch.zeros(qn, H, D, dtype=torch.float64))
+            else:
+                s = torch.einsum("qhd,khd->hqk", q[qb:qb + qn].double(), K) / math.sqrt(D)
+                refs.append(torch.einsum("hqk,khd->qhd", torch.softmax(s, -1), V))
+        kv_rows = torch.cat(rows + [torch.full((8,), -12345, dtype=torch.int32)]).to(dev)
+        streams = [(0, q0, begin[0], kv0), (q0, q1, begin[1], kv1)]
+        arr = (N.AttnStream * 2)(*[N.AttnStream(*s) for s in streams])
+        need = int(N.lib.lbm_attn_workspace_bytes(arr, 2, H, D))
+        assert need >= sum(min(max(-(-kv // 256), 1), 64) * qn for (_, qn, _, kv) in streams) * H * (D + 2) * 4
+        ws = torch.empty(max(need, 16), dtype=torch.uint8, device=dev)
+        qd, out = q.to(dev), torch.full((nq, H, D), float("nan"), device=dev)
+        ok, ov, pd = own_k.to(dev), own_v.to(dev), pool.to(dev)
+        N.check(N.lib.lbm_attn_run(ptr(qd), ptr(pd), ptr(out), ptr(ok), ptr(ov), ptr(kv_rows), arr, 2, H, D, S,
+                                   N.DTYPE_F32, 1.0 / math.sqrt(D), ptr(ws), ws.numel(), None))
+        torch.cuda.synchronize()
+        err = (out.cpu().double() - torch.cat(refs)).abs().max().item()
+        assert err <= 1e-5, ((q0, kv0), (q1, kv1), err)
+
+
+def test_fp32_running_maximum_covers_every_lane_group():
+    """In the fp32 matrix kernel the four lane groups of a wavefront hold different KV rows of a
+    16-token block (rows 4g..4g+3 in group g) and the row maximum has to be taken over all of
+    them.  Here the rows of group 0 score 0 and all others 240 (natural units): a maximum taken
+    from group 0 alone would send exp2 to infinity.  The answer is the mean of the V rows of
+    the high-scoring tokens."""
+    N = _native()
+    dev = torch.device("cuda:0")
+    H, D, S, tq, n_kv = 2, 64, 16, 20, 96
+    g = torch.Generator().manual_seed(77)
+    u = torch.ones(D)
+    q = u.repeat(tq, H, 1).contiguous()                       # q . k / sqrt(D) = 8 c for k = c u
+    c = torch.where(torch.arange(n_kv) % 16 < 4, 0.0, 30.0)
+    k = (c.view(n_kv, 1, 1) * u).expand(n_kv, H, D).contiguous()
+    v = torch.randn(n_kv, H, D, generator=g)
+    pool = torch.zeros(n_kv // S, 2, S, H, D)
+    pool[:, 0] = k.view(n_kv // S, S, H, D)
+    pool[:, 1] = v.view(n_kv // S, S, H, D)
+    rows, n_tok = rows_from_pages(list(range(n_kv // S)), [S] * (n_kv // S), S, dev)
+    arr = (N.AttnStream * 1)(N.AttnStream(0, tq, 0, n_tok))
+    ws = torch.empty(max(int(N.lib.lbm_attn_workspace_bytes(arr, 1, H, D)), 16), dtype=torch.uint8, device=dev)
+    out = torch.full((tq, H, D), float("nan"), device=dev)
+    qd, pd = q.to(dev), pool.to(dev)     # named, so that they outlive the launch
+    N.check(N.lib.lbm_attn_run(ptr(qd), ptr(pd), ptr(out), None, None, ptr(rows), arr, 1, H, D, S,
+                               N.DTYPE_F32, 1.0 / math.sqrt(D), ptr(ws), ws.numel(), None))
+    torch.cuda.synchronize()
+    want = v[c > 0].mean(dim=0)                                # [H, D]
+    assert torch.isfinite(out).all()
+    assert (out.cpu() - want[None]).abs().max().item() <= 1e-5
