@@ -56,7 +56,12 @@ def test_host_side_argument_checks_need_no_gpu():
     s = (N.AttnStream * 1)(N.AttnStream(0, 1004, 0, 17068))
     # 4 query tiles x 16 heads x 8 splits = 512 workgroups -> 8 partial results per row
     assert N.lib.lbm_attn_workspace_bytes(s, 1, 16, 64) == 8 * 1004 * 16 * (64 * 2 + 4)
-    s1 = (N.AttnStream * 1)(N.AttnStream(0, 8, 0, 64))
+    s1 = (N.AttnStream * 1)(N.AttnStream(0, 9, 0, 64))      # one workgroup per head, nothing to merge
     assert N.lib.lbm_attn_workspace_bytes(s1, 1, 16, 64) == 0
+    # at most 8 query rows: partials of the fp32 few-query path, (D + 2) floats per chunk, row and head
+    s8 = (N.AttnStream * 1)(N.AttnStream(0, 8, 0, 64))
+    assert N.lib.lbm_attn_workspace_bytes(s8, 1, 16, 64) == 1 * 8 * 16 * (64 + 2) * 4
+    s9 = (N.AttnStream * 1)(N.AttnStream(0, 1, 0, 10000))
+    assert N.lib.lbm_attn_workspace_bytes(s9, 1, 16, 128) == 40 * 1 * 16 * (128 + 2) * 4
     rc = N.lib.lbm_attn_run(None, None, None, None, None, None, s, 1, 16, 64, 16, 0, 0.125, None, 0, None)
     assert rc == N.ERR_INVALID and b"null" in N.lib.lbm_last_error()
