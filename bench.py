@@ -425,8 +425,8 @@ def main() -> None:
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-aggregator", action="store_true",
                     help="skip the full aggregator-trunk step (frame + global blocks) timed after the hot path")
-    ap.add_argument("--mode", choices=["full", "attention", "attention_f32", "append", "prepare", "residual", "tables", "copy"], default="full",
-                    help="full = the benchmark line; attention/attention_f32/append/prepare/residual/tables launch one kernel --steps "
+    ap.add_argument("--mode", choices=["full", "attention", "attention_f32", "attention_f32_few", "append", "prepare", "residual", "tables", "copy"], default="full",
+                    help="full = the benchmark line; attention/attention_f32/attention_f32_few/append/prepare/residual/tables launch one kernel --steps "
                          "times on the steady-state cache (for rocprofv3 runs); copy = a plain 256 MiB "
                          "device copy, the known-size kernel the HBM counters are calibrated on")
     args = ap.parse_args()
@@ -492,6 +492,24 @@ def main() -> None:
             m.step(b, qs[j], ks[j], vs[j], keyframe=[True], cross_frame_special=False)
 
     kv_tokens = (ANCHOR + WINDOW) * T
+    if args.mode == "attention_f32_few":
+        # the camera head's shape after 10,000 frames: one fp32 query token, 16 heads of 128
+        frames_c = 10000
+        mc = HipPagedKVCacheManager(1, frames_c + 16, 1, 16, 128, torch.float32, dev, num_special_tokens=0, scale_frames=8,
+                                    sliding_window=frames_c + 8, max_total_frames=frames_c + 16, force_fp32=True,
+                                    page_size=PAGE, layout="frame_pages")
+        torch.manual_seed(0)
+        tok = [torch.randn(1, 16, 128, device=dev) for _ in range(3)]
+        for _ in range(frames_c):
+            mc.append_frame(0, tok[1], tok[2])
+        mc._plan(0, [False])
+        fn = lambda: mc._attend_planned(0, tok[0], None, None)
+        for _ in range(args.warmup):
+            fn()
+        ms = event_time_ms(fn, args.steps, torch)
+        print(json.dumps({"mode": args.mode, "launches": args.steps, "avg_launch_us": ms * 1e3,
+                          "gbps": frames_c * 16 * 128 * 4 * 2 / (ms * 1e-3) * 1e-9}))
+        return
     if args.mode == "attention_f32":
         # config 1's last frame: 1004 fp32 queries over 8 cached frames (8032 tokens)
         m32 = HipPagedKVCacheManager(1, 32, T, H, D, torch.float32, dev, num_special_tokens=N_SPECIAL, scale_frames=1,

@@ -982,24 +982,51 @@ __global__ __launch_bounds__(256) void lbm_attn_f32_decode_kernel(DecodeArgs a) 
   }
 }
 
-// one workgroup of D threads per (stream, query row, head): merge the chunks' partials
+// one 128-thread workgroup per (stream, query row, head): merge the chunks' partials.  Thread
+// c reads chunk c's maximum and sum (all chunks at once), the weights go through LDS, then
+// thread d sums the weighted outputs with several loads in flight.
 template <int D>
-__global__ __launch_bounds__(D) void lbm_attn_f32_decode_merge_kernel(DecodeArgs a) {
-  const int b = blockIdx.z, head = blockIdx.y, qi = blockIdx.x, d = threadIdx.x;
+__global__ __launch_bounds__(128) void lbm_attn_f32_decode_merge_kernel(DecodeArgs a) {
+  static_assert(kDecMaxChunks <= 128 && D <= 128, "one thread per chunk, one per head dimension");
+  __shared__ float w[kDecMaxChunks];
+  __shared__ float red[2][2];
+  const int b = blockIdx.z, head = blockIdx.y, qi = blockIdx.x, tid = threadIdx.x;
   const lbm_attn_stream sp = a.f.s[b];
   if (qi >= sp.q_rows) return;
   const int H = a.f.num_heads, nc = a.n_chunks[b];
-  float m = -INFINITY;
-  for (int c = 0; c < nc; ++c)
-    m = fmaxf(m, a.part[(((size_t)a.part_begin[b] + (size_t)c * sp.q_rows + qi) * H + head) * (D + 2) + D]);
-  float o = 0.f, l = 0.f;
-  for (int c = 0; c < nc; ++c) {
-    const float* pp = a.part + (((size_t)a.part_begin[b] + (size_t)c * sp.q_rows + qi) * H + head) * (D + 2);
-    const float w = pp[D] > -INFINITY ? exp2f(pp[D] - m) : 0.f;   // a chunk without tokens weighs nothing
-    o += pp[d] * w;
-    l += pp[D + 1] * w;
+  const size_t stride = (size_t)sp.q_rows * H * (D + 2);      // from one chunk's partial to the next
+  const float* base = a.part + (((size_t)a.part_begin[b] + qi) * H + head) * (D + 2);
+  float m_c = -INFINITY, l_c = 0.f;
+  if (tid < nc) {
+    m_c = base[tid * stride + D];
+    l_c = base[tid * stride + D + 1];
   }
-  a.f.out[((size_t)(sp.q_begin + qi) * H + head) * D + d] = l > 0.f ? o / l : 0.f;
+  float m = m_c;
+#pragma unroll
+  for (int o = 32; o >= 1; o >>= 1) m = fmaxf(m, __shfl_xor(m, o));
+  if ((tid & 63) == 0) red[0][tid >> 6] = m;
+  __syncthreads();
+  m = fmaxf(red[0][0], red[0][1]);
+  const float w_c = m_c > -INFINITY ? exp2f(m_c - m) : 0.f;   // a chunk without tokens weighs nothing
+  if (tid < nc) w[tid] = w_c;
+  float l = l_c * w_c;
+#pragma unroll
+  for (int o = 32; o >= 1; o >>= 1) l += __shfl_xor(l, o);
+  if ((tid & 63) == 0) red[1][tid >> 6] = l;
+  __syncthreads();
+  l = red[1][0] + red[1][1];
+  if (tid >= D) return;
+  float o = 0.f;
+  int c = 0;
+  for (; c + 8 <= nc; c += 8) {
+    float x[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) x[j] = base[(c + j) * stride + tid];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) o += x[j] * w[c + j];
+  }
+  for (; c < nc; ++c) o += base[c * stride + tid] * w[c];
+  a.f.out[((size_t)(sp.q_begin + qi) * H + head) * D + tid] = l > 0.f ? o / l : 0.f;
 }
 
 // Chunks per stream for the few-query path, and the floats of partials they need.  Depends on
@@ -1220,7 +1247,7 @@ int lbm_launch_attention(const void* q, const void* pool, void* out, const void*
       const dim3 grid(max_chunks, num_heads, sch.n_streams * max_q), mgrid(max_q, num_heads, sch.n_streams);
       if (head_dim == 64) {
         hipLaunchKernelGGL(lbm_attn_f32_decode_kernel<64>, grid, dim3(256), 0, stream, d);
-        hipLaunchKernelGGL(lbm_attn_f32_decode_merge_kernel<64>, mgrid, dim3(64), 0, stream, d);
+        hipLaunchKernelGGL(lbm_attn_f32_decode_merge_kernel<64>, mgrid, dim3(128), 0, stream, d);
       } else {
         hipLaunchKernelGGL(lbm_attn_f32_decode_kernel<128>, grid, dim3(256), 0, stream, d);
         hipLaunchKernelGGL(lbm_attn_f32_decode_merge_kernel<128>, mgrid, dim3(128), 0, stream, d);
