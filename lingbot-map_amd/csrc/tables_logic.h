@@ -236,22 +236,50 @@ LBM_HD void lbm_phase_plan(int32_t* st, const lbm_cache_geom& g, const LbmTables
   const int32_t* win = st + L.off_window;
   if (kv_rows) {
     int32_t* out = kv_rows + op.kv_row_begin;
-    for (int i = tid; i < frame_tokens && i < limit; i += nthr) {
-      const int f = i / L.tpf, t = i % L.tpf;
-      const int32_t* pages = f < h.na ? anchor + f * L.ppf
-                                      : win + ((h.wh + f - h.na) % L.ring_frames) * L.ppf;
-      out[i] = pages[t / S] * 2 * S + t % S;
+    // token t of a page list sits in page t / S, slot t % S; page sizes are powers of two in
+    // every configuration but one (page = patches per frame), so the common case is a shift
+    const int shift = (S & (S - 1)) == 0 ? __builtin_ctz((unsigned)S) : -1;
+    // a thread owns token slots t, t + nthr, ... of every frame (consecutive lanes write
+    // consecutive rows); eight frames at a time so that their page-id loads are in flight
+    // together (no division per token, no load waiting on the previous frame's store)
+    for (int t = tid; t < L.tpf; t += nthr) {
+      const int pg = shift >= 0 ? t >> shift : t / S;
+      const int slot = t - pg * S;
+      for (int f0 = 0; f0 < nfr; f0 += 8) {
+        int32_t page[8];
+#ifdef __HIP_DEVICE_COMPILE__
+#pragma unroll
+#endif
+        for (int k = 0; k < 8; ++k) {
+          const int f = f0 + k < nfr ? f0 + k : nfr - 1;
+          int r = h.wh + f - h.na;                     // ring slot of window frame f - na
+          if (r >= L.ring_frames) r -= L.ring_frames;  // wh < ring_frames and at most ring_frames window frames
+          const int32_t* pages = f < h.na ? anchor + f * L.ppf : win + r * L.ppf;
+          page[k] = pages[pg];
+        }
+#ifdef __HIP_DEVICE_COMPILE__
+#pragma unroll
+#endif
+        for (int k = 0; k < 8; ++k) {
+          const int i = (f0 + k) * L.tpf + t;
+          if (f0 + k < nfr && i < limit) out[i] = page[k] * 2 * S + slot;
+        }
+      }
     }
     if (two) {
-      for (int c = tid; c < h.stc; c += nthr)
-        if (frame_tokens + c < limit) out[frame_tokens + c] = st[L.off_special + c / S] * 2 * S + c % S;
+      for (int c = tid; c < h.stc; c += nthr) {
+        const int pg = shift >= 0 ? c >> shift : c / S;
+        if (frame_tokens + c < limit) out[frame_tokens + c] = st[L.off_special + pg] * 2 * S + (c - pg * S);
+      }
     } else {
       for (int e = tid; e < h.nm; e += nthr) {
         const int t0 = st[L.off_mem_tcum + e], t1 = st[L.off_mem_tcum + e + 1];
         const int p0 = st[L.off_mem_pcum + e];
-        for (int t = 0; t < t1 - t0; ++t)
+        for (int t = 0; t < t1 - t0; ++t) {
+          const int pg = shift >= 0 ? t >> shift : t / S;
           if (frame_tokens + t0 + t < limit)
-            out[frame_tokens + t0 + t] = st[L.off_mem_pages + p0 + t / S] * 2 * S + t % S;
+            out[frame_tokens + t0 + t] = st[L.off_mem_pages + p0 + pg] * 2 * S + (t - pg * S);
+        }
       }
     }
     for (int t = tid; t < self_n; t += nthr)
