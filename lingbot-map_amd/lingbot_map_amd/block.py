@@ -38,62 +38,57 @@ def apply_rotary_emb(x: Tensor, freqs: Tensor) -> Tensor:
 
 
 class RotaryPositionEmbedding2D(nn.Module):
-    """2-D rotary embedding of the frame blocks (lingbot_map/layers/rope.py:64-198): head_dim is
-    split into a vertical and a horizontal half; in each, element j rotates with element
-    j + dim/4 by ``pos * frequency^(-4j/dim)``.  ``forward`` is the reference's sequence of
-    torch operations; ``cos_sin_table`` hands the same cos / sin values to the fused producer."""
+    """2-D rotary embedding of the frame blocks (lingbot_map/layers/rope.py:64-198).
+
+    The first half of head_dim belongs to the token's y coordinate and the second half to its
+    x coordinate.  Inside a half of ``2q`` elements, element ``j < q`` and element ``j + q``
+    form a pair that is turned by ``coordinate / frequency^(j / q)`` radians:
+    ``(a, b) -> (a cos - b sin, b cos + a sin)``.  Everything is derived from one table,
+    ``cos_sin_table``: a (cos, sin) per token and element, formed in the activations' dtype
+    (angle, cosine and sine each rounded to it, as the reference's cached tables are) and
+    handed to the fused producer as float32; ``forward`` is the same table applied with
+    torch operations."""
 
     def __init__(self, frequency: float = 100.0, scaling_factor: float = 1.0) -> None:
         super().__init__()
-        self.base_frequency = frequency
-        self.scaling_factor = scaling_factor
-        self.frequency_cache = {}
-        self._table_cache = {}
+        self.frequency = float(frequency)
+        self.scaling_factor = float(scaling_factor)
+        self._last_table = None
 
-    def _compute_frequency_components(self, dim: int, seq_len: int, device, dtype):
-        key = (dim, seq_len, device, dtype)
-        if key not in self.frequency_cache:
-            exponents = torch.arange(0, dim, 2, device=device).float() / dim
-            inv_freq = 1.0 / (self.base_frequency ** exponents)
-            positions = torch.arange(seq_len, device=device, dtype=inv_freq.dtype)
-            angles = torch.einsum("i,j->ij", positions, inv_freq).to(dtype)
-            angles = torch.cat((angles, angles), dim=-1)
-            self.frequency_cache[key] = (angles.cos().to(dtype).detach().clone(), angles.sin().to(dtype).detach().clone())
-        return self.frequency_cache[key]
-
-    @staticmethod
-    def _rotate_features(x: Tensor) -> Tensor:
-        d = x.shape[-1]
-        return torch.cat((-x[..., d // 2:], x[..., : d // 2]), dim=-1)
-
-    def _apply_1d_rope(self, tokens: Tensor, positions: Tensor, cos_comp: Tensor, sin_comp: Tensor) -> Tensor:
-        cos = F.embedding(positions, cos_comp)[:, None, :, :]
-        sin = F.embedding(positions, sin_comp)[:, None, :, :]
-        return (tokens * cos) + (self._rotate_features(tokens) * sin)
-
-    def forward(self, tokens: Tensor, positions: Tensor) -> Tensor:
-        assert tokens.size(-1) % 2 == 0, "Feature dimension must be even"
-        assert positions.ndim == 3 and positions.shape[-1] == 2, "Positions must have shape (batch_size, n_tokens, 2)"
-        feature_dim = tokens.size(-1) // 2
-        cos_comp, sin_comp = self._compute_frequency_components(feature_dim, positions.shape[1], tokens.device, tokens.dtype)
-        vertical, horizontal = tokens.chunk(2, dim=-1)
-        vertical = self._apply_1d_rope(vertical, positions[..., 0], cos_comp, sin_comp)
-        horizontal = self._apply_1d_rope(horizontal, positions[..., 1], cos_comp, sin_comp)
-        return torch.cat((vertical, horizontal), dim=-1)
+    def _pair_rates(self, pairs: int, device) -> Tensor:
+        # radians per unit of coordinate for pair j of a half: the reciprocal of frequency^(j / pairs)
+        j = torch.arange(pairs, device=device, dtype=torch.float32)
+        return torch.reciprocal(torch.pow(self.frequency, (2.0 * j) / (2 * pairs)))
 
     def cos_sin_table(self, positions: Tensor, head_dim: int, dtype: torch.dtype) -> Tensor:
-        """float32 ``[B * N, head_dim, 2]`` (cos, sin) per token and element, the values ``forward``
-        multiplies with for activations of ``dtype``.  Cached per positions tensor."""
+        """float32 ``[B * N, head_dim, 2]``: (cos, sin) of every element of every token for
+        activations of ``dtype``; ``positions`` is ``[B, N, 2]`` integer (y, x).  The table of the
+        last positions tensor is kept."""
+        if positions.ndim != 3 or positions.shape[-1] != 2:
+            raise ValueError(f"positions must be [batch, tokens, 2] (y, x), got {tuple(positions.shape)}")
+        if head_dim % 4 != 0:
+            raise ValueError(f"head_dim {head_dim} must split into two halves of pairs")
         key = (positions.data_ptr(), tuple(positions.shape), positions._version, head_dim, dtype)
-        hit = self._table_cache.get("last")
-        if hit is not None and hit[0] == key:
-            return hit[1]
-        cos_comp, sin_comp = self._compute_frequency_components(head_dim // 2, positions.shape[1], positions.device, dtype)
-        cos = torch.cat((F.embedding(positions[..., 0], cos_comp), F.embedding(positions[..., 1], cos_comp)), dim=-1)
-        sin = torch.cat((F.embedding(positions[..., 0], sin_comp), F.embedding(positions[..., 1], sin_comp)), dim=-1)
-        table = torch.stack((cos.float(), sin.float()), dim=-1).reshape(-1, head_dim, 2).contiguous()
-        self._table_cache["last"] = (key, table, positions)   # positions kept alive with its key
+        if self._last_table is not None and self._last_table[0] == key:
+            return self._last_table[1]
+        batch, n_tok, pairs = positions.shape[0], positions.shape[1], head_dim // 4
+        # [B, N, axis, pair]: one float32 product per entry, then the activations' precision
+        turn = (positions.to(torch.float32)[..., None] * self._pair_rates(pairs, positions.device)).to(dtype)
+        # both members of a pair see the same angle: [B, N, axis, member, pair] = head_dim elements
+        turn = turn[:, :, :, None, :].expand(batch, n_tok, 2, 2, pairs)
+        table = torch.stack((torch.cos(turn), torch.sin(turn)), dim=-1).float().reshape(batch * n_tok, head_dim, 2)
+        table = table.contiguous()
+        self._last_table = (key, table, positions)   # the tensor stays alive with its key
         return table
+
+    def forward(self, tokens: Tensor, positions: Tensor) -> Tensor:
+        """``tokens`` ``[B, H, N, D]``, ``positions`` ``[B, N, 2]``; every product and the sum are
+        rounded to the tokens' dtype."""
+        batch, _, n_tok, dim = tokens.shape
+        cs = self.cos_sin_table(positions, dim, tokens.dtype).view(batch, 1, n_tok, dim, 2).to(tokens.dtype)
+        halves = tokens.reshape(*tokens.shape[:-1], 2, 2, dim // 4)          # [..., axis, member, pair]
+        partner = torch.stack((-halves[..., 1, :], halves[..., 0, :]), dim=-2).reshape(tokens.shape)
+        return tokens * cs[..., 0] + partner * cs[..., 1]
 
 
 class PositionGetter:
