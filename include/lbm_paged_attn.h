@@ -131,7 +131,10 @@ int64_t lbm_tables_words(const lbm_cache_geom* geom);
  *   tables        [n_streams * lbm_tables_words]           in/out
  *   ops           host, n_streams entries
  *   append_rows   APPEND: K row of every token of the new frame, -1 if the stream does not
- *                 append (indexed q_begin + t); may be NULL without APPEND
+ *                 append (indexed q_begin + t); may be NULL without APPEND.  When it is given,
+ *                 every stream of the call - idle ones (ops == 0) included - gets its
+ *                 tokens_per_frame entries written, so the streams' q_begin ranges must not
+ *                 overlap (LBM_ERR_INVALID otherwise)
  *   kv_rows       PLAN: K row of every visible token; entries < 0 name row (-1 - e) of the
  *                 caller's own k/v tensors; may be NULL without PLAN
  *   kv_page_ids, kv_page_lens   PLAN: FlashInfer-style page table with a valid length per

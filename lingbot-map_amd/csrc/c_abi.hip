@@ -53,6 +53,17 @@ int lbm_tables_step(int32_t* tables, const lbm_cache_geom* geom, int32_t n_strea
       return lbm_fail(LBM_ERR_INVALID, "lbm_tables_step: stream %d has a negative sliding_window", i);
     if (o.q_begin < 0) return lbm_fail(LBM_ERR_INVALID, "lbm_tables_step: stream %d has a negative q_begin", i);
   }
+  // Every stream's workgroup writes its tokens_per_frame entries of append_rows (the rows of the
+  // new frame, or -1 for a stream that does not append, idle streams included): two streams
+  // with overlapping ranges would race inside one launch.
+  if (append_rows)
+    for (int i = 0; i < n_streams; ++i)
+      for (int j = 0; j < i; ++j) {
+        const long long d = (long long)ops[i].q_begin - ops[j].q_begin;
+        if ((d < 0 ? -d : d) < geom->tokens_per_frame)
+          return lbm_fail(LBM_ERR_INVALID, "lbm_tables_step: streams %d and %d overlap in append_rows (q_begin %d and %d, %d tokens per frame)",
+                          j, i, ops[j].q_begin, ops[i].q_begin, geom->tokens_per_frame);
+      }
   return lbm_launch_tables(tables, *geom, n_streams, ops, append_rows, kv_rows, kv_page_ids,
                            kv_page_lens, (hipStream_t)stream);
 }

@@ -644,7 +644,9 @@ class HipPagedKVCacheManager:
         return out
 
     def reset(self) -> None:
-        """Reset all per-block state for a new sequence (flashinfer_cache.py:423-432)."""
+        """Reset all per-block state for a new sequence (flashinfer_cache.py:423-432).  What the
+        device tables recorded about the sequence that ends here is raised first."""
+        words = self._tables[:, :, N.HDR["error"]].cpu().tolist() if getattr(self, "_tables_live", False) else []
         ops = self._ops([{"ops": N.OP_RESET} for _ in range(self.num_streams)])
         for ts in range(self._n_sets):
             self._tables_step(ts, ops)
@@ -657,20 +659,53 @@ class HipPagedKVCacheManager:
             self._n_appends[i] = 0
         self._rows_log.clear()
         self._active = [True] * self.num_streams
+        self._tables_live = True
+        for ts, row in enumerate(words):      # the cache is reset either way
+            for b, w in enumerate(row):
+                self._raise_device_errors(w, ts, b)
 
     # ----- table read-back (synchronises; for tests, debugging and parity checks) -----
     def _read_tables(self, block_idx: int, stream: int):
+        """Page ids and valid lengths of what `stream` sees, without the current frame's own
+        rows.  Side-effect free: the plan runs into the page-table outputs only (the row table
+        the blocks of the current frame attend through is not rewritten) and the two header
+        words a plan publishes - the token count the kernels of a ``device_token_counts`` manager
+        read, and the page count - are put back."""
         ts = self._set(block_idx)
-        saved_tokens = list(self._plan_tokens[ts])
-        self._plan(ts, [False] * self.num_streams, pages=True)
+        plan_words = slice(N.HDR["plan_kv_tokens"], N.HDR["plan_n_pages"] + 1)
+        saved = self._tables[ts, :, plan_words].clone()
+        per = [{"ops": N.OP_PLAN, "self_tokens": 0,
+                "expect_kv_tokens": self._expect(self._visible_tokens(self._counts[ts][b]))}
+               for b in range(self.num_streams)]
+        self._tables_step(ts, self._ops(per), pages=True)
         hdr = self._tables[ts, stream, :N.HDR_WORDS].cpu().tolist()
         n_pages = hdr[N.HDR["plan_n_pages"]]
         lo = stream * self._pages_cap
         ids = self._page_ids[lo:lo + n_pages].cpu().tolist()
         lens = self._page_lens[lo:lo + n_pages].cpu().tolist()
-        # leave the plan the following blocks may still need untouched in meaning
-        self._plan_tokens[ts], self._plan_valid[ts] = saved_tokens, False
+        self._tables[ts, :, plan_words] = saved
+        self._raise_device_errors(hdr[N.HDR["error"]], ts, stream)
         return hdr, ids, lens
+
+    # ----- device-side error word -----
+    @staticmethod
+    def _raise_device_errors(word: int, ts: int, stream: int) -> None:
+        if word:
+            what = ", ".join(name for bit, name in N.TERR_NAMES.items() if word & bit)
+            raise AssertionError(f"device page tables (set {ts}, stream {stream}) report: {what} "
+                                 f"(error word 0x{word:x})")
+
+    def check_device_errors(self) -> None:
+        """Read the sticky error word of every stream's device tables (one small copy that
+        waits for the queued work) and raise the reference's exception type for what it says:
+        pool exhausted, rollback underflow (flashinfer_cache.py:276-278,290-293,489-494,
+        533-537) or a visible-token count that disagrees with the host's.  The host's count
+        mirror normally raises first; this is the check for paths where the mirror is advanced
+        by book-keeping only (graph replay) or was bypassed.  Called by ``reset()``."""
+        words = self._tables[:, :, N.HDR["error"]].cpu().tolist()
+        for ts, row in enumerate(words):
+            for b, w in enumerate(row):
+                self._raise_device_errors(w, ts, b)
 
     def build_visible_page_table(self, block_idx: int, stream: int = 0) -> List[int]:
         """Page ids in order anchor, window, special/memory (flashinfer_cache.py:438-450)."""

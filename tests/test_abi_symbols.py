@@ -65,3 +65,8 @@ def test_host_side_argument_checks_need_no_gpu():
     assert N.lib.lbm_attn_workspace_bytes(s9, 1, 16, 128) == 40 * 1 * 16 * (128 + 2) * 4
     rc = N.lib.lbm_attn_run(None, None, None, None, None, None, s, 1, 16, 64, 16, 0, 0.125, None, 0, None)
     assert rc == N.ERR_INVALID and b"null" in N.lib.lbm_last_error()
+    # two streams whose append_rows ranges overlap (an idle stream left at q_begin 0) are refused
+    ops = (N.StepOp * 2)(N.StepOp(N.OP_APPEND, 0, 0, 0, 0, 0, 0, 0), N.StepOp(0, 0, 0, 0, 0, 0, 0, 0))
+    fake = C.c_void_p(256)   # never dereferenced: the call fails in the argument checks
+    rc = N.lib.lbm_tables_step(fake, C.byref(g), 2, ops, fake, None, None, None, None)
+    assert rc == N.ERR_INVALID and b"overlap" in N.lib.lbm_last_error()

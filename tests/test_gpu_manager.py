@@ -1,5 +1,7 @@
 """The drop-in manager on the GPU against the oracle: device page tables bit-exact after
 every operation, pool contents exact, attention within the bf16 tolerance."""
+import math
+
 import pytest
 import torch
 
@@ -93,6 +95,54 @@ def test_error_conventions():
     assert m.device_header()["error"] == 0     # the host refused before the device saw it
     with pytest.raises(AssertionError):
         m.append_frame(0, q[:5], q[:5])
+
+
+def test_device_error_word_is_raised_by_the_product_path():
+    """The device tables keep a sticky error word; the manager raises it as the reference's
+    AssertionError wherever it already waits for the device (table read-back, reset) and on
+    request.  Here the host's count mirror is made to disagree with the device on purpose -
+    one special token too many - so the plan step records LBM_TERR_KV_COUNT; the kernels only
+    ever read as many rows as the table holds."""
+    m = make("two_stream", None)
+    q = torch.zeros(7, 2, 64, dtype=torch.bfloat16, device="cuda")
+    m.append_frame(0, q, q)
+    m.check_device_errors()                      # clean so far
+    m._counts[0][0].special_tokens += 1          # the host now expects one visible token too many
+    m.compute_attention(0, q)                    # plans with the wrong expectation
+    with pytest.raises(AssertionError, match="visible token count mismatch"):
+        m.check_device_errors()
+    with pytest.raises(AssertionError, match="visible token count mismatch"):
+        m.build_visible_page_table(0)
+    with pytest.raises(AssertionError, match="visible token count mismatch"):
+        m.reset()                                # resets, then reports what the old sequence recorded
+    assert m.frame_count[0] == 0 and m.device_header()["error"] == 0
+    m.append_frame(0, q, q)
+    m.reset()                                    # nothing recorded: no raise
+
+
+def test_table_read_back_leaves_the_live_plan_alone():
+    """build_visible_page_table & co. between the blocks of a non-keyframe: the row table and
+    the device-side token count the later blocks attend through are those of the frame's plan
+    (cache plus the frame's own rows), not the read-back's."""
+    T, n_sp, H = 21, 5, 2
+    m = make("frame_pages", 4, T=T, n_sp=n_sp, scale=1, window=2, max_total=32, H=H, blocks=2, device_token_counts=True)
+    g = torch.Generator().manual_seed(4)
+    for _ in range(3):
+        for b in range(2):
+            q, k, v = frame(T, H, g)
+            m.step(b, q.cuda(), k.cuda(), v.cuda(), keyframe=[True])
+    q, k, v = (x.cuda() for x in frame(T, H, g))
+    m.step(0, q, k, v, keyframe=[False])
+    rows_before = m._kv_rows[0].clone()
+    count_before = m.device_header()["plan_kv_tokens"]
+    assert count_before == 3 * T + T             # three cached frames and the frame's own rows
+    ids = m.build_visible_page_table(0)
+    assert len(ids) == 3 * math.ceil(T / 4)
+    assert m.compute_last_page_len(0) == T - (math.ceil(T / 4) - 1) * 4
+    assert torch.equal(m._kv_rows[0], rows_before)
+    assert m.device_header()["plan_kv_tokens"] == count_before
+    out1 = m.step(1, q, k, v, keyframe=[False])
+    assert torch.isfinite(out1.float()).all()
 
 
 @pytest.mark.parametrize("layout,page_size", [("two_stream", None), ("two_stream", 16), ("frame_pages", 16)])
