@@ -24,7 +24,7 @@
 extern "C" {
 #endif
 
-#define LBM_ABI_VERSION 2
+#define LBM_ABI_VERSION 3
 
 #define LBM_OK 0
 #define LBM_ERR_INVALID 1     /* bad argument (null pointer, negative size, bad enum)      */
@@ -43,6 +43,10 @@ extern "C" {
 #define LBM_ROPE_HALF_SPLIT 1
 
 #define LBM_MAX_STREAMS 16
+
+/* MiB of device memory the library keeps as a static scratch array on every GPU it runs on
+ * (lbm_attn_run_static). */
+#define LBM_STATIC_SCRATCH_MIB 64
 
 /* Table operations, executed in this fixed order when several bits are set. */
 #define LBM_OP_RESET 1
@@ -236,6 +240,21 @@ int lbm_attn_run(const void* q, const void* pool, void* out, const void* self_k,
                  int32_t n_streams, int32_t num_heads, int32_t head_dim, int32_t page_size,
                  int32_t dtype, float sm_scale, void* workspace, size_t workspace_bytes,
                  void* stream);
+
+/* lbm_attn_run without a workspace argument and without any allocation: the split-KV partials
+ * go into a static device array of LBM_STATIC_SCRATCH_MIB MiB that lives in the library (one
+ * copy per GPU, held until the process ends).  No counterpart in the reference; it is for
+ * callers that cannot allocate device memory - code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc.  Same arguments, results (bit for bit) and error
+ * codes as lbm_attn_run; a batch whose partials do not fit returns LBM_ERR_WORKSPACE and
+ * launches nothing.  The first call on a device looks the array's address up (no allocation,
+ * but make that call outside a stream capture).  All calls on one GPU share the array: calls
+ * that overlap in time on one GPU (two streams, two threads) race on it and must be
+ * serialised by the caller; nothing in the array has to be cleared between calls. */
+int lbm_attn_run_static(const void* q, const void* pool, void* out, const void* self_k,
+                        const void* self_v, const int32_t* kv_rows, const lbm_attn_stream* streams,
+                        int32_t n_streams, int32_t num_heads, int32_t head_dim, int32_t page_size,
+                        int32_t dtype, float sm_scale, void* stream);
 
 #ifdef __cplusplus
 }

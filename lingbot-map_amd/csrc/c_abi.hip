@@ -193,4 +193,26 @@ int lbm_attn_run_live(const void* q, const void* pool, void* out, const void* se
                            stream);
 }
 
+int lbm_attn_run_static(const void* q, const void* pool, void* out, const void* self_k,
+                        const void* self_v, const int32_t* kv_rows, const lbm_attn_stream* streams,
+                        int32_t n_streams, int32_t num_heads, int32_t head_dim, int32_t page_size,
+                        int32_t dtype, float sm_scale, void* stream) {
+  int rc = lbm_check_attn_streams(streams, n_streams, "lbm_attn_run_static");
+  if (rc != LBM_OK) return rc;
+  if (num_heads <= 0 || head_dim <= 0) return lbm_fail(LBM_ERR_INVALID, "lbm_attn_run_static: non-positive size");
+  LbmAttnSchedule sch;
+  lbm_attn_schedule(streams, n_streams, num_heads, &sch);
+  const size_t need = lbm_attn_schedule_bytes(sch, num_heads, head_dim);
+  void* ws = nullptr;
+  size_t ws_bytes = 0;
+  rc = lbm_static_scratch(&ws, &ws_bytes);
+  if (rc != LBM_OK) return rc;
+  if (need > ws_bytes)
+    return lbm_fail(LBM_ERR_WORKSPACE, "lbm_attn_run_static: this batch needs %zu bytes of scratch, the static array holds %zu "
+                    "(LBM_STATIC_SCRATCH_MIB = %d); use lbm_attn_run with a workspace of your own",
+                    need, ws_bytes, LBM_STATIC_SCRATCH_MIB);
+  return lbm_attn_run_impl("lbm_attn_run_static", q, pool, out, self_k, self_v, kv_rows, nullptr, streams, n_streams,
+                           num_heads, head_dim, page_size, dtype, sm_scale, ws, ws_bytes, stream);
+}
+
 }  // extern "C"

@@ -56,4 +56,8 @@ int lbm_launch_attention(const void* q, const void* pool, void* out, const void*
                          int num_heads, int head_dim, int page_size, int dtype, float sm_scale,
                          void* workspace, hipStream_t stream);
 
+// Address and size of the library's static device scratch array on the current device (looked
+// up once per device; no allocation).
+int lbm_static_scratch(void** ptr, size_t* bytes);
+
 #endif  // LBM_INTERNAL_H

@@ -37,6 +37,7 @@
 // shared by all eight waves through a three-stage LDS ring with one workgroup barrier per tile.
 #include <hip/hip_runtime.h>
 #include <climits>
+#include <mutex>
 #include "lbm_internal.h"
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
@@ -1287,4 +1288,37 @@ int lbm_launch_attention(const void* q, const void* pool, void* out, const void*
     rc = lbm_check_launch("lbm_attn_combine_bf16_kernel");
   }
   return rc;
+}
+
+// ---------------------------------------------------------------------------- static scratch
+// Workspace for callers that cannot allocate (lbm_attn_run_static): split-KV partials and the
+// few-query partials go into this file-scope device array instead of a caller's buffer.  Every
+// GPU the library runs on holds its own copy at its own address until the process ends; the
+// array's name is only a host-side handle, so the address is looked up once per device with
+// that device current and the kernels get the looked-up pointer like any other workspace.
+// Nothing in it has to start at zero: every partial a launch reads was written by that launch.
+namespace {
+constexpr size_t kStaticScratchBytes = (size_t)LBM_STATIC_SCRATCH_MIB << 20;
+constexpr int kMaxDevices = 64;
+}  // namespace
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+static void* g_scratch_ptr[kMaxDevices];
+static std::mutex g_scratch_mutex;
+
+int lbm_static_scratch(void** ptr, size_t* bytes) {
+  int dev = -1;
+  const hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return lbm_fail(LBM_ERR_HIP, "hipGetDevice: %s", hipGetErrorString(e));
+  if (dev < 0 || dev >= kMaxDevices) return lbm_fail(LBM_ERR_UNSUPPORTED, "device ordinal %d outside [0, %d)", dev, kMaxDevices);
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (!g_scratch_ptr[dev]) {
+    void* p = nullptr;
+    const hipError_t es = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (es != hipSuccess || !p)
+      return lbm_fail(LBM_ERR_HIP, "hipGetSymbolAddress(static scratch) on device %d: %s", dev, hipGetErrorString(es));
+    g_scratch_ptr[dev] = p;
+  }
+  *ptr = g_scratch_ptr[dev];
+  *bytes = kStaticScratchBytes;
+  return LBM_OK;
 }

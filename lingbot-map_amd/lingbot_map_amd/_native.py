@@ -13,6 +13,7 @@ DTYPE_BF16, DTYPE_F32 = 0, 1
 LAYOUT_TWO_STREAM, LAYOUT_FRAME_PAGES = 0, 1
 ROPE_INTERLEAVED, ROPE_HALF_SPLIT = 0, 1
 MAX_STREAMS = 16
+STATIC_SCRATCH_MIB = 64
 OP_RESET, OP_ROLLBACK, OP_APPEND, OP_EVICT, OP_PLAN = 1, 2, 4, 8, 16
 TERR_NAMES = {1: "patch page pool exhausted", 2: "special page pool exhausted", 4: "window ring full",
               8: "trajectory memory full", 16: "rollback underflow", 32: "visible token count mismatch"}
@@ -20,7 +21,7 @@ HDR = {"frame_count": 0, "n_anchor": 1, "win_head": 2, "win_count": 3, "n_free_p
        "n_free_special": 5, "n_special_pages": 6, "special_tokens": 7, "n_memory": 8,
        "n_memory_pages": 9, "error": 10, "plan_kv_tokens": 11, "plan_n_pages": 12}
 HDR_WORDS = 16
-ABI_VERSION = 2
+ABI_VERSION = 3
 
 
 class CacheGeom(C.Structure):
@@ -40,7 +41,8 @@ class AttnStream(C.Structure):
 
 
 SYMBOLS = ("lbm_abi_version", "lbm_last_error", "lbm_tables_words", "lbm_tables_step",
-           "lbm_rows_from_pages", "lbm_kv_append", "lbm_qkv_prepare", "lbm_residual_norm", "lbm_attn_workspace_bytes", "lbm_attn_run", "lbm_attn_run_live")
+           "lbm_rows_from_pages", "lbm_kv_append", "lbm_qkv_prepare", "lbm_residual_norm", "lbm_attn_workspace_bytes", "lbm_attn_run", "lbm_attn_run_live",
+           "lbm_attn_run_static")
 
 
 def _load():
@@ -72,6 +74,8 @@ def _load():
     lib.lbm_attn_run_live.restype = C.c_int
     lib.lbm_attn_run_live.argtypes = [vp, vp, vp, vp, vp, vp, vp, p(AttnStream), i32, i32, i32, i32, i32,
                                       C.c_float, vp, C.c_size_t, vp]
+    lib.lbm_attn_run_static.restype = C.c_int
+    lib.lbm_attn_run_static.argtypes = [vp, vp, vp, vp, vp, vp, p(AttnStream), i32, i32, i32, i32, i32, C.c_float, vp]
     if lib.lbm_abi_version() != ABI_VERSION:
         raise RuntimeError(f"{LIB_PATH}: ABI version {lib.lbm_abi_version()}, binding expects {ABI_VERSION}")
     return lib

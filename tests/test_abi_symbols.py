@@ -36,6 +36,7 @@ def test_binding_constants_match_header():
     defs = {m.group(1): int(m.group(2)) for m in re.finditer(r"#define\s+(LBM_[A-Z_0-9]+)\s+(\d+)\b", text)}
     assert defs["LBM_ABI_VERSION"] == N.ABI_VERSION
     assert defs["LBM_MAX_STREAMS"] == N.MAX_STREAMS
+    assert defs["LBM_STATIC_SCRATCH_MIB"] == N.STATIC_SCRATCH_MIB
     assert (defs["LBM_OP_RESET"], defs["LBM_OP_ROLLBACK"], defs["LBM_OP_APPEND"], defs["LBM_OP_EVICT"],
             defs["LBM_OP_PLAN"]) == (N.OP_RESET, N.OP_ROLLBACK, N.OP_APPEND, N.OP_EVICT, N.OP_PLAN)
     assert defs["LBM_HDR_WORDS"] == N.HDR_WORDS
