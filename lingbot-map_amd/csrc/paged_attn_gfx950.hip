@@ -112,6 +112,7 @@ __device__ __forceinline__ float swap_max(float x) {
 __global__ __launch_bounds__(kThreads, 1) void lbm_attn_bf16_d64_kernel(AttnArgs a) {
   __shared__ __attribute__((aligned(16))) unsigned short lds_k[kStages][kKvTile * kKStride];
   __shared__ __attribute__((aligned(16))) unsigned short lds_v[kStages][kKvTile * kVStride];
+  __shared__ __attribute__((aligned(16))) unsigned short lds_q[kWaves][kQPerWave * kKStride];   // per-wave patch: Q on the way in
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int n32 = lane & 31, g = lane >> 5;
@@ -157,24 +158,36 @@ __global__ __launch_bounds__(kThreads, 1) void lbm_attn_bf16_d64_kernel(AttnArgs
   const unsigned row_bytes = (unsigned)H * 128u;
 
   // ---- Q fragments (B operand of S^T = K Q^T): lane holds q row n32, d = ks*16 + g*8 .. +8.
+  // Each wavefront reads its 64 query rows as whole 128-byte rows (eight lanes per row), parks
+  // them in its own LDS patch and picks the fragments up from there; read directly in the
+  // fragment layout every load instruction would touch 64 different rows with 16 bytes each.
   // The softmax scale and log2(e) are folded into Q here (one extra bf16 rounding of q), so
   // the MFMA result is already the exponent of 2.
   bf16x8 qf[2][4];
   const int q_row0 = qt * kQTile + wave * kQPerWave;
+  {
+    unsigned short* patch = lds_q[wave];
+    u32x4 raw[kQPerWave / 8];
 #pragma unroll
-  for (int qb = 0; qb < 2; ++qb) {
-    const int r = q_row0 + qb * 32 + n32;
-    const unsigned short* qp = a.q + ((size_t)(sp.q_begin + r) * H + head) * 64 + g * 8;
-#pragma unroll
-    for (int ks = 0; ks < 4; ++ks) {
-      u32x4 v = {0u, 0u, 0u, 0u};
-      if (r < sp.q_rows) v = *(const u32x4*)(qp + ks * 16);
-      const bf16x8 raw = __builtin_bit_cast(bf16x8, v);
-      f32x8 f = __builtin_convertvector(raw, f32x8);
-#pragma unroll
-      for (int j = 0; j < 8; ++j) f[j] *= a.scale_log2;
-      qf[qb][ks] = __builtin_convertvector(f, bf16x8);
+    for (int k = 0; k < kQPerWave / 8; ++k) {
+      const int r = q_row0 + k * 8 + (lane >> 3);
+      raw[k] = u32x4{0u, 0u, 0u, 0u};
+      if (r < sp.q_rows) raw[k] = *(const u32x4*)(a.q + ((size_t)(sp.q_begin + r) * H + head) * 64 + (lane & 7) * 8);
     }
+#pragma unroll
+    for (int k = 0; k < kQPerWave / 8; ++k)
+      *(u32x4*)&patch[(k * 8 + (lane >> 3)) * kKStride + (lane & 7) * 8] = raw[k];
+    __syncthreads();   // (a wavefront only reads its own patch; the barrier orders its lanes' writes and reads)
+#pragma unroll
+    for (int qb = 0; qb < 2; ++qb)
+#pragma unroll
+      for (int ks = 0; ks < 4; ++ks) {
+        const bf16x8 rawf = __builtin_bit_cast(bf16x8, *(const u32x4*)&patch[(qb * 32 + n32) * kKStride + ks * 16 + g * 8]);
+        f32x8 f = __builtin_convertvector(rawf, f32x8);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) f[j] *= a.scale_log2;
+        qf[qb][ks] = __builtin_convertvector(f, bf16x8);
+      }
   }
   // One more 16-wide step of the QK contraction carries the softmax reference: K side is the
   // constant row (-1, -1, 0, ...), Q side is (m_hi, m_lo, 0, ...) with m_hi + m_lo = m_run
@@ -186,21 +199,16 @@ __global__ __launch_bounds__(kThreads, 1) void lbm_attn_bf16_d64_kernel(AttnArgs
   u32x4 qaug_bits[2] = {{0u, 0u, 0u, 0u}, {0u, 0u, 0u, 0u}};
   if (g == 0) qaug_bits[0][1] = qaug_bits[1][1] = 0x7180u;  // bf16 2^100
 
+  // Accumulators and softmax reference; (re)initialised at the start of each pass below.
   f32x16 o[2][2];
-#pragma unroll
-  for (int qb = 0; qb < 2; ++qb)
-#pragma unroll
-    for (int db = 0; db < 2; ++db)
-#pragma unroll
-      for (int i = 0; i < 16; ++i) o[qb][db][i] = 0.f;
-  float m_run[2] = {0.f, 0.f};  // moved to the first half's maxima before the loop
+  float m_run[2];
   // Row sums (softmax denominators) are accumulated by the matrix pipe as well: a 16x16x32 MFMA
   // with a 0/1 selector as A and the numerators, exactly as they sit in the registers for PV,
   // as B.  Read as a 32x16 B operand the numerator registers hold, for column n, query n in
   // k rows 0-7 and 16-23 and query n+16 in k rows 8-15 and 24-31; selector row 0 picks the
   // former and row 1 the latter, so lane n < 16 ends up with the sums of query n (element 0)
   // and of query n+16 (element 1) of the block, and every other element stays 0.
-  f32x4 lacc[2] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
+  f32x4 lacc[2];
   const unsigned sel_word = (lane == 0 || lane == 32 || lane == 17 || lane == 49) ? 0x3F803F80u : 0u;
   const bf16x8 lsel = __builtin_bit_cast(bf16x8, u32x4{sel_word, sel_word, sel_word, sel_word});
 
@@ -422,82 +430,203 @@ __global__ __launch_bounds__(kThreads, 1) void lbm_attn_bf16_d64_kernel(AttnArgs
     asm volatile("" : "+v"(pd[0][0]), "+v"(pd[0][1]), "+v"(pd[1][0]), "+v"(pd[1][1]));             \
     hot = (chk & 0x40004000u) != 0u;                                                             \
   }
+// The same half-step without a softmax reference (scores go to exp2 as they come out of the
+// QK^T product) and without the test: 20 slices, QK^T in slices 12-19 with its first k-step
+// starting from zero.  Only for half-steps whose 32 KV rows are all valid tokens.
+#define LBM_FSLICE(j, cur, pd, prev, next, st_pv, ks_pv, st_qk, h_qk, st_vn, ks_vn)                \
+  {                                                                                              \
+    if ((j) < 4)                                                                                 \
+      o[(j) & 1][(j) >> 1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(                            \
+          vnext[(j) >> 1], prev[(j) & 1][0], o[(j) & 1][(j) >> 1], 0, 0, 0);                     \
+    else if ((j) < 8)                                                                            \
+      o[(j) & 1][((j) - 4) >> 1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(                      \
+          va[((j) - 4) >> 1], prev[(j) & 1][1], o[(j) & 1][((j) - 4) >> 1], 0, 0, 0);            \
+    else if ((j) < 12)                                                                           \
+      lacc[(j) & 1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(                                   \
+          lsel, prev[(j) & 1][((j) - 8) >> 1], lacc[(j) & 1], 0, 0, 0);                          \
+    else if ((j) < 14)                                                                           \
+      next[(j) & 1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka[0], qf[(j) & 1][0], zero16, 0, 0, 0); \
+    else                                                                                         \
+      next[(j) & 1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(                                   \
+          ka[((j) - 12) >> 1], qf[(j) & 1][((j) - 12) >> 1], next[(j) & 1], 0, 0, 0);            \
+    if ((j) < 16) {                                                                              \
+      e[2 * (j)] = __builtin_amdgcn_exp2f(cur[(j) >> 3][(2 * (j)) & 15]);                        \
+      e[2 * (j) + 1] = __builtin_amdgcn_exp2f(cur[(j) >> 3][(2 * (j) + 1) & 15]);                \
+    }                                                                                            \
+    if ((j) >= 1 && (j) <= 16) {                                                                 \
+      constexpr int c = (j) - 1, ci = (2 * c) & 15;                                              \
+      pd[c >> 3][ci >> 3][ci & 7] = (__bf16)e[2 * c];                                            \
+      pd[c >> 3][ci >> 3][(ci & 7) + 1] = (__bf16)e[2 * c + 1];                                  \
+    }                                                                                            \
+    if ((j) == 0) va[0] = v_frag(st_pv, ks_pv, 0);                                               \
+    if ((j) == 1) va[1] = v_frag(st_pv, ks_pv, 1);                                               \
+    if ((j) == 8 || (j) == 10 || (j) == 12 || (j) == 14)                                         \
+      ka[((j) - 8) >> 1] = __builtin_bit_cast(                                                   \
+          bf16x8, *(const u32x4*)&lds_k[st_qk][((h_qk) * 32 + n32) * kKStride + (((j) - 8) >> 1) * 16 + g * 8]); \
+    if ((j) == 16) vnext[0] = v_frag(st_vn, ks_vn, 0);                                           \
+    if ((j) == 17) vnext[1] = v_frag(st_vn, ks_vn, 1);                                           \
+    __builtin_amdgcn_sched_barrier(0);                                                           \
+  }
+#define LBM_F4(j, ...) LBM_FSLICE(j, __VA_ARGS__) LBM_FSLICE(j + 1, __VA_ARGS__) LBM_FSLICE(j + 2, __VA_ARGS__) LBM_FSLICE(j + 3, __VA_ARGS__)
+#define LBM_FAST_HALF_STEP(cur, pd, prev, next, st_pv, ks_pv, st_qk, h_qk, st_vn, ks_vn)           \
+  {                                                                                              \
+    bf16x8 va[2], ka[4];                                                                         \
+    float e[32];                                                                                 \
+    __builtin_amdgcn_sched_barrier(0);                                                           \
+    LBM_F4(0, cur, pd, prev, next, st_pv, ks_pv, st_qk, h_qk, st_vn, ks_vn)                       \
+    LBM_F4(4, cur, pd, prev, next, st_pv, ks_pv, st_qk, h_qk, st_vn, ks_vn)                       \
+    LBM_F4(8, cur, pd, prev, next, st_pv, ks_pv, st_qk, h_qk, st_vn, ks_vn)                       \
+    LBM_F4(12, cur, pd, prev, next, st_pv, ks_pv, st_qk, h_qk, st_vn, ks_vn)                      \
+    LBM_F4(16, cur, pd, prev, next, st_pv, ks_pv, st_qk, h_qk, st_vn, ks_vn)                      \
+  }
   f32x16 zero16;
 #pragma unroll
   for (int i = 0; i < 16; ++i) zero16[i] = 0.f;
 
-  // ---- prologue: K(0), K(1), V(0) into the ring; the V stage the first PV reads is zeroed
-  put_k(0, fetch(row_entry(t0), pool_k, own_k));
-  put_k(1, fetch(row_entry(t0 + 1), pool_k, own_k));
-  put_v(0, fetch(row_entry(t0), pool_v, own_v));
-  {
-    const u32x4 zero = {0u, 0u, 0u, 0u};
-    put_v(2, zero);
-  }
-#pragma unroll
-  for (int qb = 0; qb < 2; ++qb)
-#pragma unroll
-    for (int kk = 0; kk < 2; ++kk) pB[qb][kk] = __builtin_bit_cast(bf16x8, u32x4{0u, 0u, 0u, 0u});
-  int ek = row_entry(t0 + 2), ev = row_entry(t0 + 1);
-  __syncthreads();
-  qk_half(0, 0, kv_tokens - t0 * kKvTile, sA);
-  {
-    // the reference starts at the maxima of the first half
-    float mx[2];
-    row_max(sA, mx);
+  // Iterations [0, n_fast) of this split see only complete 32-token halves (their own second
+  // half and the first half of the tile after them) and take the half-step without reference;
+  // the iterations around the ragged end of the KV list take the one with the masking k-step.
+  const int n_fast = min(max((kv_tokens - 96) / kKvTile - t0 + (kv_tokens >= 96 ? 1 : 0), 0), n);
+
+  // Two passes at most.  The first one uses no softmax reference at all: the numerators are
+  // 2^score, which is exact softmax arithmetic as long as nothing leaves the range of fp32 /
+  // bf16 (both carry 8 exponent bits and the relative precision does not depend on the
+  // magnitude).  Scores in log2 units beyond about +-100 - unheard of behind a q/k LayerNorm -
+  // make a row sum or an output overflow or vanish; the check after the pass sees that and the
+  // whole workgroup repeats its split with a reference that follows the row maxima (pass 1).
+  for (int pass = 0; pass < 2; ++pass) {
+    const bool safe = pass != 0;
 #pragma unroll
     for (int qb = 0; qb < 2; ++qb) {
-      const float d = move_reference(qb, mx[qb] + kHeadroom);
 #pragma unroll
-      for (int i = 0; i < 16; ++i) sA[qb][i] -= d;
+      for (int db = 0; db < 2; ++db)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) o[qb][db][i] = 0.f;
+      lacc[qb] = f32x4{0.f, 0.f, 0.f, 0.f};
+      m_run[qb] = 0.f;
+      qaug_bits[qb][0] = 0u;
     }
-  }
-  vnext[0] = v_frag(2, 2, 0);
-  vnext[1] = v_frag(2, 2, 1);
 
-  int st_k = 0, st_v = 0, st_vm1 = 2;  // stages of K(i), V(i), V(i-1)
-  for (int i = 0; i < n; ++i) {
-    const int t = t0 + i;
-    int st_k1 = st_k + 1; if (st_k1 >= kStages) st_k1 -= kStages;
-    int st_k2 = st_k1 + 1; if (st_k2 >= kStages) st_k2 -= kStages;
-    int st_v1 = st_v + 1; if (st_v1 >= kStages) st_v1 -= kStages;
-    const int n_valid = kv_tokens - t * kKvTile;
-    bool hot;
-
-    // global fetches of K(i+2), V(i+1) start here and land in the ring at the end of the step
-    const u32x4 kreg = fetch(ek, pool_k, own_k);
-    const u32x4 vreg = fetch(ev, pool_v, own_v);
-    ek = row_entry(t + 3);
-    ev = row_entry(t + 2);
-
-    // half 0 of tile i: softmax(sA) -> pA | PV(tile i-1, half 1) with pB | QK(tile i, half 1) -> sB
-    LBM_HALF_STEP(sA, pA, pB, sB, st_vm1, 3, st_k, 1, n_valid, st_v, 0, hot);
-    if (__builtin_amdgcn_ballot_w64(hot)) raise_reference(sA, pA, sB);
-
-    // half 1 of tile i: softmax(sB) -> pB | PV(tile i, half 0) with pA | QK(tile i+1, half 0) -> sA
-    // (after the last tile that QK reads a stale stage; its result is unused)
-    LBM_HALF_STEP(sB, pB, pA, sA, st_v, 1, st_k1, 0, n_valid - kKvTile, st_v, 2, hot);
-    if (__builtin_amdgcn_ballot_w64(hot)) raise_reference(sB, pB, sA);
-
-    // ring upkeep: K(i+2), V(i+1) (past the last tile: stages nobody reads any more)
-    put_k(st_k2, kreg);
-    put_v(st_v1, vreg);
-    __syncthreads();
-    st_k = st_k1;
-    st_vm1 = st_v;
-    st_v = st_v1;
-  }
-  // PV and row sums of the last half: pB with half 1 of V(n-1), first k-step already in vnext
-  {
-    pv_step(vnext, pB, 0);
-    bf16x8 va[2] = {v_frag(st_vm1, 3, 0), v_frag(st_vm1, 3, 1)};
-    pv_step(va, pB, 1);
+    // ---- prologue: K(0), K(1), V(0) into the ring; the V stage the first PV reads is zeroed
+    put_k(0, fetch(row_entry(t0), pool_k, own_k));
+    put_k(1, fetch(row_entry(t0 + 1), pool_k, own_k));
+    put_v(0, fetch(row_entry(t0), pool_v, own_v));
+    {
+      const u32x4 zero = {0u, 0u, 0u, 0u};
+      put_v(2, zero);
+    }
 #pragma unroll
     for (int qb = 0; qb < 2; ++qb)
 #pragma unroll
-      for (int kk = 0; kk < 2; ++kk)
-        lacc[qb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(lsel, pB[qb][kk], lacc[qb], 0, 0, 0);
+      for (int kk = 0; kk < 2; ++kk) pB[qb][kk] = __builtin_bit_cast(bf16x8, u32x4{0u, 0u, 0u, 0u});
+    // in flight across the first iteration: K(2), V(1); entries of the fetches after them
+    u32x4 kreg = fetch(row_entry(t0 + 2), pool_k, own_k);
+    u32x4 vreg = fetch(row_entry(t0 + 1), pool_v, own_v);
+    int ek = row_entry(t0 + 3), ev = row_entry(t0 + 2);
+    __syncthreads();
+    qk_half(0, 0, kv_tokens - t0 * kKvTile, sA);
+    if (safe) {
+      // the reference starts kHeadroom above the maxima of the first half
+      float mx[2];
+      row_max(sA, mx);
+#pragma unroll
+      for (int qb = 0; qb < 2; ++qb) {
+        const float d = move_reference(qb, mx[qb] + kHeadroom);
+#pragma unroll
+        for (int i = 0; i < 16; ++i) sA[qb][i] -= d;
+      }
+    }
+    vnext[0] = v_frag(2, 2, 0);
+    vnext[1] = v_frag(2, 2, 1);
+
+    int st_k = 0, st_v = 0, st_vm1 = 2;  // stages of K(i), V(i), V(i-1)
+    // Common frame of one tile iteration.  K/V rows travel global -> registers -> LDS ring with
+    // a full iteration in the registers: the fetches of K(i+3), V(i+2) start at the top of
+    // iteration i, and the rows fetched one iteration earlier (K(i+2), V(i+1), long since
+    // arrived) are written into the ring between the two half-steps, so neither the wait for
+    // the loads nor the LDS write sits in front of the barrier that ends the iteration.  Past
+    // the last tile the data lands in stages nobody reads any more.  The row entry fetched for
+    // K now serves V in the next iteration.
+#define LBM_TILE_ITERATION(PRE, HALF0, HALF1)                                        \
+    {                                                                                \
+      const int t = t0 + i;                                                          \
+      int st_k1 = st_k + 1; if (st_k1 >= kStages) st_k1 -= kStages;                  \
+      int st_k2 = st_k1 + 1; if (st_k2 >= kStages) st_k2 -= kStages;                 \
+      int st_v1 = st_v + 1; if (st_v1 >= kStages) st_v1 -= kStages;                  \
+      const u32x4 khold = kreg, vhold = vreg;                                        \
+      kreg = fetch(ek, pool_k, own_k);                                               \
+      vreg = fetch(ev, pool_v, own_v);                                               \
+      ev = ek;                                                                       \
+      ek = row_entry(t + 4);                                                         \
+      PRE                                                                            \
+      HALF0                                                                          \
+      put_k(st_k2, khold);                                                           \
+      put_v(st_v1, vhold);                                                           \
+      HALF1                                                                          \
+      __syncthreads();                                                               \
+      st_k = st_k1;                                                                  \
+      st_vm1 = st_v;                                                                 \
+      st_v = st_v1;                                                                  \
+    }
+    int i = 0;
+    // half 0 of tile i: softmax(sA) -> pA | PV(tile i-1, half 1) with pB | QK(tile i, half 1) -> sB
+    // half 1 of tile i: softmax(sB) -> pB | PV(tile i, half 0) with pA | QK(tile i+1, half 0) -> sA
+    for (const int n_f = safe ? 0 : n_fast; i < n_f; ++i)
+      LBM_TILE_ITERATION(
+        ,
+        LBM_FAST_HALF_STEP(sA, pA, pB, sB, st_vm1, 3, st_k, 1, st_v, 0);,
+        LBM_FAST_HALF_STEP(sB, pB, pA, sA, st_v, 1, st_k1, 0, st_v, 2);
+      )
+    for (; i < n; ++i)
+      LBM_TILE_ITERATION(
+        const int n_valid = kv_tokens - t * kKvTile;
+        bool hot;,
+        LBM_HALF_STEP(sA, pA, pB, sB, st_vm1, 3, st_k, 1, n_valid, st_v, 0, hot);
+        if (safe && __builtin_amdgcn_ballot_w64(hot)) raise_reference(sA, pA, sB);,
+        /* after the last tile this QK reads a stale stage; its result is unused */
+        LBM_HALF_STEP(sB, pB, pA, sA, st_v, 1, st_k1, 0, n_valid - kKvTile, st_v, 2, hot);
+        if (safe && __builtin_amdgcn_ballot_w64(hot)) raise_reference(sB, pB, sA);
+      )
+#undef LBM_TILE_ITERATION
+    // PV and row sums of the last half: pB with half 1 of V(n-1), first k-step already in vnext
+    {
+      pv_step(vnext, pB, 0);
+      bf16x8 va[2] = {v_frag(st_vm1, 3, 0), v_frag(st_vm1, 3, 1)};
+      pv_step(va, pB, 1);
+#pragma unroll
+      for (int qb = 0; qb < 2; ++qb)
+#pragma unroll
+        for (int kk = 0; kk < 2; ++kk)
+          lacc[qb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(lsel, pB[qb][kk], lacc[qb], 0, 0, 0);
+    }
+    if (safe) break;
+    // Did the pass without reference stay in range?  Compared as integers (non-negative floats
+    // order like their bit patterns; NaN, infinity and negative values land above every bound).
+    bool bad = false;
+    if (n > 0) {
+      unsigned top = 0u;
+#pragma unroll
+      for (int qb = 0; qb < 2; ++qb)
+#pragma unroll
+        for (int db = 0; db < 2; ++db)
+#pragma unroll
+          for (int i = 0; i < 16; ++i) top = max(top, __builtin_bit_cast(unsigned, o[qb][db][i]) & 0x7FFFFFFFu);
+      bad = top >= 0x7F800000u;
+      if (lane < 16) {
+#pragma unroll
+        for (int qb = 0; qb < 2; ++qb)
+#pragma unroll
+          for (int h2 = 0; h2 < 2; ++h2) {
+            const unsigned lb = __builtin_bit_cast(unsigned, lacc[qb][h2]);
+            bad = bad || lb < 0x12800000u /* 2^-90 */ || lb > 0x71800000u /* 2^100 */;
+          }
+      }
+    }
+    if (!__syncthreads_or(bad)) break;
   }
+#undef LBM_FAST_HALF_STEP
+#undef LBM_F4
+#undef LBM_FSLICE
 #undef LBM_HALF_STEP
 #undef LBM_S4
 #undef LBM_SLICE
