@@ -50,11 +50,17 @@ def rows_from_pages(page_ids, page_lens, page_size, dev):
     return rows, n_tok
 
 
-def check_bf16(out, ref):
+def check_bf16(out, ref, rel_mean=None):
+    """The absolute bars; with ``rel_mean`` also mean-abs error <= rel_mean * mean |ref|, for
+    shapes whose outputs are small (N(0,1) values averaged over thousands of tokens), where the
+    absolute bars alone would let a dropped tile pass."""
     err = (out.float() - ref.float()).abs()
     assert torch.isfinite(out.float()).all()
     assert err.max().item() <= BF16_MAX_ABS, f"max-abs {err.max().item()}"
     assert err.mean().item() <= BF16_MEAN_ABS, f"mean-abs {err.mean().item()}"
+    if rel_mean is not None:
+        assert err.mean().item() <= rel_mean * ref.float().abs().mean().item(), (
+            f"mean-abs {err.mean().item()} against mean |ref| {ref.float().abs().mean().item()}")
 
 
 @pytest.mark.parametrize("tq,n_pages,page_size,H", [(7, 3, 4, 2), (64, 9, 16, 16), (300, 70, 16, 4), (1004, 140, 16, 16)])
@@ -103,7 +109,7 @@ def test_attention_config2_shape_split_kv():
     rows, n_tok = rows_from_pages(ids, lens, S, dev)
     assert n_tok == 17068
     out = run_attention(q.to(dev), pool.to(dev), rows, [(0, T, 0, n_tok)], S)
-    check_bf16(out.cpu(), ref)
+    check_bf16(out.cpu(), ref, rel_mean=0.01)
 
 
 def test_attention_read_only_tail_and_two_streams():
@@ -247,24 +253,23 @@ def test_attention_edge_shapes():
     assert rc != N.OK and b"n_streams" in N.lib.lbm_last_error()
 
 
-@pytest.mark.parametrize("seed", range(6))
-def test_attention_random_shapes(seed):
-    """Seeded sweep over shapes the fixed cases do not hit: 1-3 streams with unrelated query
-    and KV sizes (1..1100 rows, 1..6000 tokens), 1..16 heads, page sizes 1..64, rows scattered
-    over the pool, sometimes a read-only tail, score spread from flat to peaked (for which the
-    bar is doubled, see below)."""
+def _random_shape_cases(seed, spreads, n_cases=5):
+    """Seeded draws of shapes the fixed cases do not hit: 1-3 streams with unrelated query and KV
+    sizes (1..1100 rows, 1..6000 tokens), 1..16 heads, page sizes 1..64, rows scattered over the
+    pool, sometimes a read-only tail; the keys are N(0, spread^2).  Yields (what, max-abs error,
+    mean-abs error) per stream of every launch."""
     from oracle.sdpa_cache import sdpa_nhd
     dev = torch.device("cuda:0")
     g = torch.Generator().manual_seed(1000 + seed)
     ri = lambda lo, hi: int(torch.randint(lo, hi + 1, (1,), generator=g))
-    for case in range(5):
+    for case in range(n_cases):
         H, D = [1, 2, 3, 8, 16][ri(0, 4)], 64
         S = [1, 4, 16, 64][ri(0, 3)]
         n_streams = ri(1, 3)
         qn = [ri(1, 1100) if ri(0, 2) else ri(1, 70) for _ in range(n_streams)]
         kn = [ri(1, 6000) if ri(0, 2) else ri(1, 130) for _ in range(n_streams)]
         tail = ri(0, 2) == 0
-        spread = [0.05, 1.0, 3.0][ri(0, 2)]
+        spread = spreads[ri(0, len(spreads) - 1)]
         n_slots = sum(kn) + 37
         pages = -(-n_slots // S)
         pool = torch.randn(pages, 2, S, H, D, generator=g)
@@ -293,11 +298,33 @@ def test_attention_random_shapes(seed):
         for (qb, nq, _, _), ref in zip(streams, refs):
             err = (out[qb:qb + nq].float() - ref.float()).abs()
             assert torch.isfinite(out[qb:qb + nq].float()).all()
-            # peaked scores (keys three times as long): the kernel rounds q * scale * log2(e) to
-            # bf16 once more than the reference does, which costs about 1 % of the output there
-            bar = 1.0 if spread <= 1.0 else 2.0
-            assert err.max().item() <= bar * BF16_MAX_ABS and err.mean().item() <= bar * BF16_MEAN_ABS, (
-                seed, case, H, S, qn, kn, tail, spread, err.max().item())
+            yield (seed, case, H, S, qn, kn, tail, spread), err.max().item(), err.mean().item()
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_attention_random_shapes(seed):
+    """Keys from nearly flat (spread 0.05) to the N(0,1) of every benchmark configuration."""
+    for what, err_max, err_mean in _random_shape_cases(seed, [0.05, 1.0, 1.0]):
+        assert err_max <= BF16_MAX_ABS and err_mean <= BF16_MEAN_ABS, (what, err_max, err_mean)
+
+
+@pytest.mark.xfail(strict=False, reason=(
+    "keys three times as long as any benchmark configuration draws them (N(0, 9) against N(0, 1)): the softmax "
+    "is then dominated by a handful of tokens and the one rounding the kernel adds to the reference's arithmetic - "
+    "q * scale * log2(e) is rounded to bf16 before the QK^T product - shows up undamped; the worst element of "
+    "some draws lands between 2e-2 and 4e-2.  The mean-abs bar holds; see test_attention_peaked_scores_mean_bar."))
+@pytest.mark.parametrize("seed", range(3))
+def test_attention_peaked_scores_max_bar(seed):
+    for what, err_max, _ in _random_shape_cases(seed, [3.0], n_cases=4):
+        assert err_max <= BF16_MAX_ABS, (what, err_max)
+
+
+@pytest.mark.parametrize("seed", range(3))
+def test_attention_peaked_scores_mean_bar(seed):
+    """The same peaked inputs: finite everywhere, mean-abs within the bar, and no element further
+    off than 4e-2 (two bf16 roundings of an O(1) output instead of one)."""
+    for what, err_max, err_mean in _random_shape_cases(seed, [3.0], n_cases=4):
+        assert err_mean <= BF16_MEAN_ABS and err_max <= 2 * BF16_MAX_ABS, (what, err_max, err_mean)
 
 
 @pytest.mark.parametrize("src,dst", [(torch.bfloat16, torch.bfloat16), (torch.float32, torch.bfloat16),
