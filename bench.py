@@ -330,90 +330,73 @@ def cpu_baseline(torch, kv_tokens: int, blocks: int) -> dict:
     }
 
 
-def aggregator_step(torch, blocks: int, steps: int, warmup: int, windows=(WINDOW,)) -> dict:
-    """One streamed frame (a 3 x 378 x 518 image) through the image encoder's ViT-L trunk (patch
-    embedding, 24 blocks; lingbot_map/layers/vision_transformer.py:383-394) and through `blocks`
-    groups of (frame block, global block) of the aggregator (lingbot_map/aggregator/stream.py:
-    415-529), all at ViT-L size (dim 1024, 16 heads, MLP 4096, LayerNorm, LayerScale; qk-norm and
-    rotary embedding in the aggregator blocks), random init, bf16.  The global blocks run the HIP
-    cache path, every block's pre-attention producer and cache-less attention are HIP kernels
-    too; linears, LayerNorm, GELU and the patch-embedding convolution are PyTorch-ROCm library
-    calls.  The prediction heads are not part of the step.  `windows` holds one sliding window
-    per stream: more than one entry runs that many independent streams as one ragged batch (a
-    step is then one frame of every stream)."""
-    from lingbot_map_amd import (HipPagedBlock, HipPagedKVCacheManager, PositionGetter, RotaryPositionEmbedding2D,
-                                 RotaryPositionEmbedding3D)
+def aggregator_step(torch, blocks: int, steps: int, warmup: int, windows=(WINDOW,), keyframe_interval: int = 1) -> dict:
+    """One streamed frame (a 3 x 378 x 518 image) of every stream through the product's aggregator
+    shell (`lingbot_map_amd.HipAggregatorStream`): the image encoder's ViT-L trunk (patch
+    convolution + 24 plain blocks + LayerNorm; lingbot_map/layers/vision_transformer.py:383-394)
+    and `blocks` groups of (frame block, global block) (lingbot_map/aggregator/stream.py:415-529,
+    base.py:575-606), special tokens first, group outputs concatenated, all at ViT-L size (dim
+    1024, 16 heads, MLP 4096, LayerNorm, LayerScale; qk-norm and rotary embeddings in the
+    aggregator blocks), random init, bf16.  The global blocks run the HIP cache path, every
+    block's pre-attention producer and cache-less attention are HIP kernels too; linears,
+    LayerNorm, GELU and the patch convolution are PyTorch-ROCm library calls.  The prediction
+    heads are not part of the step.  `windows` holds one sliding window per stream: more than
+    one entry runs that many independent streams as one ragged batch (a step is then one frame
+    of every stream).  `keyframe_interval` > 1 caches every n-th frame only (config 4)."""
+    from lingbot_map_amd import GraphedAggregator, HipAggregatorStream, set_skip_append
     dev = torch.device("cuda:0")
-    dim = H * D
     torch.manual_seed(4)
-    # evicted frames leave no trajectory memory (as in the hot-path loop above), so the KV set
-    # stays at 17,068 tokens and a frame can also be replayed as a HIP graph
-    kw = dict(dim=dim, num_heads=H, mlp_ratio=4.0, qk_norm=True, init_values=0.01,
-              kv_cache_sliding_window=WINDOW, kv_cache_scale_frames=ANCHOR, kv_cache_cross_frame_special=False)
-    rope2d = RotaryPositionEmbedding2D()    # frame blocks: 2-D embedding over the 27 x 37 patch grid
-    frame_blocks = [HipPagedBlock(rope=rope2d, **kw).to(dev, torch.bfloat16).eval() for _ in range(blocks)]
-    global_blocks = [HipPagedBlock(rope=True, **kw).to(dev, torch.bfloat16).eval() for _ in range(blocks)]
-    encoder_blocks = [HipPagedBlock(dim=dim, num_heads=H, mlp_ratio=4.0, init_values=1.0).to(dev, torch.bfloat16).eval()
-                      for _ in range(24)]
-    patch_embed = torch.nn.Conv2d(3, dim, kernel_size=14, stride=14).to(dev, torch.bfloat16).eval()
     B = len(windows)
-    special = torch.randn(1, N_SPECIAL, dim, device=dev).to(torch.bfloat16).expand(B, -1, -1)   # class + register tokens
-    m = HipPagedKVCacheManager(blocks, ANCHOR + max(windows) + 16, T, H, D, torch.bfloat16, dev,
-                               num_special_tokens=N_SPECIAL, scale_frames=ANCHOR,
-                               sliding_window=list(windows) if B > 1 else windows[0],
-                               max_total_frames=256, page_size=PAGE, layout="frame_pages", num_streams=B)
+    # evicted frames leave no trajectory memory (as in the hot-path loop above), so the KV set
+    # stays at 17,068 tokens per full window
+    model = HipAggregatorStream(
+        img_size=518, patch_size=14, embed_dim=H * D, depth=blocks, num_heads=H, mlp_ratio=4.0, num_register_tokens=4,
+        qk_norm=True, init_values=0.01, patch_embed="vit", encoder_depth=24, enable_3d_rope=True, max_frame_num=156,
+        kv_cache_sliding_window=list(windows) if B > 1 else windows[0], kv_cache_scale_frames=ANCHOR,
+        kv_cache_cross_frame_special=False, use_scale_token=False, page_size=PAGE, layout="frame_pages",
+        num_streams=B).to(dev, torch.bfloat16).eval()
     g = torch.Generator(device=dev).manual_seed(4)
-    # rotary table of the global blocks for frame 40 of a stream (frame / row / column pairs 10 / 11 / 11)
-    rope3d = RotaryPositionEmbedding3D(attention_head_dim=D, patch_size=(1, 14, 14), max_seq_len=1024)
-    freqs = rope3d(ppf=1, pph=27, ppw=37, patch_start_idx=N_SPECIAL, device=dev, f_start=40, f_end=41)
-    assert freqs.shape == (1, 1, T, D // 2)
-    xs = [torch.rand(B, 3, 378, 518, generator=g, device=dev, dtype=torch.float32).to(torch.bfloat16) for _ in range(4)]
-    # (y, x) of every token: specials at (0, 0), patches on the grid shifted by one (lingbot_map/aggregator/base.py:434-440)
-    grid = PositionGetter()(1, 27, 37, dev)[0] + 1
-    pos2d = torch.cat([torch.zeros(N_SPECIAL, 2, dtype=grid.dtype, device=dev), grid])[None].expand(B, -1, -1).contiguous()
-    assert pos2d.shape == (B, T, 2)
+    xs = [torch.rand(B, 1, 3, 378, 518, generator=g, device=dev, dtype=torch.float32).to(torch.bfloat16) for _ in range(4)]
+    selected = [4, 11, 17, blocks - 1] if blocks >= 24 else [blocks - 1]
+    is_key = lambda i: keyframe_interval <= 1 or i % keyframe_interval == 0
 
     @torch.no_grad()
-    def frame_x(image):
-        x = torch.cat([special, patch_embed(image).flatten(2).transpose(1, 2)], dim=1)   # [B, 1004, 1024]
-        for blk in encoder_blocks:
-            x = blk(x)
-        for b in range(blocks):
-            x = frame_blocks[b](x, pos=pos2d)
-            x = global_blocks[b](x, pos=freqs, enable_3d_rope=True, kv_cache=m, global_idx=b)
-        return x
-
-    def frame(i: int):
-        return frame_x(xs[i % len(xs)])
+    def frame(i: int, keyframe: bool = True):
+        set_skip_append(model.kv_cache_manager, not keyframe) if model.kv_cache_manager is not None else None
+        return model(xs[i % len(xs)], selected_idx=selected)[0][-1]
 
     for i in range(ANCHOR + max(windows) + warmup):
         frame(i)
+    assert model.kv_cache_manager.tokens_per_frame == T
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for i in range(steps):
-        out = frame(i)
+        out = frame(i, is_key(i))
     torch.cuda.synchronize()
     dt = (time.perf_counter() - t0) / steps
-    assert torch.isfinite(out.float()).all() and m.device_header()["error"] == 0
-    # the same frame captured once and replayed as one HIP graph
-    from lingbot_map_amd import GraphedFrame
-    graphed = GraphedFrame(m, lambda x: frame_x(x), [xs[0]], cross_frame_special=False)
+    set_skip_append(model.kv_cache_manager, False)
+    assert torch.isfinite(out.float()).all()
+    model.kv_cache_manager.check_device_errors()
+    # the same frames replayed as HIP graphs (one for keyframes, one for read-only frames)
+    graphed = GraphedAggregator(model, xs[0], selected_idx=selected)
     for i in range(3):
-        graphed(xs[i % len(xs)])
+        graphed(xs[i % len(xs)], keyframe=is_key(i))
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for i in range(steps):
-        out = graphed(xs[i % len(xs)])
+        out = graphed(xs[i % len(xs)], keyframe=is_key(i))
     torch.cuda.synchronize()
     dt_graph = (time.perf_counter() - t0) / steps
-    assert torch.isfinite(out.float()).all() and m.device_header()["error"] == 0
+    assert torch.isfinite(out.float()).all()
+    model.kv_cache_manager.check_device_errors()
     kv = " / ".join(str((ANCHOR + w) * T) for w in windows)
     return {"value": B / dt, "unit": "frames/s", "ms_per_step": dt * 1e3, "steps": steps, "streams": B,
+            "keyframe_interval": keyframe_interval,
             "hip_graph": {"value": B / dt_graph, "unit": "frames/s", "ms_per_step": dt_graph * 1e3},
-            "what": f"patch embedding + 24 encoder blocks + {blocks} x (frame block + global block), dim {dim}, {H} heads, "
-                    f"MLP {4 * dim}, {B} stream(s), {T} tokens/frame, steady-state cache of {kv} KV tokens; "
-                    f"PyTorch-ROCm for linears / LayerNorm / GELU / convolution, HIP kernels for q/k norm + rotary + "
-                    f"append, the cache path and every block's cache-less attention; prediction heads excluded"}
+            "what": f"HipAggregatorStream: patch convolution + 24 encoder blocks + {blocks} x (frame block + global block), "
+                    f"dim {H * D}, {H} heads, MLP {4 * H * D}, {B} stream(s), {T} tokens/frame, steady-state cache of {kv} "
+                    f"KV tokens; PyTorch-ROCm for linears / LayerNorm / GELU / convolution, HIP kernels for q/k norm + "
+                    f"rotary + append, the cache path and every block's cache-less attention; prediction heads excluded"}
 
 
 def main() -> None:
@@ -614,6 +597,9 @@ def main() -> None:
         torch.cuda.empty_cache()
         # config 5: four independent streams with windows 4 / 8 / 16 / 16 as one ragged batch
         line["aggregator_step_4_streams"] = aggregator_step(torch, blocks, 10, 2, windows=(4, 8, 16, 16))
+        torch.cuda.empty_cache()
+        # config 4: keyframe interval 4 - three of four frames only read the cache
+        line["aggregator_step_keyframe_interval_4"] = aggregator_step(torch, blocks, 20, 3, keyframe_interval=4)
     if not args.no_cpu_baseline:
         line["cpu_baseline"] = cpu_baseline(torch, kv_tokens, blocks)
     print(json.dumps(line))

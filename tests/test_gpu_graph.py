@@ -46,8 +46,9 @@ def test_graph_replay_equals_eager():
     for i in range(fill + 2):
         f_e(xs[i % 6]); f_g(xs[i % 6])
     assert graphed.steady_state(cross_frame_special=False)
-    g = GraphedFrame(graphed, f_g, [xs[0]], cross_frame_special=False)   # runs one eager frame with xs[0] itself
-    f_e(xs[0])
+    before = graphed._tables.clone()
+    g = GraphedFrame(graphed, f_g, [xs[0]], cross_frame_special=False)   # warm-up and capture leave the cache alone
+    assert torch.equal(graphed._tables[..., :11], before[..., :11])
     assert graphed.frame_count == eager.frame_count
     for i in range(8):
         x = xs[(3 * i + 1) % 6]
@@ -122,23 +123,93 @@ def test_graph_replay_with_growing_trajectory_memory():
         f_e(xs[i % 6]); f_g(xs[i % 6])
     assert graphed.steady_state(cross_frame_special=True)
     g = GraphedFrame(graphed, f_g, [xs[0]], cross_frame_special=True)
-    f_e(xs[0])
-    tokens0 = graphed.device_header()["plan_kv_tokens"]
+    tokens0 = eager.device_header()["plan_kv_tokens"]      # the last keyframe's plan
     for i in range(8):
         x = xs[(3 * i + 1) % 6]
         want = f_e(x)
         got = g(x)
         torch.cuda.synchronize()
+        # block outputs of magnitude up to several units: two bf16 steps at the top of the range
         err = (got.float() - want.float()).abs()
-        assert err.max().item() <= 3e-2 and err.mean().item() <= 2e-3, f"replay {i}"
+        assert err.max().item() <= 2 ** -6 * want.float().abs().max().item() and err.mean().item() <= 2e-3, f"replay {i}"
         _ = (torch.randn(256, 256, device=x.device) @ torch.randn(256, 256, device=x.device)).sum().item()
     assert graphed.device_header()["plan_kv_tokens"] == tokens0 + 8 * 5       # five memory tokens per evicted frame
     assert graphed.frame_count == eager.frame_count
     assert graphed.get_cache_stats(0) == eager.get_cache_stats(0)
     assert graphed.build_visible_page_table(0) == eager.build_visible_page_table(0)
     assert graphed.build_visible_page_lens(0) == eager.build_visible_page_lens(0)
-    for a, b in zip(graphed.kv_caches, eager.kv_caches):
-        assert ((a.float() - b.float()).abs() / b.float().abs().clamp_min(1.0)).max().item() <= 2 ** -6
+    for a, b in zip(graphed.kv_caches, eager.kv_caches):   # K/V of the later blocks inherit those last-bit differences
+        assert ((a.float() - b.float()).abs() / b.float().abs().clamp_min(1.0)).max().item() <= 2 ** -5
     assert graphed.device_header()["error"] == 0
-    err = (f_g(xs[2]).float() - f_e(xs[2]).float()).abs()   # the eager path carries on from the replayed state
-    assert err.max().item() <= 3e-2
+    want = f_e(xs[2]).float()
+    err = (f_g(xs[2]).float() - want).abs()   # the eager path carries on from the replayed state
+    assert err.max().item() <= 2 ** -6 * want.abs().max().item()
+
+
+def test_keyframe_interval_stream_replayed_as_two_graphs():
+    """Keyframe interval 4 in the steady state (K, N, N, N, K, ...): the keyframe graph and the
+    read-only graph replayed in that pattern against the eager path - outputs bit for bit, and
+    tables, counts and pools identical afterwards; a read-only replay changes no table word."""
+    from lingbot_map_amd import GraphedStream, set_skip_append
+    mk, frame_on, xs, fill = _setup(cross_frame_special=False)
+    eager, graphed = mk(), mk()
+    f_e, f_g = frame_on(eager), frame_on(graphed)
+    for i in range(fill + 2):
+        f_e(xs[i % 6]); f_g(xs[i % 6])
+    stream = GraphedStream(graphed, f_g, [xs[0]], cross_frame_special=False)
+    assert graphed.frame_count == eager.frame_count and not graphed._skip_append
+    for i in range(13):
+        keyframe = i % 4 == 0
+        x = xs[(5 * i + 2) % 6]
+        set_skip_append(eager, not keyframe)
+        want = f_e(x)
+        tables_before = graphed._tables.clone()
+        got = stream(x, keyframe=keyframe)
+        torch.cuda.synchronize()
+        assert torch.equal(got, want), f"frame {i} keyframe={keyframe}"
+        if not keyframe:
+            assert torch.equal(graphed._tables[..., :11], tables_before[..., :11])
+        _ = (torch.randn(128, 128, device=x.device) @ torch.randn(128, 128, device=x.device)).sum().item()
+    set_skip_append(eager, False)
+    assert graphed.frame_count == eager.frame_count
+    assert graphed.build_visible_page_table(0) == eager.build_visible_page_table(0)
+    assert graphed.get_cache_stats(0) == eager.get_cache_stats(0)
+    for a, b in zip(graphed.kv_caches, eager.kv_caches):
+        assert torch.equal(a, b)
+    graphed.check_device_errors()
+    assert torch.equal(f_g(xs[1]), f_e(xs[1]))      # the eager path carries on from the replayed state
+
+
+def test_graphed_aggregator_equals_eager_aggregator():
+    """The whole aggregator shell (image in, group outputs out) replayed as graphs against the
+    same weights run eagerly, two ragged streams, the 3-D rotary table fed per frame."""
+    from lingbot_map_amd import GraphedAggregator, HipAggregatorStream, set_skip_append
+    dev = torch.device("cuda:0")
+    torch.manual_seed(9)
+    kw = dict(img_size=56, patch_size=14, embed_dim=128, depth=2, num_heads=2, init_values=0.5, patch_embed="conv",
+              enable_3d_rope=True, max_frame_num=64, kv_cache_sliding_window=[2, 3], kv_cache_scale_frames=1,
+              kv_cache_cross_frame_special=False, use_scale_token=False, page_size=4, layout="frame_pages", num_streams=2)
+    a = HipAggregatorStream(**kw).to(dev, torch.bfloat16).eval()
+    b = HipAggregatorStream(**kw).to(dev, torch.bfloat16).eval()
+    b.load_state_dict(a.state_dict())
+    g = torch.Generator(device=dev).manual_seed(10)
+    imgs = [torch.rand(2, 1, 3, 42, 56, generator=g, device=dev).to(torch.bfloat16) for _ in range(5)]
+    with torch.no_grad():
+        for i in range(6):                       # anchor and both windows full
+            a(imgs[i % 5]); b(imgs[i % 5])
+        graphed = GraphedAggregator(b, imgs[0], selected_idx=[1])
+        assert b.total_frames_processed == a.total_frames_processed == 6
+        for i in range(9):
+            keyframe = i % 3 != 1
+            set_skip_append(a.kv_cache_manager, not keyframe)
+            want = a(imgs[(2 * i + 1) % 5], selected_idx=[1])[0][0]
+            got = graphed(imgs[(2 * i + 1) % 5], keyframe=keyframe)[0]
+            torch.cuda.synchronize()
+            assert torch.equal(got, want), (i, keyframe)
+    assert a.total_frames_processed == b.total_frames_processed == 12
+    ma, mb = a.kv_cache_manager, b.kv_cache_manager
+    for s in range(2):
+        assert ma.build_visible_page_table(0, stream=s) == mb.build_visible_page_table(0, stream=s)
+    for x, y in zip(ma.kv_caches, mb.kv_caches):
+        assert torch.equal(x, y)
+    mb.check_device_errors()
