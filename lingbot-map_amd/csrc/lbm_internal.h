@@ -43,6 +43,7 @@ struct LbmAttnStreamPlan {
 struct LbmAttnSchedule {
   int32_t n_streams;
   int32_t total_wgs;
+  int32_t small;       // every stream's KV is short: the in-workgroup split kernel, no partial results
   int64_t part_rows;   // rows of partial results over all streams (0 when nothing is split)
   LbmAttnStreamPlan s[LBM_MAX_STREAMS];
 };

@@ -673,6 +673,308 @@ __global__ __launch_bounds__(kThreads, 1) void lbm_attn_bf16_d64_kernel(AttnArgs
   }
 }
 
+// ---------------------------------------------------------------------------- bf16, short KV
+// Streams with at most kSmMaxKv KV tokens - the frame blocks' attention of a frame over itself
+// (lingbot_map/layers/block.py:27-101: 1004 x 1004 tokens), the first frames of a stream - have
+// too few KV tiles to amortise the split-KV machinery above (a workgroup per (512 rows, head,
+// split) with a prologue of several tile-times, partial results through HBM and a second
+// kernel).  Here one 4-wave workgroup owns 64 query rows of one head and the KV axis is split
+// INSIDE it: wavefront w walks its own quarter of the KV tiles with its own K/V patch in LDS
+// (rows loaded as whole 128-byte lines, eight lanes per row, one tile ahead in registers), and
+// the four partial results are summed through LDS at the end.  No workspace, no second kernel.
+// Same arithmetic as the main kernel's first pass: scores straight into exp2 without a
+// reference, a range check at the end, and - only if that fails - a second pass with the
+// textbook running-maximum recurrence.
+namespace {
+constexpr int kSmWaves = 4;
+constexpr int kSmThreads = kSmWaves * 64;
+constexpr int kSmMaxKv = 4096;
+constexpr int kSmOStride = 68;   // floats per row of a partial output parked in LDS (4-bank shift per row)
+constexpr int kSmPatchBytes = kKvTile * (kKStride + kVStride) * 2;   // one wave's K and V tile
+static_assert(kSmWaves * kSmPatchBytes >= kSmWaves * (kQPerWave * kSmOStride + 2 * kQPerWave) * 4,
+              "the merge area reuses the tile patches");
+}  // namespace
+
+__global__ __launch_bounds__(kSmThreads, 1) void lbm_attn_bf16_d64_small_kernel(AttnArgs a) {
+  __shared__ __attribute__((aligned(16))) unsigned char lds_raw[kSmWaves * kSmPatchBytes];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int n32 = lane & 31, g = lane >> 5;
+  unsigned short* patch_k = (unsigned short*)(lds_raw + wave * kSmPatchBytes);
+  unsigned short* patch_v = patch_k + kKvTile * kKStride;
+
+  // ---- which (stream, 64 query rows, head)
+  int b = 0;
+  for (int i = 1; i < a.sch.n_streams; ++i)
+    if ((int)blockIdx.x >= a.sch.s[i].wg_begin) b = i;
+  const LbmAttnStreamPlan sp = a.sch.s[b];
+  const int H = a.num_heads;
+  const int local = (int)blockIdx.x - sp.wg_begin;
+  int qb64, head;
+  if ((H & 7) == 0) {   // the query blocks of one head on one XCD (blockIdx mod 8): its L2 serves their K/V
+    const int x = local & 7, i = local >> 3;
+    head = (i % (H >> 3)) * 8 + x;
+    qb64 = i / (H >> 3);
+  } else {
+    head = local % H;
+    qb64 = local / H;
+  }
+  if (qb64 >= sp.n_qtiles) return;   // padding between streams (whole workgroups)
+  const int kv_tokens = max(a.live_kv_tokens ? a.live_kv_tokens[sp.live_at] : sp.kv_tokens, 0);
+  const int n_tiles = (kv_tokens + kKvTile - 1) / kKvTile;
+  const int tps = (n_tiles + kSmWaves - 1) / kSmWaves;
+  const int t0 = wave * tps, t1 = min(t0 + tps, n_tiles);   // this wavefront's tiles (possibly none)
+  const unsigned row_bytes = (unsigned)H * 128u;
+  const int q_row0 = qb64 * kQPerWave;
+
+  // ---- Q: whole rows -> own patch -> fragments, scale * log2(e) folded in (as in the main kernel)
+  bf16x8 qf[2][4];
+  {
+    u32x4 raw[kQPerWave / 8];
+#pragma unroll
+    for (int k = 0; k < kQPerWave / 8; ++k) {
+      const int r = q_row0 + k * 8 + (lane >> 3);
+      raw[k] = u32x4{0u, 0u, 0u, 0u};
+      if (r < sp.q_rows) raw[k] = *(const u32x4*)(a.q + ((size_t)(sp.q_begin + r) * H + head) * 64 + (lane & 7) * 8);
+    }
+#pragma unroll
+    for (int k = 0; k < kQPerWave / 8; ++k)
+      *(u32x4*)&patch_k[(k * 8 + (lane >> 3)) * kKStride + (lane & 7) * 8] = raw[k];
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+#pragma unroll
+    for (int qb = 0; qb < 2; ++qb)
+#pragma unroll
+      for (int ks = 0; ks < 4; ++ks) {
+        const bf16x8 rawf = __builtin_bit_cast(bf16x8, *(const u32x4*)&patch_k[(qb * 32 + n32) * kKStride + ks * 16 + g * 8]);
+        f32x8 f = __builtin_convertvector(rawf, f32x8);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) f[j] *= a.scale_log2;
+        qf[qb][ks] = __builtin_convertvector(f, bf16x8);
+      }
+  }
+
+  // ---- K/V rows of a tile: lane l takes the 16-byte piece (l & 7) of rows (l >> 3) + 8 j
+  const char* pool_k = (const char*)(a.pool + (size_t)head * 64 + (lane & 7) * 8);
+  const char* pool_v = pool_k + (size_t)a.page_size * row_bytes;
+  const char* own_k = (const char*)(a.self_k + (size_t)head * 64 + (lane & 7) * 8);
+  const char* own_v = (const char*)(a.self_v + (size_t)head * 64 + (lane & 7) * 8);
+  const int32_t* rows = a.kv_rows + sp.kv_row_begin;
+  const int last_token = max(kv_tokens - 1, 0);
+  auto fetch = [&](int e, const char* pool_base, const char* own_base) -> u32x4 {
+    const char* base = e < 0 ? own_base : pool_base;
+    const unsigned r = (unsigned)(e ^ (e >> 31));
+    return *(const u32x4*)(base + (unsigned long long)r * row_bytes);
+  };
+  // rows past the last token re-read the last token: finite data, masked below
+  auto load_tile = [&](int t, u32x4 (&kk)[8], u32x4 (&vv)[8]) {
+    const int mine = rows[min(t * kKvTile + lane, last_token)];   // lane l: the entry of the tile's row l
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const int e = __builtin_amdgcn_ds_bpermute(4 * (j * 8 + (lane >> 3)), mine);
+      kk[j] = fetch(e, pool_k, own_k);
+      vv[j] = fetch(e, pool_v, own_v);
+    }
+  };
+  auto store_tile = [&](const u32x4 (&kk)[8], const u32x4 (&vv)[8]) {
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      *(u32x4*)&patch_k[(j * 8 + (lane >> 3)) * kKStride + (lane & 7) * 8] = kk[j];
+      *(u32x4*)&patch_v[(j * 8 + (lane >> 3)) * kVStride + (lane & 7) * 8] = vv[j];
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+  };
+  auto v_frag = [&](int ks, int db) -> bf16x8 {   // as in the main kernel, on this wave's patch
+    const int row = ks * 16 + 4 * g + ((lane & 15) >> 2);
+    const int col = db * 32 + ((lane >> 4) & 1) * 16 + (lane & 3) * 4;
+    const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+        (s16x4 __attribute__((address_space(3)))*)&patch_v[row * kVStride + col]);
+    const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+        (s16x4 __attribute__((address_space(3)))*)&patch_v[(row + 8) * kVStride + col]);
+    s16x8 both;
+    both[0] = lo[0]; both[1] = lo[1]; both[2] = lo[2]; both[3] = lo[3];
+    both[4] = hi[0]; both[5] = hi[1]; both[6] = hi[2]; both[7] = hi[3];
+    return __builtin_bit_cast(bf16x8, both);
+  };
+
+  f32x16 o[2][2];
+  f32x4 lacc[2];                 // first pass: row sums on the matrix pipe (layout as in the main kernel)
+  float m_run[2], l_lane[2];     // second pass: running maximum of the row, this lane's share of its sum
+  const unsigned sel_word = (lane == 0 || lane == 32 || lane == 17 || lane == 49) ? 0x3F803F80u : 0u;
+  const bf16x8 lsel = __builtin_bit_cast(bf16x8, u32x4{sel_word, sel_word, sel_word, sel_word});
+  f32x16 zero16;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) zero16[i] = 0.f;
+
+  bool safe = false;
+  for (int pass = 0; pass < 2; ++pass) {
+#pragma unroll
+    for (int qb = 0; qb < 2; ++qb) {
+#pragma unroll
+      for (int db = 0; db < 2; ++db) o[qb][db] = zero16;
+      lacc[qb] = f32x4{0.f, 0.f, 0.f, 0.f};
+      m_run[qb] = safe ? -INFINITY : 0.f;
+      l_lane[qb] = 0.f;
+    }
+    u32x4 kk[8], vv[8];
+    if (t0 < t1) load_tile(t0, kk, vv);
+    for (int t = t0; t < t1; ++t) {
+      store_tile(kk, vv);
+      if (t + 1 < t1) load_tile(t + 1, kk, vv);   // in flight while this tile is computed
+      const int n_valid = kv_tokens - t * kKvTile;
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        // S^T = K Q^T for the 32 kv rows of this half: s[qb][i] is kv = 32 h + 8 (i / 4) + 4 g + i % 4, q = 32 qb + n32
+        f32x16 sc[2] = {zero16, zero16};
+#pragma unroll
+        for (int ks = 0; ks < 4; ++ks) {
+          const bf16x8 ka = __builtin_bit_cast(bf16x8, *(const u32x4*)&patch_k[(h * 32 + n32) * kKStride + ks * 16 + g * 8]);
+#pragma unroll
+          for (int qb = 0; qb < 2; ++qb) sc[qb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka, qf[qb][ks], sc[qb], 0, 0, 0);
+        }
+        if (n_valid < kKvTile) {   // the ragged last tile of the stream
+#pragma unroll
+          for (int qb = 0; qb < 2; ++qb)
+#pragma unroll
+            for (int i = 0; i < 16; ++i)
+              if (h * 32 + 8 * (i >> 2) + 4 * g + (i & 3) >= n_valid) sc[qb][i] = -INFINITY;
+        }
+        bf16x8 p[2][2];
+#pragma unroll
+        for (int qb = 0; qb < 2; ++qb) {
+          if (safe) {
+            float mx = max3(sc[qb][0], sc[qb][1], sc[qb][2]);
+#pragma unroll
+            for (int i = 3; i < 15; i += 2) mx = max3(mx, sc[qb][i], sc[qb][i + 1]);
+            mx = swap_max(max2(mx, sc[qb][15]));
+            const float m_new = max2(m_run[qb], mx);     // finite: the first row of a tile is a token
+            const float alpha = __builtin_amdgcn_exp2f(m_run[qb] - m_new);   // 0 on the first tile
+            m_run[qb] = m_new;
+            l_lane[qb] *= alpha;
+#pragma unroll
+            for (int db = 0; db < 2; ++db)
+#pragma unroll
+              for (int i = 0; i < 16; ++i) o[qb][db][i] *= alpha;
+#pragma unroll
+            for (int i = 0; i < 16; ++i) sc[qb][i] -= m_new;
+          }
+#pragma unroll
+          for (int kk2 = 0; kk2 < 2; ++kk2) {
+            f32x8 e;
+#pragma unroll
+            for (int j = 0; j < 8; ++j) e[j] = __builtin_amdgcn_exp2f(sc[qb][kk2 * 8 + j]);
+            p[qb][kk2] = __builtin_convertvector(e, bf16x8);
+            if (safe) {
+#pragma unroll
+              for (int j = 0; j < 8; ++j) l_lane[qb] += e[j];
+            } else {
+              lacc[qb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(lsel, p[qb][kk2], lacc[qb], 0, 0, 0);
+            }
+          }
+        }
+        // O^T += V^T P^T over the half's two 16-row k-steps
+#pragma unroll
+        for (int kk2 = 0; kk2 < 2; ++kk2) {
+          const bf16x8 va[2] = {v_frag(h * 2 + kk2, 0), v_frag(h * 2 + kk2, 1)};
+#pragma unroll
+          for (int db = 0; db < 2; ++db)
+#pragma unroll
+            for (int qb = 0; qb < 2; ++qb)
+              o[qb][db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va[db], p[qb][kk2], o[qb][db], 0, 0, 0);
+        }
+      }
+    }
+    if (safe) break;
+    // range check of the pass without reference (integer compares, see the main kernel)
+    bool bad = false;
+    if (t0 < t1) {
+      unsigned top = 0u;
+#pragma unroll
+      for (int qb = 0; qb < 2; ++qb)
+#pragma unroll
+        for (int db = 0; db < 2; ++db)
+#pragma unroll
+          for (int i = 0; i < 16; ++i) top = max(top, __builtin_bit_cast(unsigned, o[qb][db][i]) & 0x7FFFFFFFu);
+      bad = top >= 0x7F800000u;
+      if (lane < 16) {
+#pragma unroll
+        for (int qb = 0; qb < 2; ++qb)
+#pragma unroll
+          for (int h2 = 0; h2 < 2; ++h2) {
+            const unsigned lb = __builtin_bit_cast(unsigned, lacc[qb][h2]);
+            bad = bad || lb < 0x12800000u /* 2^-90 */ || lb > 0x71800000u /* 2^100 */;
+          }
+      }
+    }
+    if (!__syncthreads_or(bad)) break;
+    safe = true;
+  }
+
+  // ---- merge the four wavefronts' partial results through LDS (the patches are dead)
+  __syncthreads();
+  float* so = (float*)lds_raw + wave * (kQPerWave * kSmOStride);
+  float* sl = (float*)lds_raw + kSmWaves * (kQPerWave * kSmOStride);   // [wave][64] row sums, then [wave][64] references
+  float* sm = sl + kSmWaves * kQPerWave;
+#pragma unroll
+  for (int qb = 0; qb < 2; ++qb) {
+#pragma unroll
+    for (int db = 0; db < 2; ++db)
+#pragma unroll
+      for (int c4 = 0; c4 < 4; ++c4)
+        *(f32x4*)&so[(qb * 32 + n32) * kSmOStride + db * 32 + c4 * 8 + g * 4] =
+            f32x4{o[qb][db][c4 * 4], o[qb][db][c4 * 4 + 1], o[qb][db][c4 * 4 + 2], o[qb][db][c4 * 4 + 3]};
+    if (safe) {
+      float lo, hi;
+      swap_halves(l_lane[qb], lo, hi);
+      if (g == 0) sl[wave * kQPerWave + qb * 32 + n32] = lo + hi;
+    } else if (lane < 16) {
+      sl[wave * kQPerWave + qb * 32 + lane] = lacc[qb][0];
+      sl[wave * kQPerWave + qb * 32 + 16 + lane] = lacc[qb][1];
+    }
+    if (g == 0) sm[wave * kQPerWave + qb * 32 + n32] = (t0 < t1) ? m_run[qb] : -INFINITY;
+  }
+  __syncthreads();
+  {
+    // wavefront w finishes rows 16 w .. 16 w + 15: four lanes per row, 16 head dims each
+    const int row = wave * 16 + (lane >> 2), d0 = (lane & 3) * 16;
+    float mw[kSmWaves], mx = -INFINITY;
+#pragma unroll
+    for (int w = 0; w < kSmWaves; ++w) {
+      mw[w] = sm[w * kQPerWave + row];
+      mx = max2(mx, mw[w]);
+    }
+    float acc[16], l_tot = 0.f;
+#pragma unroll
+    for (int j = 0; j < 16; ++j) acc[j] = 0.f;
+#pragma unroll
+    for (int w = 0; w < kSmWaves; ++w) {
+      // a wavefront without tiles (reference -inf) weighs nothing; with a common reference the weights are 1
+      const float wgt = mw[w] > -INFINITY ? __builtin_amdgcn_exp2f(mw[w] - mx) : 0.f;
+      l_tot += wgt * sl[w * kQPerWave + row];
+      const float* src = (const float*)lds_raw + w * (kQPerWave * kSmOStride) + row * kSmOStride + d0;
+#pragma unroll
+      for (int j4 = 0; j4 < 4; ++j4) {
+        const f32x4 x = *(const f32x4*)(src + 4 * j4);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) acc[4 * j4 + e] += wgt * x[e];
+      }
+    }
+    const float inv = l_tot > 0.f ? 1.0f / l_tot : 0.f;   // nothing visible: zeros (flashinfer_cache.py:368-370)
+    const int r = q_row0 + row;
+    if (r < sp.q_rows) {
+      f32x8 lo8, hi8;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        lo8[j] = acc[j] * inv;
+        hi8[j] = acc[8 + j] * inv;
+      }
+      unsigned short* dst = a.out + ((size_t)(sp.q_begin + r) * H + head) * 64 + d0;
+      *(bf16x8*)dst = __builtin_convertvector(lo8, bf16x8);
+      *(bf16x8*)(dst + 8) = __builtin_convertvector(hi8, bf16x8);
+    }
+  }
+}
+
 // Merge split-KV partial results: out = sum_s w_s * o_s with w_s = 2^(lse_s - max) / sum.
 // One thread per (query row, head, 8 consecutive d).
 __global__ __launch_bounds__(256) void lbm_attn_combine_bf16_kernel(AttnArgs a) {
@@ -1259,6 +1561,34 @@ void lbm_attn_schedule(const lbm_attn_stream* streams, int n_streams, int num_he
     work += (long long)qt[i] * num_heads * nt[i];
     if (nt[i] > max_nt) max_nt = nt[i];
   }
+  // short KV everywhere: the in-workgroup split kernel, one workgroup per (64 query rows, head),
+  // no partial results
+  bool small = n_streams > 0;
+  for (int i = 0; i < n_streams; ++i) small = small && streams[i].kv_tokens <= kSmMaxKv;
+  if (small) {
+    sch.small = 1;
+    int wg = 0;
+    for (int i = 0; i < n_streams; ++i) {
+      LbmAttnStreamPlan& p = sch.s[i];
+      p.q_begin = streams[i].q_begin;
+      p.q_rows = streams[i].q_rows;
+      p.kv_row_begin = streams[i].kv_row_begin;
+      p.kv_tokens = streams[i].kv_tokens;
+      p.live_at = streams[i].live_at;
+      p.n_qtiles = (streams[i].q_rows + kQPerWave - 1) / kQPerWave;
+      p.n_splits = 1;
+      p.tiles_per_split = nt[i] > 0 ? nt[i] : 1;
+      wg = (wg + 7) & ~7;   // each stream starts on XCD 0 so the in-kernel head -> XCD map lines up
+      p.wg_begin = wg;
+      p.part_begin = 0;
+      // whole groups of 8 workgroups when the heads are dealt over the XCDs
+      const int per_q = num_heads;
+      wg += p.n_qtiles * per_q;
+    }
+    sch.total_wgs = wg;
+    sch.part_rows = 0;
+    return;
+  }
   ScheduleKey& memo = g_last_schedule;
   bool hit = memo.n_streams == n_streams && memo.num_heads == num_heads;
   for (int i = 0; hit && i < n_streams; ++i) hit = memo.q_rows[i] == q_rows[i] && memo.n_tiles[i] == nt[i];
@@ -1404,6 +1734,10 @@ int lbm_launch_attention(const void* q, const void* pool, void* out, const void*
   a.scale_log2 = sm_scale * 1.4426950408889634f;
   a.sch = sch;
   if (sch.total_wgs == 0) return LBM_OK;
+  if (sch.small) {
+    hipLaunchKernelGGL(lbm_attn_bf16_d64_small_kernel, dim3(sch.total_wgs), dim3(kSmThreads), 0, stream, a);
+    return lbm_check_launch("lbm_attn_bf16_d64_small_kernel");
+  }
   hipLaunchKernelGGL(lbm_attn_bf16_d64_kernel, dim3(sch.total_wgs), dim3(kThreads), 0, stream, a);
   int rc = lbm_check_launch("lbm_attn_bf16_d64_kernel");
   if (rc != LBM_OK) return rc;
