@@ -678,29 +678,33 @@ __global__ __launch_bounds__(kThreads, 1) void lbm_attn_bf16_d64_kernel(AttnArgs
 // (lingbot_map/layers/block.py:27-101: 1004 x 1004 tokens), the first frames of a stream - have
 // too few KV tiles to amortise the split-KV machinery above (a workgroup per (512 rows, head,
 // split) with a prologue of several tile-times, partial results through HBM and a second
-// kernel).  Here one 4-wave workgroup owns 64 query rows of one head and the KV axis is split
-// INSIDE it: wavefront w walks its own quarter of the KV tiles with its own K/V patch in LDS
-// (rows loaded as whole 128-byte lines, eight lanes per row, one tile ahead in registers), and
-// the four partial results are summed through LDS at the end.  No workspace, no second kernel.
-// Same arithmetic as the main kernel's first pass: scores straight into exp2 without a
-// reference, a range check at the end, and - only if that fails - a second pass with the
-// textbook running-maximum recurrence.
+// kernel).  Here one 8-wave workgroup owns 64 query rows of one head and the KV axis is split
+// INSIDE it: wavefront w walks its own eighth of the KV axis in 32-token pieces with its own
+// K/V patch in LDS (rows loaded as whole 128-byte lines, eight lanes per row, one piece ahead in
+// registers), two wavefronts per SIMD covering each other's waits, and the eight partial
+// results are summed through LDS at the end.  No workspace, no second kernel.  Same arithmetic
+// as the main kernel's first pass: scores straight into exp2 without a reference, a range
+// check at the end, and - only if that fails - a second pass with the textbook running-maximum
+// recurrence.
 namespace {
-constexpr int kSmWaves = 4;
+constexpr int kSmWaves = 8;
 constexpr int kSmThreads = kSmWaves * 64;
 constexpr int kSmMaxKv = 4096;
+constexpr int kSmPiece = 32;     // KV tokens per step of a wavefront
 constexpr int kSmOStride = 68;   // floats per row of a partial output parked in LDS (4-bank shift per row)
-constexpr int kSmPatchBytes = kKvTile * (kKStride + kVStride) * 2;   // one wave's K and V tile
-static_assert(kSmWaves * kSmPatchBytes >= kSmWaves * (kQPerWave * kSmOStride + 2 * kQPerWave) * 4,
-              "the merge area reuses the tile patches");
+constexpr int kSmPatchBytes = kSmPiece * (kKStride + kVStride) * 2;             // one wave's K and V piece
+constexpr int kSmMergeBytes = kSmWaves * (kQPerWave * kSmOStride + 2 * kQPerWave) * 4;
+constexpr int kSmQBytes = kQPerWave * kKStride * 2;                              // Q on its way to the fragments
+constexpr int kSmLdsBytes = kSmMergeBytes > kSmWaves * kSmPatchBytes ? kSmMergeBytes : kSmWaves * kSmPatchBytes;
+static_assert(kSmLdsBytes >= kSmQBytes && kSmLdsBytes <= 160 * 1024, "LDS budget of the short-KV kernel");
 }  // namespace
 
 __global__ __launch_bounds__(kSmThreads, 1) void lbm_attn_bf16_d64_small_kernel(AttnArgs a) {
-  __shared__ __attribute__((aligned(16))) unsigned char lds_raw[kSmWaves * kSmPatchBytes];
+  __shared__ __attribute__((aligned(16))) unsigned char lds_raw[kSmLdsBytes];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int n32 = lane & 31, g = lane >> 5;
   unsigned short* patch_k = (unsigned short*)(lds_raw + wave * kSmPatchBytes);
-  unsigned short* patch_v = patch_k + kKvTile * kKStride;
+  unsigned short* patch_v = patch_k + kSmPiece * kKStride;
 
   // ---- which (stream, 64 query rows, head)
   int b = 0;
@@ -720,40 +724,36 @@ __global__ __launch_bounds__(kSmThreads, 1) void lbm_attn_bf16_d64_small_kernel(
   }
   if (qb64 >= sp.n_qtiles) return;   // padding between streams (whole workgroups)
   const int kv_tokens = max(a.live_kv_tokens ? a.live_kv_tokens[sp.live_at] : sp.kv_tokens, 0);
-  const int n_tiles = (kv_tokens + kKvTile - 1) / kKvTile;
-  const int tps = (n_tiles + kSmWaves - 1) / kSmWaves;
-  const int t0 = wave * tps, t1 = min(t0 + tps, n_tiles);   // this wavefront's tiles (possibly none)
+  const int n_pieces = (kv_tokens + kSmPiece - 1) / kSmPiece;
+  const int pps = (n_pieces + kSmWaves - 1) / kSmWaves;
+  const int p0 = wave * pps, p1 = min(p0 + pps, n_pieces);   // this wavefront's pieces (possibly none)
   const unsigned row_bytes = (unsigned)H * 128u;
   const int q_row0 = qb64 * kQPerWave;
 
-  // ---- Q: whole rows -> own patch -> fragments, scale * log2(e) folded in (as in the main kernel)
+  // ---- Q: the workgroup reads the 64 rows once as whole rows, every wavefront picks its
+  // fragments up from LDS; scale * log2(e) folded in (as in the main kernel)
   bf16x8 qf[2][4];
   {
-    u32x4 raw[kQPerWave / 8];
-#pragma unroll
-    for (int k = 0; k < kQPerWave / 8; ++k) {
-      const int r = q_row0 + k * 8 + (lane >> 3);
-      raw[k] = u32x4{0u, 0u, 0u, 0u};
-      if (r < sp.q_rows) raw[k] = *(const u32x4*)(a.q + ((size_t)(sp.q_begin + r) * H + head) * 64 + (lane & 7) * 8);
-    }
-#pragma unroll
-    for (int k = 0; k < kQPerWave / 8; ++k)
-      *(u32x4*)&patch_k[(k * 8 + (lane >> 3)) * kKStride + (lane & 7) * 8] = raw[k];
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    __builtin_amdgcn_wave_barrier();
+    unsigned short* patch_q = (unsigned short*)lds_raw;
+    const int r = q_row0 + (tid >> 3);
+    u32x4 raw = {0u, 0u, 0u, 0u};
+    if (r < sp.q_rows) raw = *(const u32x4*)(a.q + ((size_t)(sp.q_begin + r) * H + head) * 64 + (tid & 7) * 8);
+    *(u32x4*)&patch_q[(tid >> 3) * kKStride + (tid & 7) * 8] = raw;
+    __syncthreads();
 #pragma unroll
     for (int qb = 0; qb < 2; ++qb)
 #pragma unroll
       for (int ks = 0; ks < 4; ++ks) {
-        const bf16x8 rawf = __builtin_bit_cast(bf16x8, *(const u32x4*)&patch_k[(qb * 32 + n32) * kKStride + ks * 16 + g * 8]);
+        const bf16x8 rawf = __builtin_bit_cast(bf16x8, *(const u32x4*)&patch_q[(qb * 32 + n32) * kKStride + ks * 16 + g * 8]);
         f32x8 f = __builtin_convertvector(rawf, f32x8);
 #pragma unroll
         for (int j = 0; j < 8; ++j) f[j] *= a.scale_log2;
         qf[qb][ks] = __builtin_convertvector(f, bf16x8);
       }
+    __syncthreads();   // the patches below overlay the Q rows
   }
 
-  // ---- K/V rows of a tile: lane l takes the 16-byte piece (l & 7) of rows (l >> 3) + 8 j
+  // ---- K/V rows of a piece: lane l takes the 16-byte part (l & 7) of rows (l >> 3) + 8 j
   const char* pool_k = (const char*)(a.pool + (size_t)head * 64 + (lane & 7) * 8);
   const char* pool_v = pool_k + (size_t)a.page_size * row_bytes;
   const char* own_k = (const char*)(a.self_k + (size_t)head * 64 + (lane & 7) * 8);
@@ -765,21 +765,22 @@ __global__ __launch_bounds__(kSmThreads, 1) void lbm_attn_bf16_d64_small_kernel(
     const unsigned r = (unsigned)(e ^ (e >> 31));
     return *(const u32x4*)(base + (unsigned long long)r * row_bytes);
   };
+  constexpr int kRowsPerPass = 8, kPasses = kSmPiece / kRowsPerPass;
   // rows past the last token re-read the last token: finite data, masked below
-  auto load_tile = [&](int t, u32x4 (&kk)[8], u32x4 (&vv)[8]) {
-    const int mine = rows[min(t * kKvTile + lane, last_token)];   // lane l: the entry of the tile's row l
+  auto load_piece = [&](int pc, u32x4 (&kk)[kPasses], u32x4 (&vv)[kPasses]) {
+    const int mine = rows[min(pc * kSmPiece + n32, last_token)];   // lanes l and l + 32: the entry of the piece's row l
 #pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      const int e = __builtin_amdgcn_ds_bpermute(4 * (j * 8 + (lane >> 3)), mine);
+    for (int j = 0; j < kPasses; ++j) {
+      const int e = __builtin_amdgcn_ds_bpermute(4 * (j * kRowsPerPass + (lane >> 3)), mine);
       kk[j] = fetch(e, pool_k, own_k);
       vv[j] = fetch(e, pool_v, own_v);
     }
   };
-  auto store_tile = [&](const u32x4 (&kk)[8], const u32x4 (&vv)[8]) {
+  auto store_piece = [&](const u32x4 (&kk)[kPasses], const u32x4 (&vv)[kPasses]) {
 #pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      *(u32x4*)&patch_k[(j * 8 + (lane >> 3)) * kKStride + (lane & 7) * 8] = kk[j];
-      *(u32x4*)&patch_v[(j * 8 + (lane >> 3)) * kVStride + (lane & 7) * 8] = vv[j];
+    for (int j = 0; j < kPasses; ++j) {
+      *(u32x4*)&patch_k[(j * kRowsPerPass + (lane >> 3)) * kKStride + (lane & 7) * 8] = kk[j];
+      *(u32x4*)&patch_v[(j * kRowsPerPass + (lane >> 3)) * kVStride + (lane & 7) * 8] = vv[j];
     }
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
@@ -816,78 +817,75 @@ __global__ __launch_bounds__(kSmThreads, 1) void lbm_attn_bf16_d64_small_kernel(
       m_run[qb] = safe ? -INFINITY : 0.f;
       l_lane[qb] = 0.f;
     }
-    u32x4 kk[8], vv[8];
-    if (t0 < t1) load_tile(t0, kk, vv);
-    for (int t = t0; t < t1; ++t) {
-      store_tile(kk, vv);
-      if (t + 1 < t1) load_tile(t + 1, kk, vv);   // in flight while this tile is computed
-      const int n_valid = kv_tokens - t * kKvTile;
+    u32x4 kk[kPasses], vv[kPasses];
+    if (p0 < p1) load_piece(p0, kk, vv);
+    for (int pc = p0; pc < p1; ++pc) {
+      store_piece(kk, vv);
+      if (pc + 1 < p1) load_piece(pc + 1, kk, vv);   // in flight while this piece is computed
+      const int n_valid = kv_tokens - pc * kSmPiece;
+      // S^T = K Q^T for the piece's 32 kv rows: sc[qb][i] is kv = 8 (i / 4) + 4 g + i % 4, q = 32 qb + n32
+      f32x16 sc[2] = {zero16, zero16};
 #pragma unroll
-      for (int h = 0; h < 2; ++h) {
-        // S^T = K Q^T for the 32 kv rows of this half: s[qb][i] is kv = 32 h + 8 (i / 4) + 4 g + i % 4, q = 32 qb + n32
-        f32x16 sc[2] = {zero16, zero16};
+      for (int ks = 0; ks < 4; ++ks) {
+        const bf16x8 ka = __builtin_bit_cast(bf16x8, *(const u32x4*)&patch_k[n32 * kKStride + ks * 16 + g * 8]);
 #pragma unroll
-        for (int ks = 0; ks < 4; ++ks) {
-          const bf16x8 ka = __builtin_bit_cast(bf16x8, *(const u32x4*)&patch_k[(h * 32 + n32) * kKStride + ks * 16 + g * 8]);
+        for (int qb = 0; qb < 2; ++qb) sc[qb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka, qf[qb][ks], sc[qb], 0, 0, 0);
+      }
+      const bf16x8 va0[2] = {v_frag(0, 0), v_frag(0, 1)};   // requested early: they arrive under the exp2 work
+      const bf16x8 va1[2] = {v_frag(1, 0), v_frag(1, 1)};
+      if (n_valid < kSmPiece) {   // the ragged last piece of the stream
 #pragma unroll
-          for (int qb = 0; qb < 2; ++qb) sc[qb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka, qf[qb][ks], sc[qb], 0, 0, 0);
-        }
-        if (n_valid < kKvTile) {   // the ragged last tile of the stream
+        for (int qb = 0; qb < 2; ++qb)
 #pragma unroll
-          for (int qb = 0; qb < 2; ++qb)
+          for (int i = 0; i < 16; ++i)
+            if (8 * (i >> 2) + 4 * g + (i & 3) >= n_valid) sc[qb][i] = -INFINITY;
+      }
+      bf16x8 p[2][2];
 #pragma unroll
-            for (int i = 0; i < 16; ++i)
-              if (h * 32 + 8 * (i >> 2) + 4 * g + (i & 3) >= n_valid) sc[qb][i] = -INFINITY;
-        }
-        bf16x8 p[2][2];
+      for (int qb = 0; qb < 2; ++qb) {
+        if (safe) {
+          float mx = max3(sc[qb][0], sc[qb][1], sc[qb][2]);
 #pragma unroll
-        for (int qb = 0; qb < 2; ++qb) {
-          if (safe) {
-            float mx = max3(sc[qb][0], sc[qb][1], sc[qb][2]);
-#pragma unroll
-            for (int i = 3; i < 15; i += 2) mx = max3(mx, sc[qb][i], sc[qb][i + 1]);
-            mx = swap_max(max2(mx, sc[qb][15]));
-            const float m_new = max2(m_run[qb], mx);     // finite: the first row of a tile is a token
-            const float alpha = __builtin_amdgcn_exp2f(m_run[qb] - m_new);   // 0 on the first tile
-            m_run[qb] = m_new;
-            l_lane[qb] *= alpha;
-#pragma unroll
-            for (int db = 0; db < 2; ++db)
-#pragma unroll
-              for (int i = 0; i < 16; ++i) o[qb][db][i] *= alpha;
-#pragma unroll
-            for (int i = 0; i < 16; ++i) sc[qb][i] -= m_new;
-          }
-#pragma unroll
-          for (int kk2 = 0; kk2 < 2; ++kk2) {
-            f32x8 e;
-#pragma unroll
-            for (int j = 0; j < 8; ++j) e[j] = __builtin_amdgcn_exp2f(sc[qb][kk2 * 8 + j]);
-            p[qb][kk2] = __builtin_convertvector(e, bf16x8);
-            if (safe) {
-#pragma unroll
-              for (int j = 0; j < 8; ++j) l_lane[qb] += e[j];
-            } else {
-              lacc[qb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(lsel, p[qb][kk2], lacc[qb], 0, 0, 0);
-            }
-          }
-        }
-        // O^T += V^T P^T over the half's two 16-row k-steps
-#pragma unroll
-        for (int kk2 = 0; kk2 < 2; ++kk2) {
-          const bf16x8 va[2] = {v_frag(h * 2 + kk2, 0), v_frag(h * 2 + kk2, 1)};
+          for (int i = 3; i < 15; i += 2) mx = max3(mx, sc[qb][i], sc[qb][i + 1]);
+          mx = swap_max(max2(mx, sc[qb][15]));
+          const float m_new = max2(m_run[qb], mx);     // finite: the first row of a piece is a token
+          const float alpha = __builtin_amdgcn_exp2f(m_run[qb] - m_new);   // 0 on the first piece
+          m_run[qb] = m_new;
+          l_lane[qb] *= alpha;
 #pragma unroll
           for (int db = 0; db < 2; ++db)
 #pragma unroll
-            for (int qb = 0; qb < 2; ++qb)
-              o[qb][db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va[db], p[qb][kk2], o[qb][db], 0, 0, 0);
+            for (int i = 0; i < 16; ++i) o[qb][db][i] *= alpha;
+#pragma unroll
+          for (int i = 0; i < 16; ++i) sc[qb][i] -= m_new;
+        }
+#pragma unroll
+        for (int kk2 = 0; kk2 < 2; ++kk2) {
+          f32x8 e;
+#pragma unroll
+          for (int j = 0; j < 8; ++j) e[j] = __builtin_amdgcn_exp2f(sc[qb][kk2 * 8 + j]);
+          p[qb][kk2] = __builtin_convertvector(e, bf16x8);
+          if (safe) {
+#pragma unroll
+            for (int j = 0; j < 8; ++j) l_lane[qb] += e[j];
+          } else {
+            lacc[qb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(lsel, p[qb][kk2], lacc[qb], 0, 0, 0);
+          }
         }
       }
+      // O^T += V^T P^T over the piece's two 16-row k-steps
+#pragma unroll
+      for (int db = 0; db < 2; ++db)
+#pragma unroll
+        for (int qb = 0; qb < 2; ++qb) {
+          o[qb][db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va0[db], p[qb][0], o[qb][db], 0, 0, 0);
+          o[qb][db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va1[db], p[qb][1], o[qb][db], 0, 0, 0);
+        }
     }
     if (safe) break;
     // range check of the pass without reference (integer compares, see the main kernel)
     bool bad = false;
-    if (t0 < t1) {
+    if (p0 < p1) {
       unsigned top = 0u;
 #pragma unroll
       for (int qb = 0; qb < 2; ++qb)
@@ -910,7 +908,7 @@ __global__ __launch_bounds__(kSmThreads, 1) void lbm_attn_bf16_d64_small_kernel(
     safe = true;
   }
 
-  // ---- merge the four wavefronts' partial results through LDS (the patches are dead)
+  // ---- merge the wavefronts' partial results through LDS (the patches are dead)
   __syncthreads();
   float* so = (float*)lds_raw + wave * (kQPerWave * kSmOStride);
   float* sl = (float*)lds_raw + kSmWaves * (kQPerWave * kSmOStride);   // [wave][64] row sums, then [wave][64] references
@@ -931,46 +929,41 @@ __global__ __launch_bounds__(kSmThreads, 1) void lbm_attn_bf16_d64_small_kernel(
       sl[wave * kQPerWave + qb * 32 + lane] = lacc[qb][0];
       sl[wave * kQPerWave + qb * 32 + 16 + lane] = lacc[qb][1];
     }
-    if (g == 0) sm[wave * kQPerWave + qb * 32 + n32] = (t0 < t1) ? m_run[qb] : -INFINITY;
+    if (g == 0) sm[wave * kQPerWave + qb * 32 + n32] = (p0 < p1) ? m_run[qb] : -INFINITY;
   }
   __syncthreads();
   {
-    // wavefront w finishes rows 16 w .. 16 w + 15: four lanes per row, 16 head dims each
-    const int row = wave * 16 + (lane >> 2), d0 = (lane & 3) * 16;
+    // wavefront w finishes rows 8 w .. 8 w + 7: eight lanes per row, 8 head dims (16 bytes) each
+    const int row = wave * (kQPerWave / kSmWaves) + (lane >> 3), d0 = (lane & 7) * 8;
     float mw[kSmWaves], mx = -INFINITY;
 #pragma unroll
     for (int w = 0; w < kSmWaves; ++w) {
       mw[w] = sm[w * kQPerWave + row];
       mx = max2(mx, mw[w]);
     }
-    float acc[16], l_tot = 0.f;
+    f32x8 acc;
 #pragma unroll
-    for (int j = 0; j < 16; ++j) acc[j] = 0.f;
+    for (int j = 0; j < 8; ++j) acc[j] = 0.f;
+    float l_tot = 0.f;
 #pragma unroll
     for (int w = 0; w < kSmWaves; ++w) {
-      // a wavefront without tiles (reference -inf) weighs nothing; with a common reference the weights are 1
+      // a wavefront without pieces (reference -inf) weighs nothing; with a common reference the weights are 1
       const float wgt = mw[w] > -INFINITY ? __builtin_amdgcn_exp2f(mw[w] - mx) : 0.f;
       l_tot += wgt * sl[w * kQPerWave + row];
       const float* src = (const float*)lds_raw + w * (kQPerWave * kSmOStride) + row * kSmOStride + d0;
+      const f32x4 x0 = *(const f32x4*)src, x1 = *(const f32x4*)(src + 4);
 #pragma unroll
-      for (int j4 = 0; j4 < 4; ++j4) {
-        const f32x4 x = *(const f32x4*)(src + 4 * j4);
-#pragma unroll
-        for (int e = 0; e < 4; ++e) acc[4 * j4 + e] += wgt * x[e];
+      for (int e = 0; e < 4; ++e) {
+        acc[e] += wgt * x0[e];
+        acc[4 + e] += wgt * x1[e];
       }
     }
     const float inv = l_tot > 0.f ? 1.0f / l_tot : 0.f;   // nothing visible: zeros (flashinfer_cache.py:368-370)
     const int r = q_row0 + row;
     if (r < sp.q_rows) {
-      f32x8 lo8, hi8;
 #pragma unroll
-      for (int j = 0; j < 8; ++j) {
-        lo8[j] = acc[j] * inv;
-        hi8[j] = acc[8 + j] * inv;
-      }
-      unsigned short* dst = a.out + ((size_t)(sp.q_begin + r) * H + head) * 64 + d0;
-      *(bf16x8*)dst = __builtin_convertvector(lo8, bf16x8);
-      *(bf16x8*)(dst + 8) = __builtin_convertvector(hi8, bf16x8);
+      for (int j = 0; j < 8; ++j) acc[j] *= inv;
+      *(bf16x8*)(a.out + ((size_t)(sp.q_begin + r) * H + head) * 64 + d0) = __builtin_convertvector(acc, bf16x8);
     }
   }
 }
