@@ -102,11 +102,11 @@ def attention_shapes(torch) -> list:
         out = torch.empty_like(q)
         own = q if tail else None
         vp = lambda t: None if t is None else C.c_void_p(t.data_ptr())
-        stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
 
-        def launch():
+        def launch():   # on whatever stream is current (the timing helpers launch on a stream of their own)
             N.check(N.lib.lbm_attn_run(vp(q), vp(pool), vp(out), vp(own), vp(own), vp(kv_rows), streams, ns, H, D, PAGE,
-                                       N.DTYPE_BF16, 1.0 / math.sqrt(D), vp(ws), ws.numel(), stream))
+                                       N.DTYPE_BF16, 1.0 / math.sqrt(D), vp(ws), ws.numel(),
+                                       C.c_void_p(torch.cuda.current_stream().cuda_stream)))
 
         for _ in range(100):
             launch()
