@@ -26,10 +26,13 @@ T, N_SPECIAL, H, D, PAGE = 1004, 5, 16, 64, 16
 ANCHOR, WINDOW = 1, 16
 PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA
 PEAK_HBM_GBPS = 8000.0
-# HBM bytes of one lbm_attn_bf16_d64_kernel launch at this workload, from rocprofv3 --pmc
-# FETCH_SIZE (x2.0, the factor a 256 MiB plain copy gives) and WRITE_SIZE (x1.0), in KiB:
-# 35,738 * 2 + 20,592 KiB  (profiles/attention_config2_hbm_traffic.md)
-ATTN_TRAFFIC_BYTES = (35738.0 * 2.0 + 20592.0) * 1024.0
+# HBM bytes of one lbm_attn_run at this workload - the main kernel AND the combine kernel that
+# merges its split-KV partial results - from rocprofv3 --pmc FETCH_SIZE (x2.0, the factor a
+# 256 MiB plain copy gives) and WRITE_SIZE (x1.0), in KiB per dispatch
+# (profiles/attention_config2_hbm_traffic.md): main ATTN_MAIN_KIB, combine ATTN_COMBINE_KIB
+ATTN_MAIN_KIB = (35738.0, 20592.0)       # (FETCH_SIZE, WRITE_SIZE) of lbm_attn_bf16_d64_kernel
+ATTN_COMBINE_KIB = (8315.3, 2008.0)      # of lbm_attn_combine_bf16_kernel
+ATTN_TRAFFIC_BYTES = ((ATTN_MAIN_KIB[0] + ATTN_COMBINE_KIB[0]) * 2.0 + ATTN_MAIN_KIB[1] + ATTN_COMBINE_KIB[1]) * 1024.0
 METRIC = "frames/sec streaming @518x378 (1 GPU); attention TFLOPS & % bf16 MFMA peak"
 
 
@@ -124,6 +127,41 @@ def attention_shapes(torch) -> list:
         run("config 5: four streams, 5,020 / 9,036 / 17,068 / 17,068", [5020, 9036, 17068, 17068]),
         run("frame block: 1,004 x 1,004, no cache", [1004], tail=True),
     ]
+
+
+def config3_stream(torch) -> dict:
+    """Configuration 3 as a stream: one global block's cache after 10,000 frames (1 anchor + 16 window frames and
+    9,983 evicted frames that kept their 5 special tokens in place: 66,983 visible tokens over 11,054 pages), then
+    streamed keyframe steps on it.  Reports the table step alone (allocate + evict + compact + the 268 KB row table
+    with its 9,983 memory frames) and a whole step of the block (table step + paged append + attention)."""
+    from lingbot_map_amd import HipPagedKVCacheManager
+    dev = torch.device("cuda:0")
+    frames = 10000
+    m = HipPagedKVCacheManager(1, ANCHOR + WINDOW + 16, T, H, D, torch.bfloat16, dev, num_special_tokens=N_SPECIAL,
+                               scale_frames=ANCHOR, sliding_window=WINDOW, max_total_frames=frames + 64, page_size=PAGE,
+                               layout="frame_pages")
+    g = torch.Generator(device=dev).manual_seed(2)
+    q, k, v = (torch.randn(T, H, D, generator=g, device=dev, dtype=torch.float32).to(torch.bfloat16) for _ in range(3))
+    for _ in range(frames):
+        m.append_frame(0, k, v)
+        m.evict_frames(0, ANCHOR, WINDOW)
+    kv = (ANCHOR + WINDOW) * T + N_SPECIAL * (frames - ANCHOR - WINDOW)
+    m._plan(0, [False])
+    assert m._plan_tokens[0][0] == kv == 66983
+    ops = m._ops([{"ops": 16, "expect_kv_tokens": kv}])
+    plan_ms = kernel_time_ms(lambda: m._tables_step(0, ops, kv_rows=True), 50, torch)
+    for _ in range(5):
+        m.step(0, q, k, v, keyframe=[True])
+    step_ms = event_time_ms(lambda: m.step(0, q, k, v, keyframe=[True]), 20, torch)
+    attn_ms = event_time_ms(lambda: m._attend_planned(0, q, None, None), 50, torch)
+    m.check_device_errors()
+    kv_now = m._plan_tokens[0][0]
+    flop = 4.0 * T * kv_now * H * D
+    return {"kv_tokens": kv_now, "memory_frames": frames + 25 - ANCHOR - WINDOW, "tables_plan_us": plan_ms * 1e3,
+            "block_step_us": step_ms * 1e3, "attention_us": attn_ms * 1e3,
+            "attention_tflops": flop / (attn_ms * 1e-3) * 1e-12,
+            "what": "one block: keyframe step = table step (allocate, evict, compact, row table) + paged append + attention "
+                    "over anchor + window + trajectory memory; tables_plan_us is the row-table plan alone"}
 
 
 def hbm_kernels_4_streams(torch) -> dict:
@@ -582,6 +620,8 @@ def main() -> None:
                    "blocks": blocks, "kv_tokens": kv_tokens, "q_tokens": T, "page_size": PAGE},
         "roofline": {"bound": "mfma", "achieved": attn_tflops, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                      "frac": attn_tflops / PEAK_BF16_TFLOPS, "traffic": ATTN_TRAFFIC_BYTES,
+                     "traffic_main_kernel": (ATTN_MAIN_KIB[0] * 2.0 + ATTN_MAIN_KIB[1]) * 1024.0,
+                     "algorithmic_bytes": 2.0 * kv_tokens * H * D * 2 + 2.0 * T * H * D * 2,
                      "kernel": "lbm_attn_bf16_d64_kernel + lbm_attn_combine_bf16_kernel (one lbm_attn_run)",
                      "flop_per_launch": flops, "avg_launch_us": attn_ms * 1e3},
         "attention_tflops": attn_tflops,
@@ -601,6 +641,7 @@ def main() -> None:
         "attention_shapes": attention_shapes(torch),
         "hbm_kernels_4_streams": hbm_kernels_4_streams(torch),
         "camera_head_cache": camera_head_cache(torch),
+        "config3_stream": config3_stream(torch),
     }
     if not args.no_aggregator:
         del m

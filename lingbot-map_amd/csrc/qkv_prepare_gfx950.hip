@@ -20,6 +20,11 @@
 #include <hip/hip_runtime.h>
 #include "lbm_internal.h"
 
+// Every product and sum below is rounded on its own, as the reference's separate torch ops are.
+// The math header's __fmul_rn / __fadd_rn are plain operators compiled with contraction allowed
+// (the compiler fuses them into FMAs), so the kernel uses its own, defined under this pragma.
+#pragma clang fp contract(off)
+
 typedef __attribute__((ext_vector_type(4))) unsigned int u32x4;
 typedef __attribute__((ext_vector_type(4))) float f32x4;
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
@@ -28,6 +33,9 @@ namespace {
 
 // round-to-nearest-even to bf16 and back (torch's .to(bfloat16)); the hardware conversion
 // v_cvt_pk_bf16_f32 rounds the same way
+__device__ __forceinline__ float mul_rn(float a, float b) { return a * b; }
+__device__ __forceinline__ float add_rn(float a, float b) { return a + b; }
+__device__ __forceinline__ float sub_rn(float a, float b) { return a - b; }
 __device__ __forceinline__ float round_bf16(float f) { return (float)(__bf16)f; }
 
 template <int DT>  // 0 = bf16, 1 = f32
@@ -65,11 +73,15 @@ __device__ __forceinline__ void store8(void* base, long long elem, const float (
 
 struct PrepareArgs {
   const void* qkv;
-  const float* norm_w[2];  // q, k
-  const float* norm_b[2];
+  const float* q_norm_w;   // all four NULL: no qk-norm
+  const float* q_norm_b;
+  const float* k_norm_w;
+  const float* k_norm_b;
   const float* rope_cs;
   int rope_layout;
-  void* out[3];            // q_out, k_out, v_out
+  void* q_out;
+  void* k_out;             // k_out / v_out may be NULL (keyframes: only the pool copy is wanted)
+  void* v_out;
   void* pool;
   const int32_t* append_rows;
   float eps;
@@ -77,91 +89,145 @@ struct PrepareArgs {
 };
 
 // head_dim 64.  SRC = activation dtype, DST = cache dtype.
-template <int SRC, int DST>
+//
+// The kernel is a chain of short memory latencies, not of bandwidth: 12 MB per frame move in
+// about a microsecond, a dependent load costs as much again, and launching a wave costs more
+// than the 16 bytes per lane it would move.  So a group of 8 lanes carries three rows, and every
+// load it needs - 3 x 16 bytes of qkv, the LayerNorm parameters, the rotary table entries, the
+// append row - sits in one straight line of code ahead of the arithmetic.
+// ROPE: 0 none, 1 interleaved pairs, 2 half-split pairs; NORM: qk-LayerNorm; APPEND: pool writes.
+// Compile-time so that the loads below sit in one straight line of code: the compiler waits
+// for every outstanding load at the end of a conditional block.
+template <int SRC, int DST, int ROPE, bool NORM, bool APPEND>
 __global__ __launch_bounds__(256) void lbm_qkv_prepare_d64_kernel(PrepareArgs a) {
   const int H = a.num_heads;
-  // 32 rows of (token, q|k|v, head) per workgroup; the host checks that the row count fits 32 bits
-  const unsigned rw = blockIdx.x * 32u + (threadIdx.x >> 3);
-  const unsigned rows = (unsigned)a.n_tokens * 3u * (unsigned)H;
+  // 16 or 32 (token, head) groups per workgroup, 8 lanes each; a group carries the q, k and v
+  // row of its head, so the rotary entries and the append row are loaded once for the three and
+  // a third as many waves are launched as with a group per row.  The host checks that the group
+  // count fits 32 bits.
+  const unsigned g = blockIdx.x * (blockDim.x >> 3) + (threadIdx.x >> 3);
+  const unsigned groups = (unsigned)a.n_tokens * (unsigned)H;
   // whole 8-lane groups leave together, so the shuffles below see all their lanes
-  if (rw >= rows) return;
+  if (g >= groups) return;
   const int c = (int)(threadIdx.x & 7);
-  const unsigned th = rw / (unsigned)H;       // token * 3 + which
-  const int h = (int)(rw - th * (unsigned)H);
-  const int t = (int)(th / 3u);
-  const int which = (int)(th - (unsigned)t * 3u);
+  const int t = (int)(g / (unsigned)H);
+  const int h = (int)(g - (unsigned)t * (unsigned)H);
+  constexpr bool has_norm = NORM, has_rope = ROPE != 0, interleaved = ROPE == 1;
 
-  float x[8];
-  load8<SRC>(a.qkv, (long long)rw * 64 + c * 8, x);
+  // ---- every load of this group, back to back
+  const long long in0 = ((long long)t * 3 * H + h) * 64 + c * 8;   // q row; k and v follow H rows apart
+  u32x4 raw16[3] = {};
+  f32x4 raw32[3][2] = {};
+#pragma unroll
+  for (int w = 0; w < 3; ++w) {
+    if (SRC == 0) {
+      raw16[w] = *(const u32x4*)((const unsigned short*)a.qkv + in0 + (long long)w * H * 64);
+    } else {
+      const f32x4* xp = (const f32x4*)((const float*)a.qkv + in0 + (long long)w * H * 64);
+      raw32[w][0] = xp[0];
+      raw32[w][1] = xp[1];
+    }
+  }
+  f32x4 w4[2][2] = {}, b4[2][2] = {};
+  if (has_norm) {
+    const f32x4* qw = (const f32x4*)(a.q_norm_w + c * 8);
+    const f32x4* qb = (const f32x4*)(a.q_norm_b + c * 8);
+    const f32x4* kw = (const f32x4*)(a.k_norm_w + c * 8);
+    const f32x4* kb = (const f32x4*)(a.k_norm_b + c * 8);
+    w4[0][0] = qw[0]; w4[0][1] = qw[1]; b4[0][0] = qb[0]; b4[0][1] = qb[1];
+    w4[1][0] = kw[0]; w4[1][1] = kw[1]; b4[1][0] = kb[0]; b4[1][1] = kb[1];
+  }
+  f32x4 cs4[4] = {};
+  if (interleaved) {   // (cos, sin) of this lane's four pairs
+    const f32x4* cs = (const f32x4*)(a.rope_cs + ((long long)t * 32 + c * 4) * 2);
+    cs4[0] = cs[0]; cs4[1] = cs[1];
+  } else if (has_rope) {   // (cos, sin) of this lane's eight elements
+    const f32x4* cs = (const f32x4*)(a.rope_cs + ((long long)t * 64 + c * 8) * 2);
+    cs4[0] = cs[0]; cs4[1] = cs[1]; cs4[2] = cs[2]; cs4[3] = cs[3];
+  }
+  int pool_row = -1;
+  if (APPEND) pool_row = a.append_rows[t];
 
-  if (which < 2) {
-    if (a.norm_w[which]) {
+  float x[3][8];
+#pragma unroll
+  for (int w = 0; w < 3; ++w) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      if (SRC == 0) {
+        const unsigned pair = raw16[w][i >> 1];
+        x[w][i] = __builtin_bit_cast(float, (i & 1) ? (pair & 0xffff0000u) : (pair << 16));
+      } else {
+        x[w][i] = raw32[w][i >> 2][i & 3];
+      }
+    }
+  }
+
+  // q and k rows: LayerNorm and rotary embedding
+#pragma unroll
+  for (int w = 0; w < 2; ++w) {
+    if (has_norm) {
       float s = 0.f;
 #pragma unroll
-      for (int i = 0; i < 8; ++i) s += x[i];
+      for (int i = 0; i < 8; ++i) s += x[w][i];
       s += __shfl_xor(s, 1);
       s += __shfl_xor(s, 2);
       s += __shfl_xor(s, 4);
       const float mean = s * (1.0f / 64.0f);
       float v = 0.f;
 #pragma unroll
-      for (int i = 0; i < 8; ++i) v += (x[i] - mean) * (x[i] - mean);
+      for (int i = 0; i < 8; ++i) v += (x[w][i] - mean) * (x[w][i] - mean);
       v += __shfl_xor(v, 1);
       v += __shfl_xor(v, 2);
       v += __shfl_xor(v, 4);
       const float rstd = __builtin_amdgcn_rsqf(v * (1.0f / 64.0f) + a.eps);  // torch's LayerNorm uses rsqrt too
-      const float* w = a.norm_w[which] + c * 8;
-      const float* b = a.norm_b[which] + c * 8;
 #pragma unroll
       for (int i = 0; i < 8; ++i) {
-        const float y = __fadd_rn(__fmul_rn(__fmul_rn(x[i] - mean, rstd), w[i]), b[i]);
-        x[i] = SRC == 0 ? round_bf16(y) : y;
+        const float y = add_rn(mul_rn(mul_rn(x[w][i] - mean, rstd), w4[w][i >> 2][i & 3]), b4[w][i >> 2][i & 3]);
+        x[w][i] = SRC == 0 ? round_bf16(y) : y;
       }
     }
-    if (a.rope_cs && a.rope_layout == LBM_ROPE_INTERLEAVED) {
-      const f32x4* cs = (const f32x4*)(a.rope_cs + ((long long)t * 32 + c * 4) * 2);
+    if (interleaved) {
 #pragma unroll
       for (int p = 0; p < 2; ++p) {
-        const f32x4 q4 = cs[p];  // (cos, sin) of two pairs
+        const f32x4 q4 = cs4[p];  // (cos, sin) of two pairs
 #pragma unroll
         for (int j = 0; j < 2; ++j) {
           const int i = 4 * p + 2 * j;
           float co = q4[2 * j], si = q4[2 * j + 1];
-          const float x1 = x[i], x2 = x[i + 1];
+          const float x1 = x[w][i], x2 = x[w][i + 1];
           if (SRC == 0) {
             co = round_bf16(co);
             si = round_bf16(si);
-            x[i] = round_bf16(__fsub_rn(round_bf16(__fmul_rn(x1, co)), round_bf16(__fmul_rn(x2, si))));
-            x[i + 1] = round_bf16(__fadd_rn(round_bf16(__fmul_rn(x1, si)), round_bf16(__fmul_rn(x2, co))));
+            x[w][i] = round_bf16(sub_rn(round_bf16(mul_rn(x1, co)), round_bf16(mul_rn(x2, si))));
+            x[w][i + 1] = round_bf16(add_rn(round_bf16(mul_rn(x1, si)), round_bf16(mul_rn(x2, co))));
           } else {
-            x[i] = __fsub_rn(__fmul_rn(x1, co), __fmul_rn(x2, si));
-            x[i + 1] = __fadd_rn(__fmul_rn(x1, si), __fmul_rn(x2, co));
+            x[w][i] = sub_rn(mul_rn(x1, co), mul_rn(x2, si));
+            x[w][i + 1] = add_rn(mul_rn(x1, si), mul_rn(x2, co));
           }
         }
       }
-    } else if (a.rope_cs) {
+    } else if (has_rope) {
       // half-split pairs: in each 32-element half, element j < 16 rotates with element j + 16
       // (x * cos + rotate(x) * sin with rotate = (-second, first), rope.py:123-152); the partner
       // sits two lanes away in the 8-lane group
-      const f32x4* cs = (const f32x4*)(a.rope_cs + ((long long)t * 64 + c * 8) * 2);
       const bool first = (c & 2) == 0;
 #pragma unroll
       for (int p = 0; p < 4; ++p) {
-        const f32x4 q4 = cs[p];  // (cos, sin) of two elements
+        const f32x4 q4 = cs4[p];  // (cos, sin) of two elements
 #pragma unroll
         for (int j = 0; j < 2; ++j) {
           const int i = 2 * p + j;
           float co = q4[2 * j], si = q4[2 * j + 1];
-          const float own = x[i];
+          const float own = x[w][i];
           const float other = __shfl_xor(own, 2);
           if (SRC == 0) {
             co = round_bf16(co);
             si = round_bf16(si);
-            const float a0 = round_bf16(__fmul_rn(own, co)), b0 = round_bf16(__fmul_rn(other, si));
-            x[i] = round_bf16(first ? __fsub_rn(a0, b0) : __fadd_rn(a0, b0));
+            const float a0 = round_bf16(mul_rn(own, co)), b0 = round_bf16(mul_rn(other, si));
+            x[w][i] = round_bf16(first ? sub_rn(a0, b0) : add_rn(a0, b0));
           } else {
-            const float a0 = __fmul_rn(own, co), b0 = __fmul_rn(other, si);
-            x[i] = first ? __fsub_rn(a0, b0) : __fadd_rn(a0, b0);
+            const float a0 = mul_rn(own, co), b0 = mul_rn(other, si);
+            x[w][i] = first ? sub_rn(a0, b0) : add_rn(a0, b0);
           }
         }
       }
@@ -169,15 +235,14 @@ __global__ __launch_bounds__(256) void lbm_qkv_prepare_d64_kernel(PrepareArgs a)
   }
 
   const long long nhd = ((long long)t * H + h) * 64 + c * 8;
-  if (a.out[which]) store8<DST>(a.out[which], nhd, x);
-  if (which > 0 && a.append_rows) {
-    const int row = a.append_rows[t];
-    if (row >= 0) {
-      const long long row_elems = (long long)H * 64;
-      const long long d = (long long)row * row_elems + (which == 2 ? (long long)a.page_size * row_elems : 0) +
-                          h * 64 + c * 8;
-      store8<DST>(a.pool, d, x);
-    }
+  store8<DST>(a.q_out, nhd, x[0]);
+  if (a.k_out) store8<DST>(a.k_out, nhd, x[1]);
+  if (a.v_out) store8<DST>(a.v_out, nhd, x[2]);
+  if (pool_row >= 0) {
+    const long long row_elems = (long long)H * 64;
+    const long long d = (long long)pool_row * row_elems + h * 64 + c * 8;
+    store8<DST>(a.pool, d, x[1]);
+    store8<DST>(a.pool, d + (long long)a.page_size * row_elems, x[2]);
   }
 }
 
@@ -190,11 +255,11 @@ int lbm_launch_qkv_prepare(const void* qkv, int src_dtype, const float* q_norm_w
                            int num_heads, int page_size, hipStream_t stream) {
   PrepareArgs a;
   a.qkv = qkv;
-  a.norm_w[0] = q_norm_w; a.norm_b[0] = q_norm_b;
-  a.norm_w[1] = k_norm_w; a.norm_b[1] = k_norm_b;
+  a.q_norm_w = q_norm_w; a.q_norm_b = q_norm_b;
+  a.k_norm_w = k_norm_w; a.k_norm_b = k_norm_b;
   a.rope_cs = rope_cs;
   a.rope_layout = rope_layout;
-  a.out[0] = q_out; a.out[1] = k_out; a.out[2] = v_out;
+  a.q_out = q_out; a.k_out = k_out; a.v_out = v_out;
   a.pool = pool;
   a.append_rows = append_rows;
   a.eps = norm_eps;
@@ -202,12 +267,33 @@ int lbm_launch_qkv_prepare(const void* qkv, int src_dtype, const float* q_norm_w
   const long long rows = (long long)n_tokens * 3 * num_heads;
   if (rows == 0) return LBM_OK;
   if (rows > 0x7fffffffLL) return lbm_fail(LBM_ERR_UNSUPPORTED, "lbm_qkv_prepare: %lld rows exceed 2^31", rows);
-  const dim3 grid((unsigned)((rows + 31) / 32)), block(256);
-#define LBM_PREPARE_CASE(S, D) hipLaunchKernelGGL((lbm_qkv_prepare_d64_kernel<S, D>), grid, block, 0, stream, a)
-  if (src_dtype == LBM_DTYPE_BF16 && dst_dtype == LBM_DTYPE_BF16) LBM_PREPARE_CASE(0, 0);
-  else if (src_dtype == LBM_DTYPE_F32 && dst_dtype == LBM_DTYPE_F32) LBM_PREPARE_CASE(1, 1);
-  else if (src_dtype == LBM_DTYPE_F32 && dst_dtype == LBM_DTYPE_BF16) LBM_PREPARE_CASE(1, 0);
-  else LBM_PREPARE_CASE(0, 1);
+  // one frame (16,064 groups) spreads better over 256 CUs in workgroups of 16 groups; several
+  // streams' worth of rows run a little faster in workgroups of 32
+  const int bs = rows / 3 <= 32768 ? 128 : 256;
+  const dim3 grid((unsigned)((rows / 3 + bs / 8 - 1) / (bs / 8))), block(bs);
+  const int rope = !rope_cs ? 0 : (rope_layout == LBM_ROPE_INTERLEAVED ? 1 : 2);
+  const bool norm = q_norm_w != nullptr, append = append_rows != nullptr;
+#define LBM_PREPARE_LAUNCH(S, D, R, N, A) \
+  hipLaunchKernelGGL((lbm_qkv_prepare_d64_kernel<S, D, R, N, A>), grid, block, 0, stream, a)
+#define LBM_PREPARE_NA(S, D, R)                            \
+  {                                                        \
+    if (norm && append) LBM_PREPARE_LAUNCH(S, D, R, true, true);         \
+    else if (norm) LBM_PREPARE_LAUNCH(S, D, R, true, false);             \
+    else if (append) LBM_PREPARE_LAUNCH(S, D, R, false, true);           \
+    else LBM_PREPARE_LAUNCH(S, D, R, false, false);                      \
+  }
+#define LBM_PREPARE_CASE(S, D)                \
+  {                                           \
+    if (rope == 0) LBM_PREPARE_NA(S, D, 0)    \
+    else if (rope == 1) LBM_PREPARE_NA(S, D, 1) \
+    else LBM_PREPARE_NA(S, D, 2)              \
+  }
+  if (src_dtype == LBM_DTYPE_BF16 && dst_dtype == LBM_DTYPE_BF16) LBM_PREPARE_CASE(0, 0)
+  else if (src_dtype == LBM_DTYPE_F32 && dst_dtype == LBM_DTYPE_F32) LBM_PREPARE_CASE(1, 1)
+  else if (src_dtype == LBM_DTYPE_F32 && dst_dtype == LBM_DTYPE_BF16) LBM_PREPARE_CASE(1, 0)
+  else LBM_PREPARE_CASE(0, 1)
 #undef LBM_PREPARE_CASE
+#undef LBM_PREPARE_NA
+#undef LBM_PREPARE_LAUNCH
   return lbm_check_launch("lbm_qkv_prepare_d64_kernel");
 }

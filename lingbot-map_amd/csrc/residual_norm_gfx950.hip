@@ -97,10 +97,15 @@ __global__ __launch_bounds__(kThreads) void lbm_residual_norm_kernel(ResidualNor
       float x[8], y[8];
       load8<DT>(a.x, base + col, x);
       load8<DT>(a.y, base + col, y);
+      f32x4 ga[2] = {{1.f, 1.f, 1.f, 1.f}, {1.f, 1.f, 1.f, 1.f}};
+      if (a.gamma) {   // a launch parameter: uniform
+        ga[0] = *(const f32x4*)(a.gamma + col);
+        ga[1] = *(const f32x4*)(a.gamma + col + 4);
+      }
 #pragma unroll
       for (int i = 0; i < 8; ++i) {
         float t = y[i];
-        if (a.gamma) t = DT == 0 ? round_bf16(__fmul_rn(t, a.gamma[col + i])) : __fmul_rn(t, a.gamma[col + i]);
+        if (a.gamma) t = DT == 0 ? round_bf16(__fmul_rn(t, ga[i >> 2][i & 3])) : __fmul_rn(t, ga[i >> 2][i & 3]);
         const float s = __fadd_rn(x[i], t);
         v[c][i] = DT == 0 ? round_bf16(s) : s;
         sum += v[c][i];
@@ -127,10 +132,12 @@ __global__ __launch_bounds__(kThreads) void lbm_residual_norm_kernel(ResidualNor
   for (int c = 0; c < NCH; ++c) {
     const int col = c * 1024 + threadIdx.x * 8;
     if (c < n_chunks && col < a.cols) {
+      const f32x4 w0 = *(const f32x4*)(a.norm_w + col), w1 = *(const f32x4*)(a.norm_w + col + 4);
+      const f32x4 b0 = *(const f32x4*)(a.norm_b + col), b1 = *(const f32x4*)(a.norm_b + col + 4);
       float o[8];
 #pragma unroll
       for (int i = 0; i < 8; ++i)
-        o[i] = __fadd_rn(__fmul_rn(__fmul_rn(v[c][i] - mean, rstd), a.norm_w[col + i]), a.norm_b[col + i]);
+        o[i] = __fadd_rn(__fmul_rn(__fmul_rn(v[c][i] - mean, rstd), i < 4 ? w0[i & 3] : w1[i & 3]), i < 4 ? b0[i & 3] : b1[i & 3]);
       store8<DT>(a.n_out, base + col, o);
     }
   }
@@ -145,20 +152,43 @@ __global__ __launch_bounds__(256) void lbm_residual_norm_wave_kernel(ResidualNor
   const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
   if (row >= a.rows) return;   // whole wavefronts leave; nothing below synchronises across them
   const long long base = (long long)row * a.cols;
+  const bool has_gamma = a.gamma != nullptr, has_norm = a.norm_w != nullptr;   // launch parameters: uniform
+  // Every load of the row is issued before the first use of any of them - x, y, LayerScale and
+  // the LayerNorm parameters: the kernel is a chain of memory latencies, not of bandwidth.
+  float x[NV][8], y[NV][8];
+  f32x4 ga[NV][2], nw[NV][2], nb[NV][2];
+#pragma unroll
+  for (int c = 0; c < NV; ++c) {
+    const int col = (c * 64 + lane) * 8;
+    ga[c][0] = ga[c][1] = f32x4{1.f, 1.f, 1.f, 1.f};
+    nw[c][0] = nw[c][1] = nb[c][0] = nb[c][1] = f32x4{0.f, 0.f, 0.f, 0.f};
+    if (col < a.cols) {
+      load8<DT>(a.x, base + col, x[c]);
+      load8<DT>(a.y, base + col, y[c]);
+      if (has_gamma) {
+        ga[c][0] = *(const f32x4*)(a.gamma + col);
+        ga[c][1] = *(const f32x4*)(a.gamma + col + 4);
+      }
+      if (has_norm) {
+        nw[c][0] = *(const f32x4*)(a.norm_w + col);
+        nw[c][1] = *(const f32x4*)(a.norm_w + col + 4);
+        nb[c][0] = *(const f32x4*)(a.norm_b + col);
+        nb[c][1] = *(const f32x4*)(a.norm_b + col + 4);
+      }
+    }
+  }
   float v[NV][8];
   float sum = 0.f;
 #pragma unroll
   for (int c = 0; c < NV; ++c) {
     const int col = (c * 64 + lane) * 8;
     if (col < a.cols) {
-      float x[8], y[8];
-      load8<DT>(a.x, base + col, x);
-      load8<DT>(a.y, base + col, y);
 #pragma unroll
       for (int i = 0; i < 8; ++i) {
-        float t = y[i];
-        if (a.gamma) t = DT == 0 ? round_bf16(__fmul_rn(t, a.gamma[col + i])) : __fmul_rn(t, a.gamma[col + i]);
-        const float s = __fadd_rn(x[i], t);
+        float t = y[c][i];
+        // without LayerScale the factor is 1 and the product is y itself
+        if (has_gamma) t = DT == 0 ? round_bf16(__fmul_rn(t, ga[c][i >> 2][i & 3])) : __fmul_rn(t, ga[c][i >> 2][i & 3]);
+        const float s = __fadd_rn(x[c][i], t);
         v[c][i] = DT == 0 ? round_bf16(s) : s;
         sum += v[c][i];
       }
@@ -168,7 +198,7 @@ __global__ __launch_bounds__(256) void lbm_residual_norm_wave_kernel(ResidualNor
       for (int i = 0; i < 8; ++i) v[c][i] = 0.f;
     }
   }
-  if (!a.norm_w) return;  // uniform: a launch parameter
+  if (!has_norm) return;
 #pragma unroll
   for (int o = 32; o >= 1; o >>= 1) sum += __shfl_xor(sum, o);
   const float mean = sum / (float)a.cols;
@@ -189,7 +219,7 @@ __global__ __launch_bounds__(256) void lbm_residual_norm_wave_kernel(ResidualNor
       float o[8];
 #pragma unroll
       for (int i = 0; i < 8; ++i)
-        o[i] = __fadd_rn(__fmul_rn(__fmul_rn(v[c][i] - mean, rstd), a.norm_w[col + i]), a.norm_b[col + i]);
+        o[i] = __fadd_rn(__fmul_rn(__fmul_rn(v[c][i] - mean, rstd), nw[c][i >> 2][i & 3]), nb[c][i >> 2][i & 3]);
       store8<DT>(a.n_out, base + col, o);
     }
   }
