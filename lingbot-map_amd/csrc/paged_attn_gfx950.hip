@@ -107,13 +107,24 @@ __device__ __forceinline__ float swap_max(float x) {
   return max2(lo, hi);
 }
 
-}  // namespace
+// LDS of the split-KV kernel, at namespace scope because the kernel and the out-of-line second
+// pass below both work in it.
+__shared__ __attribute__((aligned(16))) unsigned short lds_k[kStages][kKvTile * kKStride];
+__shared__ __attribute__((aligned(16))) unsigned short lds_v[kStages][kKvTile * kVStride];
+__shared__ __attribute__((aligned(16))) unsigned short lds_q[kWaves][kQPerWave * kKStride];   // per-wave patch: Q on the way in
 
-__global__ __launch_bounds__(kThreads, 1) void lbm_attn_bf16_d64_kernel(AttnArgs a) {
-  __shared__ __attribute__((aligned(16))) unsigned short lds_k[kStages][kKvTile * kKStride];
-  __shared__ __attribute__((aligned(16))) unsigned short lds_v[kStages][kKvTile * kVStride];
-  __shared__ __attribute__((aligned(16))) unsigned short lds_q[kWaves][kQPerWave * kKStride];   // per-wave patch: Q on the way in
+// The repeat pass is a function of its own, not inlined: it is entered once in a blue moon,
+// and compiled into the kernel body its registers would push the common path into scratch
+// memory (spill stores and reloads on every launch, tens of MB of HBM traffic).
+__device__ __noinline__ void lbm_attn_split_safe(AttnArgs a);
 
+// One workgroup's share of the split-KV attention: 512 query rows of one head over one run of
+// KV tiles, start to finish.  SAFE = false is the common path (no softmax reference, range
+// check at the end); when the check fails it writes nothing, hands the workgroup to the
+// repeat pass and ends the program there, so that nothing of the common path is live across
+// the call.  SAFE = true is the repeat with a reference that follows the row maxima.
+template <bool SAFE>
+__device__ __forceinline__ void lbm_attn_split(const AttnArgs& a) {
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int n32 = lane & 31, g = lane >> 5;
 
@@ -494,8 +505,8 @@ __global__ __launch_bounds__(kThreads, 1) void lbm_attn_bf16_d64_kernel(AttnArgs
   // magnitude).  Scores in log2 units beyond about +-100 - unheard of behind a q/k LayerNorm -
   // make a row sum or an output overflow or vanish; the check after the pass sees that and the
   // whole workgroup repeats its split with a reference that follows the row maxima (pass 1).
-  for (int pass = 0; pass < 2; ++pass) {
-    const bool safe = pass != 0;
+  {
+    constexpr bool safe = SAFE;
 #pragma unroll
     for (int qb = 0; qb < 2; ++qb) {
 #pragma unroll
@@ -599,11 +610,10 @@ __global__ __launch_bounds__(kThreads, 1) void lbm_attn_bf16_d64_kernel(AttnArgs
         for (int kk = 0; kk < 2; ++kk)
           lacc[qb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(lsel, pB[qb][kk], lacc[qb], 0, 0, 0);
     }
-    if (safe) break;
     // Did the pass without reference stay in range?  Compared as integers (non-negative floats
     // order like their bit patterns; NaN, infinity and negative values land above every bound).
     bool bad = false;
-    if (n > 0) {
+    if (!safe && n > 0) {
       unsigned top = 0u;
 #pragma unroll
       for (int qb = 0; qb < 2; ++qb)
@@ -622,7 +632,10 @@ __global__ __launch_bounds__(kThreads, 1) void lbm_attn_bf16_d64_kernel(AttnArgs
           }
       }
     }
-    if (!__syncthreads_or(bad)) break;
+    if (!safe && __builtin_amdgcn_readfirstlane(__syncthreads_or(bad))) {
+      lbm_attn_split_safe(a);
+      __builtin_amdgcn_endpgm();
+    }
   }
 #undef LBM_FAST_HALF_STEP
 #undef LBM_F4
@@ -671,6 +684,14 @@ __global__ __launch_bounds__(kThreads, 1) void lbm_attn_bf16_d64_kernel(AttnArgs
     if (!direct && g == 0 && r < sp.q_rows)
       a.part_lse[(dst_row0 + r) * H + head] = m_run[qb] + __builtin_amdgcn_logf(l_tot);
   }
+}
+
+__device__ __noinline__ void lbm_attn_split_safe(AttnArgs a) { lbm_attn_split<true>(a); }
+
+}  // namespace
+
+__global__ __launch_bounds__(kThreads, 1) void lbm_attn_bf16_d64_kernel(AttnArgs a) {
+  lbm_attn_split<false>(a);
 }
 
 // ---------------------------------------------------------------------------- bf16, short KV

@@ -192,6 +192,57 @@ def test_attention_late_dominant_tokens():
         assert (out[r].float() - v[t].float()).abs().max().item() <= 1e-2
 
 
+@pytest.mark.parametrize("n_kv", [1000, 6000])
+@pytest.mark.parametrize("case", ["overflow", "vanish"])
+def test_attention_scores_out_of_range_take_the_repeat_pass(case, n_kv):
+    """The first pass of both bf16 kernels (short KV: 1,000 tokens; split KV: 6,000) feeds the
+    scores to exp2 without a softmax reference; a score beyond 2^+-100 fails its range check and
+    the workgroup repeats its work with a running-maximum reference.  "overflow": a few keys are
+    12 x their query row (score 138 in log2 units, 2^138 is not an fp32 number), the row's output
+    is that key's V row.  "vanish": every key is -12 x the common query direction (all scores
+    -138, every numerator flushes to 0), the output is the mean of V."""
+    from oracle.sdpa_cache import sdpa_nhd
+    dev = torch.device("cuda:0")
+    g = torch.Generator().manual_seed(29)
+    tq, H, D, S = 200, 4, 64, 16
+    n_pages = -(-n_kv // S)
+    v = torch.randn(n_pages * S, H, D, generator=g).to(torch.bfloat16)
+    if case == "overflow":
+        # spike rows live in head dimensions 0-7, every other row in 8-63, so a spike key scores
+        # exactly 0 against the other rows and only its own row is peaked
+        spikes = [(3, 17), (64, n_kv // 2), (199, n_kv - 1)]
+        q = torch.randn(tq, H, D, generator=g)
+        q[:, :, :8] = 0.0
+        for r, _ in spikes:
+            q[r] = 0.0
+            q[r, :, :8] = torch.randn(H, 8, generator=g)
+        q = (q * (8.0 / q.norm(dim=-1, keepdim=True))).to(torch.bfloat16)     # |q| = 8
+        k = 0.1 * torch.randn(n_pages * S, H, D, generator=g)
+        for r, t in spikes:
+            k[t] = 12.0 * q[r].float()                                         # score 12 * 64 / 8 = 96, x log2(e) = 138
+    else:
+        u = torch.randn(1, H, D, generator=g)
+        u = u * (8.0 / u.norm(dim=-1, keepdim=True))
+        q = u.expand(tq, H, D).contiguous().to(torch.bfloat16)
+        k = (-12.0 * u).expand(n_pages * S, H, D).contiguous()
+    k = k.to(torch.bfloat16)
+    pool = torch.zeros(n_pages, 2, S, H, D, dtype=torch.bfloat16)
+    pool[:, 0] = k.view(n_pages, S, H, D)
+    pool[:, 1] = v.view(n_pages, S, H, D)
+    lens = [S] * (n_pages - 1) + [n_kv - (n_pages - 1) * S]
+    rows, n_tok = rows_from_pages(list(range(n_pages)), lens, S, dev)
+    assert n_tok == n_kv
+    out = run_attention(q.to(dev), pool.to(dev), rows, [(0, tq, 0, n_tok)], S).cpu()
+    assert torch.isfinite(out.float()).all()
+    err = (out.float() - sdpa_nhd(q, k[:n_kv], v[:n_kv]).float()).abs()
+    assert err.mean().item() <= BF16_MEAN_ABS and err.max().item() <= BF16_MAX_ABS, (err.mean().item(), err.max().item())
+    if case == "overflow":
+        for r, t in spikes:
+            assert (out[r].float() - v[t].float()).abs().max().item() <= 1e-2
+    else:
+        assert (out.float() - v[:n_kv].float().mean(0)).abs().max().item() <= 1e-2
+
+
 def test_attention_closed_forms():
     dev = torch.device("cuda:0")
     H, D, S = 2, 64, 16
