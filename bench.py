@@ -30,8 +30,8 @@ PEAK_HBM_GBPS = 8000.0
 # merges its split-KV partial results - from rocprofv3 --pmc FETCH_SIZE (x2.0, the factor a
 # 256 MiB plain copy gives) and WRITE_SIZE (x1.0), in KiB per dispatch
 # (profiles/attention_config2_hbm_traffic.md): main ATTN_MAIN_KIB, combine ATTN_COMBINE_KIB
-ATTN_MAIN_KIB = (35738.0, 20592.0)       # (FETCH_SIZE, WRITE_SIZE) of lbm_attn_bf16_d64_kernel
-ATTN_COMBINE_KIB = (8315.3, 2008.0)      # of lbm_attn_combine_bf16_kernel
+ATTN_MAIN_KIB = (35503.5, 20080.0)       # (FETCH_SIZE, WRITE_SIZE) of lbm_attn_bf16_d64_kernel
+ATTN_COMBINE_KIB = (8313.9, 2008.0)      # of lbm_attn_combine_bf16_kernel
 ATTN_TRAFFIC_BYTES = ((ATTN_MAIN_KIB[0] + ATTN_COMBINE_KIB[0]) * 2.0 + ATTN_MAIN_KIB[1] + ATTN_COMBINE_KIB[1]) * 1024.0
 METRIC = "frames/sec streaming @518x378 (1 GPU); attention TFLOPS & % bf16 MFMA peak"
 

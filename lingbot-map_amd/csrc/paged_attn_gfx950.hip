@@ -168,6 +168,39 @@ __device__ __forceinline__ void lbm_attn_split(const AttnArgs& a) {
   const int n = t1 - t0;
   const unsigned row_bytes = (unsigned)H * 128u;
 
+  // ---- tile staging: each thread moves one 16-byte piece of a K row and of a V row per tile.
+  // Rows past the last token re-read the last token (finite data; the softmax masks them).
+  const int ld_r = tid >> 3, ld_c = (tid & 7) * 8;
+  const char* pool_k = (const char*)(a.pool + (size_t)head * 64 + ld_c);
+  const char* pool_v = pool_k + (size_t)a.page_size * row_bytes;
+  const char* own_k = (const char*)(a.self_k + (size_t)head * 64 + ld_c);
+  const char* own_v = (const char*)(a.self_v + (size_t)head * 64 + ld_c);
+  const int32_t* rows = a.kv_rows + sp.kv_row_begin;
+  const int last_token = max(kv_tokens - 1, 0);
+  // Tiles past the end of this split re-read its last tile: the data lands in ring stages
+  // nobody reads any more, and the code stays free of branches.
+  auto row_entry = [&](int t) -> int { return rows[min(max(min(t, t1 - 1), 0) * kKvTile + ld_r, last_token)]; };
+  auto fetch = [&](int e, const char* pool_base, const char* own_base) -> u32x4 {
+    // negative entries name rows of the caller's own K/V (read-only tail of a non-keyframe)
+    const char* base = e < 0 ? own_base : pool_base;
+    const unsigned r = (unsigned)(e ^ (e >> 31));
+    return *(const u32x4*)(base + (unsigned long long)r * row_bytes);
+  };
+  auto put_k = [&](int stage, u32x4 v) { *(u32x4*)&lds_k[stage][ld_r * kKStride + ld_c] = v; };
+  auto put_v = [&](int stage, u32x4 v) { *(u32x4*)&lds_v[stage][ld_r * kVStride + ld_c] = v; };
+
+  // The first tiles' rows are asked for before anything else: the row table entry, then the K/V
+  // row it names, is the longest chain of memory latencies in front of the first MFMA, and the
+  // Q rows below travel at the same time.
+  const int e_t0 = row_entry(t0), e_t1 = row_entry(t0 + 1), e_t2 = row_entry(t0 + 2);
+  int ek = row_entry(t0 + 3), ev = e_t2;   // entries of the fetches after those
+  const u32x4 k_t0 = fetch(e_t0, pool_k, own_k);
+  const u32x4 k_t1 = fetch(e_t1, pool_k, own_k);
+  const u32x4 v_t0 = fetch(e_t0, pool_v, own_v);
+  // in flight across the first iteration: K(2), V(1)
+  u32x4 kreg = fetch(e_t2, pool_k, own_k);
+  u32x4 vreg = fetch(e_t1, pool_v, own_v);
+
   // ---- Q fragments (B operand of S^T = K Q^T): lane holds q row n32, d = ks*16 + g*8 .. +8.
   // Each wavefront reads its 64 query rows as whole 128-byte rows (eight lanes per row), parks
   // them in its own LDS patch and picks the fragments up from there; read directly in the
@@ -222,27 +255,6 @@ __device__ __forceinline__ void lbm_attn_split(const AttnArgs& a) {
   f32x4 lacc[2];
   const unsigned sel_word = (lane == 0 || lane == 32 || lane == 17 || lane == 49) ? 0x3F803F80u : 0u;
   const bf16x8 lsel = __builtin_bit_cast(bf16x8, u32x4{sel_word, sel_word, sel_word, sel_word});
-
-  // ---- tile staging: each thread moves one 16-byte piece of a K row and of a V row per tile.
-  // Rows past the last token re-read the last token (finite data; the softmax masks them).
-  const int ld_r = tid >> 3, ld_c = (tid & 7) * 8;
-  const char* pool_k = (const char*)(a.pool + (size_t)head * 64 + ld_c);
-  const char* pool_v = pool_k + (size_t)a.page_size * row_bytes;
-  const char* own_k = (const char*)(a.self_k + (size_t)head * 64 + ld_c);
-  const char* own_v = (const char*)(a.self_v + (size_t)head * 64 + ld_c);
-  const int32_t* rows = a.kv_rows + sp.kv_row_begin;
-  const int last_token = max(kv_tokens - 1, 0);
-  // Tiles past the end of this split re-read its last tile: the data lands in ring stages
-  // nobody reads any more, and the code stays free of branches.
-  auto row_entry = [&](int t) -> int { return rows[min(max(min(t, t1 - 1), 0) * kKvTile + ld_r, last_token)]; };
-  auto fetch = [&](int e, const char* pool_base, const char* own_base) -> u32x4 {
-    // negative entries name rows of the caller's own K/V (read-only tail of a non-keyframe)
-    const char* base = e < 0 ? own_base : pool_base;
-    const unsigned r = (unsigned)(e ^ (e >> 31));
-    return *(const u32x4*)(base + (unsigned long long)r * row_bytes);
-  };
-  auto put_k = [&](int stage, u32x4 v) { *(u32x4*)&lds_k[stage][ld_r * kKStride + ld_c] = v; };
-  auto put_v = [&](int stage, u32x4 v) { *(u32x4*)&lds_v[stage][ld_r * kVStride + ld_c] = v; };
 
   // Register state of the software pipeline.  A 64-token tile is processed as two 32-token
   // halves; while the vector ALU turns the scores of one half into softmax numerators, the
@@ -519,9 +531,9 @@ __device__ __forceinline__ void lbm_attn_split(const AttnArgs& a) {
     }
 
     // ---- prologue: K(0), K(1), V(0) into the ring; the V stage the first PV reads is zeroed
-    put_k(0, fetch(row_entry(t0), pool_k, own_k));
-    put_k(1, fetch(row_entry(t0 + 1), pool_k, own_k));
-    put_v(0, fetch(row_entry(t0), pool_v, own_v));
+    put_k(0, k_t0);
+    put_k(1, k_t1);
+    put_v(0, v_t0);
     {
       const u32x4 zero = {0u, 0u, 0u, 0u};
       put_v(2, zero);
@@ -530,10 +542,6 @@ __device__ __forceinline__ void lbm_attn_split(const AttnArgs& a) {
     for (int qb = 0; qb < 2; ++qb)
 #pragma unroll
       for (int kk = 0; kk < 2; ++kk) pB[qb][kk] = __builtin_bit_cast(bf16x8, u32x4{0u, 0u, 0u, 0u});
-    // in flight across the first iteration: K(2), V(1); entries of the fetches after them
-    u32x4 kreg = fetch(row_entry(t0 + 2), pool_k, own_k);
-    u32x4 vreg = fetch(row_entry(t0 + 1), pool_v, own_v);
-    int ek = row_entry(t0 + 3), ev = row_entry(t0 + 2);
     __syncthreads();
     qk_half(0, 0, kv_tokens - t0 * kKvTile, sA);
     if (safe) {
