@@ -5,36 +5,39 @@
 // bf16 kernel, head_dim 64.  One workgroup = 8 wavefronts x 64 query rows of one head over
 // one contiguous run of 64-token KV tiles (split-KV; partial results are merged by
 // lbm_attn_combine_bf16_kernel).  Per tile a wavefront computes
-//     S^T = K Q^T - m  v_mfma_f32_32x32x16_bf16, A = K rows from LDS, B = Q in registers; the
-//                      softmax scale (in log2 units) is folded into Q and the reference m
-//                      into one more k-step, so S arrives ready for exp2
+//     S^T = K Q^T      v_mfma_f32_32x32x16_bf16, A = K rows from LDS, B = Q in registers; the
+//                      softmax scale (in log2 units) is folded into Q, so S arrives ready
+//                      for exp2
 //     P   = exp2(S)    one query row per lane column; v_exp_f32 + v_cvt_pk_bf16_f32
 //     O^T += V^T P^T   A = V^T read with ds_read_b64_tr_b16 from the row-major V tile,
 //                      B = P^T straight from the registers the packing wrote
 //     l   += 1^T P^T   row sums on the matrix pipe too (16x16x32 with a 0/1 selector)
-// The reference m of a row is not its running maximum but a value kHeadroom above the
-// maximum seen when it was last set, and it is only raised when a numerator reaches 2, i.e.
-// when a score exceeds it; the same reference divides out of O / l, so the result is
-// mathematically unchanged, no row maximum is computed on the common path, and O is rescaled
-// only on the rare path.  The test costs a few OR instructions per half tile: a bf16 numerator
-// is >= 2 (or infinite) exactly when the top bit of its exponent field is set.
+// Common path: no softmax reference at all.  2^score is exact softmax arithmetic as long as
+// nothing leaves the range of fp32 / bf16; a range check on O and l after the last tile
+// decides, per workgroup, whether that held.  If not - scores beyond about +-100 in log2
+// units - the workgroup repeats its split in an out-of-line function (lbm_attn_split_safe)
+// with a reference m carried into the QK^T contraction as one more k-step: m is kHeadroom
+// above the row maximum seen when it was last set and is only raised when a numerator
+// reaches 2 (a bf16 numerator is >= 2 or infinite exactly when the top bit of its exponent
+// field is set: a few OR instructions per half tile), with O, l and the scores in flight
+// rescaled on that rare path.  The same extra k-step masks the rows past the last token on
+// the ragged last tiles of either path.
 //
 // Why it is built this way.  Measured on MI355X with two wavefronts per SIMD: v_exp_f32 issues
 // every ~4.6 ns per SIMD, v_cvt_pk_bf16_f32 (like v_max3_f32, v_dot2c_f32_bf16) every ~2.7 ns, plain
 // fp32 adds and multiplies every ~1.4 ns, and a 32x32x16 MFMA occupies the matrix pipe for
 // 13.8 ns.  With head_dim 64 every score needs one exp2 and half a packing instruction, so the
-// vector ALU, not the matrix pipe, bounds the loop; everything that can run as an MFMA (scale,
-// reference subtraction, masking of the ragged tail, row sums) does, and the vector ALU is
-// left with exp2, packing and the overflow test.
+// vector ALU is as busy as the matrix pipe; everything that can run as an MFMA (scale, row
+// sums, masking of the ragged tail, the reference subtraction of the repeat pass) does, and
+// the vector ALU is left with exp2 and packing.
 //
 // Schedule.  Each wavefront runs a software pipeline over 32-token half tiles: while the
 // vector ALU turns the scores of one half into numerators, the MFMAs of the next half's QK^T
 // and of the previous half's PV and row sums are issued in between.  A half-step is one basic
-// block written as 22 slices (one MFMA plus its share of the vector work and LDS reads each)
-// fenced with sched_barrier, and the two wavefronts of a SIMD fill each other's issue gaps.
-// The numerators of a half are computed before the test on them, so the test's branch is the
-// only one in the loop and its condition is ready long before it is taken.  K/V tiles are
-// shared by all eight waves through a three-stage LDS ring with one workgroup barrier per tile.
+// block written as 20 slices (22 with the extra k-step; one MFMA plus its share of the vector
+// work and LDS reads each) fenced with sched_barrier, and the two wavefronts of a SIMD fill
+// each other's issue gaps.  K/V tiles are shared by all eight waves through a three-stage
+// LDS ring with one workgroup barrier per tile.
 #include <hip/hip_runtime.h>
 #include <climits>
 #include <mutex>
