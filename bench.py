@@ -448,7 +448,7 @@ def main() -> None:
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-aggregator", action="store_true",
                     help="skip the full aggregator-trunk step (frame + global blocks) timed after the hot path")
-    ap.add_argument("--mode", choices=["full", "attention", "attention_frame", "attention_f32", "attention_f32_few", "append", "prepare", "residual", "tables", "copy"], default="full",
+    ap.add_argument("--mode", choices=["full", "attention", "attention_frame", "attention_f32", "attention_f32_few", "append", "prepare", "residual", "tables", "copy", "linear"], default="full",
                     help="full = the benchmark line; attention/attention_frame (a frame block's 1004 x 1004 without cache)/attention_f32/attention_f32_few/append/prepare/residual/tables launch one kernel --steps "
                          "times on the steady-state cache (for rocprofv3 runs); copy = a plain 256 MiB "
                          "device copy, the known-size kernel the HBM counters are calibrated on")
@@ -470,6 +470,43 @@ def main() -> None:
         ms = event_time_ms(lambda: dst.copy_(src), args.steps, torch)
         print(json.dumps({"mode": "copy", "bytes_read": src.numel(), "bytes_written": dst.numel(),
                           "launches": args.steps, "avg_launch_us": ms * 1e3}))
+        return
+    if args.mode == "linear":
+        # the four linears of a block at one frame (1004 rows) and at four streams (4016 rows):
+        # lbm_linear with its fused epilogue against the PyTorch-ROCm calls it replaces
+        from lingbot_map_amd import _native as N
+        import ctypes as C
+        import torch.nn.functional as F
+        vp = lambda t: None if t is None else C.c_void_p(t.data_ptr())
+        g = torch.Generator(device=dev).manual_seed(5)
+        rows = []
+        for M in (1004, 4016):
+            for name, K, Nn, epi in (("qkv", 1024, 3072, N.LINEAR_BIAS), ("proj + ls + residual", 1024, 1024, N.LINEAR_BIAS_RESIDUAL),
+                                     ("fc1 + gelu", 1024, 4096, N.LINEAR_BIAS_GELU), ("fc2 + ls + residual", 4096, 1024, N.LINEAR_BIAS_RESIDUAL)):
+                a = torch.randn(M, K, generator=g, device=dev).to(torch.bfloat16)
+                w = (torch.randn(Nn, K, generator=g, device=dev) / K ** 0.5).to(torch.bfloat16)
+                b = torch.randn(Nn, generator=g, device=dev).to(torch.bfloat16)
+                gam = torch.rand(Nn, generator=g, device=dev).to(torch.bfloat16)
+                res = torch.randn(M, Nn, generator=g, device=dev).to(torch.bfloat16)
+                b32, g32 = b.float(), gam.float()
+                out = torch.empty(M, Nn, dtype=torch.bfloat16, device=dev)
+                residual = epi == N.LINEAR_BIAS_RESIDUAL
+                stream = lambda: C.c_void_p(torch.cuda.current_stream().cuda_stream)
+                ours = lambda: N.check(N.lib.lbm_linear(vp(a), vp(w), vp(b32), vp(g32) if residual else None,
+                                                         vp(res) if residual else None, vp(out), M, Nn, K, epi, stream()))
+                if epi == N.LINEAR_BIAS:
+                    theirs = lambda: F.linear(a, w, b)
+                elif epi == N.LINEAR_BIAS_GELU:
+                    theirs = lambda: F.gelu(F.linear(a, w, b))
+                else:
+                    theirs = lambda: res + F.linear(a, w, b) * gam
+                for _ in range(3):
+                    ours(); theirs()
+                t_ours, t_theirs = kernel_time_ms(ours, 50, torch) * 1e3, kernel_time_ms(theirs, 50, torch) * 1e3
+                flop = 2.0 * M * K * Nn
+                rows.append({"layer": name, "M": M, "K": K, "N": Nn, "lbm_linear_us": t_ours, "torch_us": t_theirs,
+                             "lbm_linear_tflops": flop / t_ours * 1e-6, "torch_tflops": flop / t_theirs * 1e-6})
+        print(json.dumps({"mode": "linear", "rows": rows}))
         return
     blocks = args.blocks
     m = HipPagedKVCacheManager(blocks, ANCHOR + WINDOW + 16, T, H, D, torch.bfloat16, dev,

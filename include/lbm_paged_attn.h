@@ -24,7 +24,7 @@
 extern "C" {
 #endif
 
-#define LBM_ABI_VERSION 3
+#define LBM_ABI_VERSION 4
 
 #define LBM_OK 0
 #define LBM_ERR_INVALID 1     /* bad argument (null pointer, negative size, bad enum)      */
@@ -39,6 +39,11 @@ extern "C" {
 #define LBM_LAYOUT_FRAME_PAGES 1 /* whole frame in pages; eviction compacts index-only     */
 
 /* pairing of the rotary embedding in lbm_qkv_prepare */
+/* epilogue of lbm_linear */
+#define LBM_LINEAR_BIAS 0
+#define LBM_LINEAR_BIAS_GELU 1
+#define LBM_LINEAR_BIAS_RESIDUAL 2
+
 #define LBM_ROPE_INTERLEAVED 0
 #define LBM_ROPE_HALF_SPLIT 1
 
@@ -175,6 +180,22 @@ int lbm_kv_append(const void* k, const void* v, int32_t src_dtype, void* pool,
 int lbm_residual_norm(const void* x, const void* y, int32_t dtype, const float* gamma,
                       const float* norm_w, const float* norm_b, float norm_eps, void* x_out,
                       void* n_out, int32_t rows, int32_t cols, void* stream);
+
+/* A bf16 linear layer of a transformer block with the elementwise work that follows it fused
+ * into the store: out = epilogue(a @ w^T + bias).
+ *   LBM_LINEAR_BIAS           the qkv projection (attention.py:413)
+ *   LBM_LINEAR_BIAS_GELU      fc1 followed by the exact (erf) GELU (mlp.py:35-36)
+ *   LBM_LINEAR_BIAS_RESIDUAL  proj or fc2 followed by LayerScale and the residual add:
+ *                             residual + gamma * (a @ w^T + bias) (attention.py:554, mlp.py:38,
+ *                             block.py:283, layer_scale.py:21-22)
+ *   a         [M][K] bf16          w      [N][K] bf16 (nn.Linear's weight)
+ *   bias      [N] float32 or NULL  gamma  [N] float32 or NULL (RESIDUAL only)
+ *   residual  [M][N] bf16 (RESIDUAL only; may alias out)       out  [M][N] bf16
+ * K: a multiple of 128, N: a multiple of 64.  Roundings follow the sequence of separate bf16 torch ops (the
+ * linear's output rounded to bf16, then each elementwise op). */
+int lbm_linear(const void* a, const void* w, const float* bias, const float* gamma,
+               const void* residual, void* out, int32_t M, int32_t N, int32_t K, int32_t epilogue,
+               void* stream);
 
 /* lbm_attn_run with the token counts read on the device: stream i attends to
  * live_kv_tokens[streams[i].live_at] entries of its row table instead of streams[i].kv_tokens,

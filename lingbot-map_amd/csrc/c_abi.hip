@@ -122,6 +122,17 @@ int lbm_qkv_prepare(const void* qkv, int32_t src_dtype, const float* q_norm_w, c
                                 (hipStream_t)stream);
 }
 
+int lbm_linear(const void* a, const void* w, const float* bias, const float* gamma, const void* residual,
+               void* out, int32_t M, int32_t N, int32_t K, int32_t epilogue, void* stream) {
+  if (!a || !w || !out) return lbm_fail(LBM_ERR_INVALID, "lbm_linear: null a, w or out");
+  if (M < 0 || N <= 0 || K <= 0) return lbm_fail(LBM_ERR_INVALID, "lbm_linear: bad shape %d x %d x %d", M, N, K);
+  if (epilogue == LBM_LINEAR_BIAS_RESIDUAL && !residual)
+    return lbm_fail(LBM_ERR_INVALID, "lbm_linear: the residual epilogue needs a residual");
+  if (epilogue != LBM_LINEAR_BIAS_RESIDUAL && (residual || gamma))
+    return lbm_fail(LBM_ERR_INVALID, "lbm_linear: residual / gamma given without the residual epilogue");
+  return lbm_launch_linear(a, w, bias, gamma, residual, out, M, N, K, epilogue, (hipStream_t)stream);
+}
+
 int lbm_residual_norm(const void* x, const void* y, int32_t dtype, const float* gamma, const float* norm_w,
                       const float* norm_b, float norm_eps, void* x_out, void* n_out, int32_t rows, int32_t cols,
                       void* stream) {

@@ -33,6 +33,9 @@ int lbm_launch_residual_norm(const void* x, const void* y, int dtype, const floa
                              const float* norm_b, float eps, void* x_out, void* n_out, int rows, int cols,
                              hipStream_t stream);
 
+int lbm_launch_linear(const void* a, const void* w, const float* bias, const float* gamma, const void* residual,
+                      void* out, int M, int N, int K, int epilogue, hipStream_t stream);
+
 // Split-KV schedule of one attention call, computed on the host from token counts only.
 struct LbmAttnStreamPlan {
   int32_t q_begin, q_rows, kv_row_begin, kv_tokens, live_at;

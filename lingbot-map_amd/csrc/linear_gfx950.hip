@@ -1,0 +1,321 @@
+// bf16 linear layers of a transformer block for gfx950, with the elementwise work that follows
+// them fused into the store:
+//     out = epilogue(a @ w^T + bias)      a [M, K], w [N, K] (nn.Linear's weight), bf16 in and out
+//   LBM_LINEAR_BIAS            the qkv projection                (lingbot_map/layers/attention.py:413)
+//   LBM_LINEAR_BIAS_GELU       fc1 + exact (erf) GELU            (lingbot_map/layers/mlp.py:35-36)
+//   LBM_LINEAR_BIAS_RESIDUAL   proj / fc2 + LayerScale + residual: x + gamma * (a @ w^T + bias)
+//                              (attention.py:554, mlp.py:38, lingbot_map/layers/block.py:283,
+//                              lingbot_map/layers/layer_scale.py:21-22)
+// Roundings follow the sequence of separate bf16 torch ops: the linear's output is rounded to
+// bf16, then each elementwise op rounds again.
+//
+// Shapes this is written for: M about 1,000 rows per stream (one frame), K, N in 1024 .. 4096.
+// At that size a launch has only a few hundred tiles and 16-64 k-steps, so what counts is a
+// tile count that matches the 256 CUs and a short prologue, not asymptotic throughput.
+//
+// One workgroup = 8 wavefronts on a 128 x 128 tile of the output (TN = 64: 128 x 64), k-steps of
+// 128.  The product is computed transposed, C^T = W A^T with v_mfma_f32_32x32x16_bf16 (A operand
+// = 32 rows of W, B operand = 32 rows of the activations), so an accumulator register holds
+// four consecutive output columns of one row.  The eight wavefronts are two groups of four:
+// each group covers the whole tile (a wavefront owns 64 x TN / 2 of it) over its own half of
+// every k-step, which gives each SIMD two wavefronts to cover each other's LDS and barrier
+// waits without giving up the fragment reuse of the large per-wave tile; the two groups' sums
+// meet through LDS once, at the end.  Both operands are K-contiguous and travel global ->
+// registers -> LDS (rows of 128 elements padded to 272 bytes: neither the b128 fragment reads nor
+// the b128 stores put two lanes on one bank) two k-steps ahead of the multiply, the LDS stores
+// two per 16-wide slice in the shadow of the MFMAs, one workgroup barrier per k-step.  The tile
+// leaves through LDS as whole rows: 16-byte stores, and the residual is read the same way.
+#include <hip/hip_runtime.h>
+#include "lbm_internal.h"
+
+#pragma clang fp contract(off)
+
+namespace {
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
+typedef __attribute__((ext_vector_type(16))) float f32x16;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+typedef __attribute__((ext_vector_type(4))) unsigned int u32x4;
+typedef __attribute__((ext_vector_type(2))) unsigned int u32x2;
+
+constexpr int kGK = 128;         // k-step of the workgroup (64 per wave group)
+constexpr int kGStride = 136;    // bf16 per LDS row of a k-step (128 elements + 16 bytes: 272 B)
+constexpr int kGM = 128;         // activation rows per tile
+constexpr int kGThreads = 512;
+
+struct LinearArgs {
+  const unsigned short* a;       // [M, K]
+  const unsigned short* w;       // [N, K]
+  const float* bias;             // [N] or null
+  const float* gamma;            // [N] LayerScale (RESIDUAL only) or null
+  const unsigned short* res;     // [M, N] residual (RESIDUAL only)
+  unsigned short* out;           // [M, N]
+  int M, N, K;
+  int m_tiles, n_tiles;
+};
+
+__device__ __forceinline__ float round_bf16(float f) { return (float)(__bf16)f; }
+// Exact (erf) GELU as torch evaluates it in fp32, 0.5 v (1 + erf(v / sqrt 2)).  erf comes from the
+// Chebyshev fit erfc(z) = t exp(-z^2 + P(t)), t = 1 / (1 + z / 2), z >= 0 (Numerical Recipes,
+// erfcc: fractional error below 1.2e-7 for every z) - a sixth of the library erff's
+// instructions.  In the negative tail 1 + erf cancels and torch's result carries the last bits
+// of ITS erff, so there (v < -3: a few elements per thousand behind a LayerNorm) the library
+// function is called, behind a wave-uniform branch.
+__device__ __forceinline__ float gelu_erf(float v) {
+  const float x = 0.70710678118654752440f * v;
+  const float z = __builtin_fabsf(x);
+  const float t = __builtin_amdgcn_rcpf(__builtin_fmaf(0.5f, z, 1.0f));
+  float p = 0.17087277f;
+  p = __builtin_fmaf(p, t, -0.82215223f);
+  p = __builtin_fmaf(p, t, 1.48851587f);
+  p = __builtin_fmaf(p, t, -1.13520398f);
+  p = __builtin_fmaf(p, t, 0.27886807f);
+  p = __builtin_fmaf(p, t, -0.18628806f);
+  p = __builtin_fmaf(p, t, 0.09678418f);
+  p = __builtin_fmaf(p, t, 0.37409196f);
+  p = __builtin_fmaf(p, t, 1.00002368f);
+  p = __builtin_fmaf(p, t, -1.26551223f);
+  const float e = t * __builtin_amdgcn_exp2f(1.44269504088896340736f * __builtin_fmaf(-z, z, p));   // erfc(z)
+  float erf_x = 1.0f - e;
+  erf_x = x < 0.f ? -erf_x : erf_x;
+  const bool tail = v < -3.0f;
+  if (__builtin_amdgcn_ballot_w64(tail)) {
+    const float lib = erff(x);
+    erf_x = tail ? lib : erf_x;
+  }
+  return 0.5f * v * (1.0f + erf_x);
+}
+__device__ __forceinline__ float bf16_bits_to_f32(unsigned v) { return __builtin_bit_cast(float, v << 16); }
+
+// TN: output columns per tile (128 or 64); a wavefront owns 64 x (TN / 2) of the tile.
+template <int EPI, int TN>
+__global__ __launch_bounds__(kGThreads, 1) void lbm_linear_bf16_kernel(LinearArgs p) {
+  constexpr int NT = TN / 64;   // 32-column blocks of W per wavefront
+  // [buffer][k half][row][64 + pad]
+  __shared__ __attribute__((aligned(16))) unsigned short lds_a[2][kGM * kGStride];
+  __shared__ __attribute__((aligned(16))) unsigned short lds_w[2][TN * kGStride];
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int n32 = lane & 31, g = lane >> 5;
+  const int kh = wave >> 2, ws = wave & 3;    // k half of this wave's group, its sub-tile
+  // Workgroups are dealt to the 8 XCDs round-robin: an XCD keeps its own column tiles of W (read
+  // from HBM once, by it alone) and walks all row tiles of the activations with them.
+  int mt, nt;
+  {
+    const int x = blockIdx.x & 7, i = blockIdx.x >> 3;
+    if ((p.n_tiles & 7) == 0) {
+      mt = i % p.m_tiles;
+      nt = (i / p.m_tiles) * 8 + x;
+    } else {
+      mt = (int)blockIdx.x % p.m_tiles;
+      nt = (int)blockIdx.x / p.m_tiles;
+    }
+  }
+  const int m0 = mt * kGM, n0 = nt * TN;
+  const int wm = (ws & 1) * 64, wn = (ws >> 1) * (TN / 2);
+
+  // ---- staging: thread t moves the 16-byte piece (t & 15) of rows (t >> 4) + 32 j of a k-step
+  constexpr int kPassA = kGM / 32, kPassW = TN / 32;
+  const int ld_r = tid >> 4, ld_c = (tid & 15) * 8;          // ld_c: element within the 128 of the k-step
+  const unsigned short* ga[kPassA];
+  const unsigned short* gw[kPassW];
+#pragma unroll
+  for (int j = 0; j < kPassA; ++j) ga[j] = p.a + (size_t)min(m0 + ld_r + 32 * j, p.M - 1) * p.K + ld_c;   // rows past M re-read the last row
+#pragma unroll
+  for (int j = 0; j < kPassW; ++j) gw[j] = p.w + (size_t)(n0 + ld_r + 32 * j) * p.K + ld_c;
+  // Two register sets: the rows of k-step s are asked for at the top of iteration s - 2 and
+  // written into the LDS buffer at the end of iteration s - 1, so a load has two multiply
+  // phases to arrive before anything waits for it.
+  u32x4 ra0[kPassA], rw0[kPassW], ra1[kPassA], rw1[kPassW];
+  auto load_step = [&](int ks, u32x4 (&ra)[kPassA], u32x4 (&rw)[kPassW]) {
+#pragma unroll
+    for (int j = 0; j < kPassA; ++j) ra[j] = *(const u32x4*)(ga[j] + ks * kGK);
+#pragma unroll
+    for (int j = 0; j < kPassW; ++j) rw[j] = *(const u32x4*)(gw[j] + ks * kGK);
+  };
+  auto store_step = [&](int buf, const u32x4 (&ra)[kPassA], const u32x4 (&rw)[kPassW]) {
+#pragma unroll
+    for (int j = 0; j < kPassA; ++j) *(u32x4*)&lds_a[buf][(ld_r + 32 * j) * kGStride + ld_c] = ra[j];
+#pragma unroll
+    for (int j = 0; j < kPassW; ++j) *(u32x4*)&lds_w[buf][(ld_r + 32 * j) * kGStride + ld_c] = rw[j];
+  };
+
+  f32x16 acc[NT][2];   // [column block of W][row block of A]; element i: column 8 (i / 4) + 4 g + i % 4, row n32
+#pragma unroll
+  for (int a = 0; a < NT; ++a)
+#pragma unroll
+    for (int b = 0; b < 2; ++b)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) acc[a][b][i] = 0.f;
+
+  // One k-step: the fragments of 16-wide slice j + 1 are read while the MFMAs of slice j run,
+  // and the rows of the step after next (held in `ra`, `rw` since the previous iteration) go
+  // into the other LDS buffer two stores per slice, in the shadow of the MFMAs, followed by the
+  // loads that refill the set.  sched_barrier keeps the slices as written.
+  auto step = [&](int buf, u32x4 (&ra)[kPassA], u32x4 (&rw)[kPassW], bool write, int next_ks) {
+    const unsigned short* la = &lds_a[buf][kh * 64];
+    const unsigned short* lw = &lds_w[buf][kh * 64];
+    bf16x8 wf[2][NT], af[2][2];
+    auto read = [&](int k16, bf16x8 (&wfr)[NT], bf16x8 (&afr)[2]) {
+#pragma unroll
+      for (int a = 0; a < NT; ++a)
+        wfr[a] = __builtin_bit_cast(bf16x8, *(const u32x4*)&lw[(wn + a * 32 + n32) * kGStride + k16 * 16 + g * 8]);
+#pragma unroll
+      for (int b = 0; b < 2; ++b)
+        afr[b] = __builtin_bit_cast(bf16x8, *(const u32x4*)&la[(wm + b * 32 + n32) * kGStride + k16 * 16 + g * 8]);
+    };
+    read(0, wf[0], af[0]);
+#pragma unroll
+    for (int k16 = 0; k16 < 4; ++k16) {
+      if (k16 + 1 < 4) read(k16 + 1, wf[(k16 + 1) & 1], af[(k16 + 1) & 1]);
+#pragma unroll
+      for (int a = 0; a < NT; ++a)
+#pragma unroll
+        for (int b = 0; b < 2; ++b)
+          acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wf[k16 & 1][a], af[k16 & 1][b], acc[a][b], 0, 0, 0);
+      if (write) {
+        // this slice's share of the stores: the passes j with j % 4 == k16
+#pragma unroll
+        for (int j = 0; j < kPassA; ++j)
+          if ((j & 3) == k16) *(u32x4*)&lds_a[buf ^ 1][(ld_r + 32 * j) * kGStride + ld_c] = ra[j];
+#pragma unroll
+        for (int j = 0; j < kPassW; ++j)
+          if ((j & 3) == k16) *(u32x4*)&lds_w[buf ^ 1][(ld_r + 32 * j) * kGStride + ld_c] = rw[j];
+      }
+#pragma unroll
+      for (int j = 0; j < kPassA; ++j)
+        if ((j & 3) == k16) ra[j] = *(const u32x4*)(ga[j] + next_ks * kGK);
+#pragma unroll
+      for (int j = 0; j < kPassW; ++j)
+        if ((j & 3) == k16) rw[j] = *(const u32x4*)(gw[j] + next_ks * kGK);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  };
+
+  const int nk = p.K / kGK;
+  const int last = nk - 1;                       // steps past the end re-read the last one (never multiplied)
+  load_step(0, ra0, rw0);
+  load_step(min(1, last), ra1, rw1);
+  store_step(0, ra0, rw0);
+  load_step(min(2, last), ra0, rw0);
+  __syncthreads();
+  // iteration ks multiplies buffer ks & 1 and moves the set holding step ks + 1 into the other
+  // buffer, then refills that set with step ks + 3
+  for (int ks = 0; ks < nk; ks += 2) {
+    step(0, ra1, rw1, ks + 1 < nk, min(ks + 3, last));
+    __syncthreads();
+    if (ks + 1 >= nk) break;
+    step(1, ra0, rw0, ks + 2 < nk, min(ks + 4, last));
+    __syncthreads();
+  }
+
+  // ---- the two wave groups' sums meet: group 0 finishes row block 0 of every sub-tile, group 1
+  // row block 1; each parks the other's half in LDS (the operand buffers are dead)
+  float* xch = (float*)&lds_a[0][0];            // [wave][NT][16][64 lanes] floats
+  static_assert(8 * NT * 16 * 64 * 4 <= (int)sizeof(lds_a), "the exchanged halves fit the activation buffers");
+  // (selects, not indexing by kh: a run-time index would put the accumulators in scratch memory)
+  f32x16 fin[NT];
+  {
+#pragma unroll
+    for (int a = 0; a < NT; ++a)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        xch[((wave * NT + a) * 16 + i) * 64 + lane] = kh ? acc[a][0][i] : acc[a][1][i];
+        fin[a][i] = kh ? acc[a][1][i] : acc[a][0][i];
+      }
+    __syncthreads();
+    const int peer = wave ^ 4;
+#pragma unroll
+    for (int a = 0; a < NT; ++a)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) fin[a][i] += xch[((peer * NT + a) * 16 + i) * 64 + lane];
+  }
+  const int b = kh;     // the row block this wave finishes
+
+  // ---- epilogue.  In registers: + bias, round (the linear's output), GELU or LayerScale, round.
+  // Then the tile goes through LDS and leaves as whole rows.
+  constexpr int kCStride = TN + 4;   // bf16 per staged row: 8-byte writes of 32 rows hit 64 distinct banks
+  unsigned short* stage = (unsigned short*)&lds_w[0][0];
+  static_assert(kGM * kCStride * 2 <= (int)sizeof(lds_w), "the staged tile fits the weight buffers");
+#pragma unroll
+  for (int a = 0; a < NT; ++a)
+#pragma unroll
+    for (int c4 = 0; c4 < 4; ++c4) {
+      const int col = wn + a * 32 + c4 * 8 + g * 4;     // four consecutive output columns
+      f32x4 bias4 = {0.f, 0.f, 0.f, 0.f}, gamma4 = {1.f, 1.f, 1.f, 1.f};
+      if (p.bias) bias4 = *(const f32x4*)(p.bias + n0 + col);
+      if (EPI == LBM_LINEAR_BIAS_RESIDUAL && p.gamma) gamma4 = *(const f32x4*)(p.gamma + n0 + col);
+      f32x4 y;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        float v = round_bf16(fin[a][c4 * 4 + e] + bias4[e]);
+        if (EPI == LBM_LINEAR_BIAS_GELU) v = gelu_erf(v);
+        if (EPI == LBM_LINEAR_BIAS_RESIDUAL && p.gamma) v = v * gamma4[e];
+        y[e] = v;
+      }
+      *(bf16x4*)&stage[(wm + b * 32 + n32) * kCStride + col] = __builtin_convertvector(y, bf16x4);
+    }
+  __syncthreads();
+  constexpr int kPieces = TN / 8;                 // 16-byte pieces per row
+  constexpr int kRowsPerPass = kGThreads / kPieces;
+#pragma unroll
+  for (int r0 = 0; r0 < kGM; r0 += kRowsPerPass) {
+    const int r = r0 + tid / kPieces, c = (tid % kPieces) * 8;
+    const int row = m0 + r;
+    // (an 8-byte aligned read of the padded row: two halves)
+    const u32x2 lo = *(const u32x2*)&stage[r * kCStride + c], hi = *(const u32x2*)&stage[r * kCStride + c + 4];
+    u32x4 v = {lo[0], lo[1], hi[0], hi[1]};
+    if (row < p.M) {
+      unsigned short* dst = p.out + (size_t)row * p.N + n0 + c;
+      if (EPI == LBM_LINEAR_BIAS_RESIDUAL) {
+        const u32x4 x = *(const u32x4*)(p.res + (size_t)row * p.N + n0 + c);
+        u32x4 o;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const float s0 = bf16_bits_to_f32(x[e] & 0xffffu) + bf16_bits_to_f32(v[e] & 0xffffu);
+          const float s1 = bf16_bits_to_f32(x[e] >> 16) + bf16_bits_to_f32(v[e] >> 16);
+          o[e] = (unsigned)__builtin_bit_cast(unsigned short, (__bf16)s0) | ((unsigned)__builtin_bit_cast(unsigned short, (__bf16)s1) << 16);
+        }
+        v = o;
+      }
+      *(u32x4*)dst = v;
+    }
+  }
+}
+
+}  // namespace
+
+int lbm_launch_linear(const void* a, const void* w, const float* bias, const float* gamma, const void* residual,
+                      void* out, int M, int N, int K, int epilogue, hipStream_t stream) {
+  if (M == 0) return LBM_OK;
+  if (K % kGK != 0 || N % 64 != 0)
+    return lbm_fail(LBM_ERR_UNSUPPORTED, "lbm_linear: K must be a multiple of 128 and N of 64 (got K %d, N %d)", K, N);
+  LinearArgs p;
+  p.a = (const unsigned short*)a;
+  p.w = (const unsigned short*)w;
+  p.bias = bias;
+  p.gamma = gamma;
+  p.res = (const unsigned short*)residual;
+  p.out = (unsigned short*)out;
+  p.M = M; p.N = N; p.K = K;
+  p.m_tiles = (M + kGM - 1) / kGM;
+  // 128-column tiles when they give the 256 CUs at least most of a round of workgroups (or N
+  // does not split into 64s evenly); 64-column tiles otherwise (N = 1024 at one frame: 128 tiles
+  // of 128 x 64 instead of 64 of 128 x 128)
+  const bool wide = (N % 128 == 0) && ((long long)p.m_tiles * (N / 128) >= 160);
+  const int tn = wide ? 128 : 64;
+  p.n_tiles = N / tn;
+  const dim3 grid((unsigned)(p.m_tiles * p.n_tiles)), block(kGThreads);
+#define LBM_LINEAR_LAUNCH(E)                                                                         \
+  {                                                                                                  \
+    if (wide) hipLaunchKernelGGL((lbm_linear_bf16_kernel<E, 128>), grid, block, 0, stream, p);       \
+    else hipLaunchKernelGGL((lbm_linear_bf16_kernel<E, 64>), grid, block, 0, stream, p);             \
+  }
+  if (epilogue == LBM_LINEAR_BIAS) LBM_LINEAR_LAUNCH(LBM_LINEAR_BIAS)
+  else if (epilogue == LBM_LINEAR_BIAS_GELU) LBM_LINEAR_LAUNCH(LBM_LINEAR_BIAS_GELU)
+  else if (epilogue == LBM_LINEAR_BIAS_RESIDUAL) LBM_LINEAR_LAUNCH(LBM_LINEAR_BIAS_RESIDUAL)
+  else return lbm_fail(LBM_ERR_INVALID, "lbm_linear: unknown epilogue %d", epilogue);
+#undef LBM_LINEAR_LAUNCH
+  return lbm_check_launch("lbm_linear_bf16_kernel");
+}

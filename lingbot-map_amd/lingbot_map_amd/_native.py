@@ -12,6 +12,7 @@ OK, ERR_INVALID, ERR_UNSUPPORTED, ERR_WORKSPACE, ERR_HIP = 0, 1, 2, 3, 4
 DTYPE_BF16, DTYPE_F32 = 0, 1
 LAYOUT_TWO_STREAM, LAYOUT_FRAME_PAGES = 0, 1
 ROPE_INTERLEAVED, ROPE_HALF_SPLIT = 0, 1
+LINEAR_BIAS, LINEAR_BIAS_GELU, LINEAR_BIAS_RESIDUAL = 0, 1, 2
 MAX_STREAMS = 16
 STATIC_SCRATCH_MIB = 64
 OP_RESET, OP_ROLLBACK, OP_APPEND, OP_EVICT, OP_PLAN = 1, 2, 4, 8, 16
@@ -21,7 +22,7 @@ HDR = {"frame_count": 0, "n_anchor": 1, "win_head": 2, "win_count": 3, "n_free_p
        "n_free_special": 5, "n_special_pages": 6, "special_tokens": 7, "n_memory": 8,
        "n_memory_pages": 9, "error": 10, "plan_kv_tokens": 11, "plan_n_pages": 12}
 HDR_WORDS = 16
-ABI_VERSION = 3
+ABI_VERSION = 4
 
 
 class CacheGeom(C.Structure):
@@ -41,7 +42,7 @@ class AttnStream(C.Structure):
 
 
 SYMBOLS = ("lbm_abi_version", "lbm_last_error", "lbm_tables_words", "lbm_tables_step",
-           "lbm_rows_from_pages", "lbm_kv_append", "lbm_qkv_prepare", "lbm_residual_norm", "lbm_attn_workspace_bytes", "lbm_attn_run", "lbm_attn_run_live",
+           "lbm_rows_from_pages", "lbm_kv_append", "lbm_qkv_prepare", "lbm_residual_norm", "lbm_linear", "lbm_attn_workspace_bytes", "lbm_attn_run", "lbm_attn_run_live",
            "lbm_attn_run_static")
 
 
@@ -66,6 +67,8 @@ def _load():
     lib.lbm_qkv_prepare.argtypes = [vp, i32, vp, vp, vp, vp, C.c_float, vp, i32, vp, vp, vp, i32, vp, vp, i32, i32, i32, i32, vp]
     lib.lbm_residual_norm.restype = C.c_int
     lib.lbm_residual_norm.argtypes = [vp, vp, i32, vp, vp, vp, C.c_float, vp, vp, i32, i32, vp]
+    lib.lbm_linear.restype = C.c_int
+    lib.lbm_linear.argtypes = [vp, vp, vp, vp, vp, vp, i32, i32, i32, i32, vp]
     lib.lbm_attn_workspace_bytes.restype = C.c_size_t
     lib.lbm_attn_workspace_bytes.argtypes = [p(AttnStream), i32, i32, i32]
     lib.lbm_attn_run.restype = C.c_int

@@ -200,7 +200,45 @@ class Mlp(nn.Module):
         self.act = act_layer()
         self.fc2 = nn.Linear(hidden_features, in_features, bias=bias)
 
+    #: rows up to which the fused fc1 + GELU kernel beats the library GEMM followed by a GELU kernel
+    #: (one frame per call; at several streams' rows the library's larger tiles win)
+    FUSED_MAX_ROWS = 1280
+
+    def _can_fuse_fc1(self, x: Tensor) -> bool:
+        fc1 = self.fc1
+        return (x.is_cuda and x.dtype == torch.bfloat16 and fc1.weight.dtype == torch.bfloat16
+                and isinstance(self.act, nn.GELU) and self.act.approximate == "none"
+                and fc1.in_features % 128 == 0 and fc1.out_features % 64 == 0
+                and x.numel() // fc1.in_features <= self.FUSED_MAX_ROWS
+                and not (torch.is_grad_enabled() and (x.requires_grad or fc1.weight.requires_grad)))
+
+    def _bias_f32(self, m: nn.Linear) -> Optional[Tensor]:
+        if m.bias is None:
+            return None
+        key = (m.bias._version, m.bias.data_ptr(), m.bias.device)
+        cache = self.__dict__.setdefault("_bias_cache", {})
+        if cache.get(id(m), (None,))[0] != key:
+            cache[id(m)] = (key, m.bias.detach().float().contiguous())
+        return cache[id(m)][1]
+
+    def fc1_gelu(self, x: Tensor) -> Tensor:
+        """``act(fc1(x))`` as one kernel: the GEMM with bias and the exact GELU in its store
+        (mlp.py:35-36), roundings as the two separate bf16 torch ops."""
+        import ctypes as C
+        from . import _native as N
+        fc1 = self.fc1
+        a = x.reshape(-1, fc1.in_features).contiguous()
+        w = fc1.weight if fc1.weight.is_contiguous() else fc1.weight.contiguous()
+        bias = self._bias_f32(fc1)
+        out = torch.empty(a.shape[0], fc1.out_features, dtype=x.dtype, device=x.device)
+        p = lambda t: None if t is None else C.c_void_p(t.data_ptr())
+        N.check(N.lib.lbm_linear(p(a), p(w), p(bias), None, None, p(out), a.shape[0], fc1.out_features, fc1.in_features,
+                                 N.LINEAR_BIAS_GELU, C.c_void_p(torch.cuda.current_stream(x.device).cuda_stream)))
+        return out.reshape(*x.shape[:-1], fc1.out_features)
+
     def forward(self, x: Tensor) -> Tensor:
+        if self._can_fuse_fc1(x):
+            return self.fc2(self.fc1_gelu(x))
         return self.fc2(self.act(self.fc1(x)))
 
 

@@ -13,7 +13,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(os.path.dirname(HERE), "csrc")
 LIB_DIR = os.path.join(HERE, "_lib")
 LIB_PATH = os.path.join(LIB_DIR, "liblbm_paged_attn.so")
-SOURCES = ["c_abi.hip", "tables_gfx950.hip", "append_gfx950.hip", "qkv_prepare_gfx950.hip", "residual_norm_gfx950.hip",
+SOURCES = ["c_abi.hip", "tables_gfx950.hip", "append_gfx950.hip", "qkv_prepare_gfx950.hip", "residual_norm_gfx950.hip", "linear_gfx950.hip",
            "paged_attn_gfx950.hip"]
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [
