@@ -39,19 +39,8 @@ def run_linear(a, w, bias, epilogue, gamma=None, residual=None, out=None):
 
 
 def expected(a, w, bias, epilogue, gamma=None, residual=None):
-    N = _native()
-    bf = lambda t: t.to(torch.bfloat16).float()
-    y = a.float() @ w.float().t()
-    if bias is not None:
-        y = y + bias.float()
-    y = bf(y)
-    if epilogue == N.LINEAR_BIAS_GELU:
-        y = bf(torch.nn.functional.gelu(y))
-    if epilogue == N.LINEAR_BIAS_RESIDUAL:
-        if gamma is not None:
-            y = bf(y * gamma.float())
-        y = bf(residual.float() + y)
-    return y
+    from oracle.block_ops import linear_epilogue
+    return linear_epilogue(a, w, bias, epilogue, gamma, residual)
 
 
 def check(got, ref, scale=None, bar=2.0 ** -7):

@@ -164,3 +164,37 @@ def test_rope3d_table_hand_written_entries_and_structure():
     z = rope3d_freqs(1, 3, 4, 0)
     assert z.shape == (1, 1, 12, 32) and z[0, 0, 0].eq(1).all() and close(z[0, 0, 1 * 4 + 2][10 + 1], expect(1, 1, 22))
     assert close(z[0, 0, 1 * 4 + 2][21 + 1], expect(2, 1, 22))
+
+
+def test_linear_epilogue_closed_forms():
+    """Pins of oracle.block_ops.linear_epilogue that a dropped bias, a transposed weight, the tanh
+    approximation or a missing rounding would fail."""
+    from oracle.block_ops import LINEAR_BIAS, LINEAR_BIAS_GELU, LINEAR_BIAS_RESIDUAL, linear_epilogue
+    g = torch.Generator().manual_seed(4)
+    bf = lambda t: t.to(torch.bfloat16)
+    a = bf(torch.randn(5, 8, generator=g))
+    bias = bf(torch.randn(8, generator=g))
+    eye = bf(torch.eye(8))
+    # identity weight: the input plus the bias, rounded once
+    assert torch.equal(linear_epilogue(a, eye, bias, LINEAR_BIAS), bf(a.float() + bias.float()).float())
+    # a 3 x 2 weight against three float64 loops (w is [N, K]: out[m][n] = sum_k a[m][k] w[n][k])
+    w = bf(torch.randn(3, 8, generator=g))
+    want = torch.zeros(5, 3, dtype=torch.float64)
+    for m in range(5):
+        for n in range(3):
+            for k in range(8):
+                want[m, n] += float(a[m, k]) * float(w[n, k])
+    got = linear_epilogue(a, w, None, LINEAR_BIAS)
+    assert (got.double() - want).abs().max().item() <= 2.0 ** -8 * want.abs().max().item()
+    # exact GELU: 0 at 0, identity far right, 0 far left, odd part x / 2 + x / 2, and not the tanh form
+    x = bf(torch.tensor([[0.0, 8.0, -8.0, 1.0, -1.0, 3.0, -3.0, 0.5]]))
+    y = linear_epilogue(x, eye, None, LINEAR_BIAS_GELU)[0]
+    assert y[0].item() == 0.0 and y[1].item() == 8.0 and abs(y[2].item()) < 1e-6
+    assert abs((y[3] - y[4]).item() - 1.0) <= 2.0 ** -7 and abs((y[5] - y[6]).item() - 3.0) <= 2.0 ** -6
+    assert abs(y[3].item() - 0.8413447) <= 2.0 ** -8            # Phi(1)
+    # LayerScale + residual: gamma = 0 returns the residual, gamma = 1 the rounded sum
+    res = bf(torch.randn(5, 8, generator=g))
+    assert torch.equal(linear_epilogue(a, eye, bias, LINEAR_BIAS_RESIDUAL, torch.zeros(8), res), res.float())
+    one = linear_epilogue(a, eye, bias, LINEAR_BIAS_RESIDUAL, torch.ones(8), res)
+    assert torch.equal(one, bf(res.float() + bf(a.float() + bias.float()).float()).float())
+    assert torch.equal(linear_epilogue(a, eye, bias, LINEAR_BIAS_RESIDUAL, None, res), one)
