@@ -60,9 +60,11 @@ class PatchTrunk(nn.Module):
 
     def forward(self, images: Tensor) -> Tensor:
         x = self.conv(images)
-        for blk in self.blocks:
-            x = blk(x)
-        return self.norm(x)
+        normed = None
+        for i, blk in enumerate(self.blocks):   # each block hands the next one its norm1 (or the final norm)
+            nxt = self.blocks[i + 1].norm1 if i + 1 < len(self.blocks) else self.norm
+            x, normed = blk(x, normed=normed, next_norm=nxt)
+        return normed if len(self.blocks) else self.norm(x)
 
 
 def _first_then_rest(token: Tensor, first: Tensor) -> Tensor:
@@ -269,18 +271,36 @@ class HipAggregatorStream(nn.Module):
         scale_frames = self.num_frame_for_scale if num_frame_for_scale is None else num_frame_for_scale
         frame_idx = global_idx = 0
         outputs: List[Tensor] = []
+        # the blocks in the order they run: each one's last residual kernel also applies the norm1
+        # of the block after it, so only the first block of a call launches a LayerNorm of its own
+        order = [blocks[i] for g in range(self.aa_block_num) for kind, blocks in
+                 ((k, self.frame_blocks if k == "frame" else self.global_blocks) for k in self.aa_order)
+                 for i in range(g * self.aa_block_size, (g + 1) * self.aa_block_size)]
+        step, normed = 0, None
+
+        def run(block, tokens, normed, **kw):
+            nonlocal step
+            nxt = order[step + 1].norm1 if step + 1 < len(order) else None
+            assert order[step] is block
+            step += 1
+            if nxt is None:
+                return block(tokens, normed=normed, **kw), None
+            return block(tokens, normed=normed, next_norm=nxt, **kw)
+
         for group in range(self.aa_block_num):
             frame_out: List[Tensor] = []
             global_out: List[Tensor] = []
             for kind in self.aa_order:
                 if kind == "frame":
                     tokens = tokens.reshape(B * S, P, C)
+                    normed = normed.reshape(B * S, P, C) if normed is not None else None
                     for _ in range(self.aa_block_size):
-                        tokens = self.frame_blocks[frame_idx](tokens, pos=pos)
+                        tokens, normed = run(self.frame_blocks[frame_idx], tokens, normed, pos=pos)
                         frame_idx += 1
                         frame_out.append(tokens.view(B, S, P, C))
                 else:
                     tokens = tokens.reshape(B, S * P, C)
+                    normed = normed.reshape(B, S * P, C) if normed is not None else None
                     first_group = global_idx < self.aa_block_size
                     if self.rope3d is not None:     # frame index = frames streamed so far (stream.py:464-478)
                         if first_group:
@@ -289,8 +309,9 @@ class HipAggregatorStream(nn.Module):
                     else:
                         pos_g = pos.view(B, S * P, 2) if pos is not None else None
                     for _ in range(self.aa_block_size):
-                        tokens = self.global_blocks[global_idx](
-                            tokens, pos=pos_g, num_patches=P - self.num_special_tokens, num_special=self.num_special_tokens,
+                        tokens, normed = run(
+                            self.global_blocks[global_idx], tokens, normed,
+                            pos=pos_g, num_patches=P - self.num_special_tokens, num_special=self.num_special_tokens,
                             num_frames=S, enable_3d_rope=self.rope3d is not None, kv_cache=manager, global_idx=global_idx,
                             num_frame_per_block=num_frame_per_block, num_frame_for_scale=scale_frames,
                             num_register_tokens=self.num_register_tokens)

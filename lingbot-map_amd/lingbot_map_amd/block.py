@@ -495,12 +495,20 @@ class HipPagedBlock(nn.Module):
             C.c_void_p(torch.cuda.current_stream(x.device).cuda_stream)))
         return x_out, n_out
 
-    def _finish(self, x: Tensor, attn_out: Tensor) -> Tensor:
-        """x + ls1(attn_out), then the MLP branch (block.py:283-285)."""
+    def _finish(self, x: Tensor, attn_out: Tensor, next_norm: Optional[nn.LayerNorm] = None):
+        """x + ls1(attn_out), then the MLP branch (block.py:283-285).  With ``next_norm`` (the
+        ``norm1`` of the block that follows) returns ``(x, next_norm(x))``: the LayerNorm rides on
+        the last residual kernel instead of being a launch of its own in the next block."""
         if self._can_fuse_residual(x):
             x, n = self._residual(x, attn_out, self.ls1, self.norm2)
-            return self._residual(x, self.mlp(n), self.ls2, None)[0]
-        return self.ffn_residual(x + self.ls1(attn_out))
+            fuse_next = (next_norm is not None and type(next_norm) is nn.LayerNorm and next_norm.elementwise_affine
+                         and next_norm.bias is not None)
+            x, n_next = self._residual(x, self.mlp(n), self.ls2, next_norm if fuse_next else None)
+            if next_norm is None:
+                return x
+            return x, (n_next if fuse_next else next_norm(x))
+        x = self.ffn_residual(x + self.ls1(attn_out))
+        return x if next_norm is None else (x, next_norm(x))
 
     def attn_pre(self, x: Tensor, pos=None, enable_3d_rope: bool = False):
         """norm1 + projections + qk-norm + RoPE, ready for the cache (block.py:217-227)."""
@@ -511,21 +519,26 @@ class HipPagedBlock(nn.Module):
 
     def forward(self, x: Tensor, pos=None, num_patches=None, num_special=None, num_frames=None,
                 enable_3d_rope=False, kv_cache=None, global_idx=0, num_frame_per_block=1,
-                num_frame_for_scale=-1, num_register_tokens=4) -> Tensor:
+                num_frame_for_scale=-1, num_register_tokens=4, normed: Optional[Tensor] = None,
+                next_norm: Optional[nn.LayerNorm] = None):
+        """The reference's arguments (block.py:229-243) plus two for a caller that chains blocks:
+        ``normed`` = ``self.norm1(x)`` if the caller already has it, ``next_norm`` = the ``norm1``
+        of the block that follows; with ``next_norm`` the result is ``(x, next_norm(x))``."""
+        n1 = self.norm1(x) if normed is None else normed
         is_streaming = kv_cache is not None and (num_frames is None or num_frames <= 1)
         if is_streaming:
             if self.attn.can_fuse(kv_cache, pos, enable_3d_rope):
-                attn_x = self.attn.stream_attend_fused(kv_cache, global_idx, self.norm1(x), pos)
+                attn_x = self.attn.stream_attend_fused(kv_cache, global_idx, n1, pos)
             else:
-                q, k, v = self.attn_pre(x, pos=pos, enable_3d_rope=enable_3d_rope)
+                q, k, v = self.attn.prepare_qkv(n1, pos=pos, enable_3d_rope=enable_3d_rope)
                 attn_x = self.attn.stream_attend(kv_cache, global_idx, q, k, v, num_register_tokens)
             attn_x = attn_x.reshape(x.shape[0], x.shape[1], self.attn.num_heads * self.attn.head_dim).to(x.dtype)
-            return self._finish(x, self.attn.proj(attn_x))
+            return self._finish(x, self.attn.proj(attn_x), next_norm)
         return self._finish(x, self.attn(
-            self.norm1(x), pos=pos, num_patches=num_patches, num_special=num_special, num_frames=num_frames,
+            n1, pos=pos, num_patches=num_patches, num_special=num_special, num_frames=num_frames,
             enable_3d_rope=enable_3d_rope, kv_cache=kv_cache, global_idx=global_idx,
             num_frame_per_block=num_frame_per_block, num_frame_for_scale=num_frame_for_scale,
-            num_register_tokens=num_register_tokens))
+            num_register_tokens=num_register_tokens), next_norm)
 
 
 def keyframe_flags(num_frames: int, scale_frames: int, keyframe_interval: int):
