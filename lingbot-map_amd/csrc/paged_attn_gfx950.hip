@@ -1013,38 +1013,64 @@ __global__ __launch_bounds__(256) void lbm_attn_combine_bf16_kernel(AttnArgs a) 
   const long long split_stride = (long long)sp.q_rows * H;
   const float* lse = a.part_lse + (long long)sp.part_begin * H + rh;
   const int n = sp.n_splits;
-  // loads are issued in batches (the split count is a run-time value, a plain loop would
-  // wait for each load in turn)
-  float mx = -INFINITY;
-  for (int s0 = 0; s0 < n; s0 += 8) {
-    float t[8];
-#pragma unroll
-    for (int j = 0; j < 8; ++j) t[j] = lse[min(s0 + j, n - 1) * split_stride];
-#pragma unroll
-    for (int j = 0; j < 8; ++j) mx = fmaxf(mx, t[j]);
-  }
-  if (mx == -INFINITY) mx = 0.f;  // every split empty (no visible token): weights 0, output 0
+  const unsigned short* po = a.part_o + ((long long)sp.part_begin * H + rh) * 64 + d8 * 8;
   float wsum = 0.f;
   f32x8 acc;
 #pragma unroll
   for (int e = 0; e < 8; ++e) acc[e] = 0.f;
-  const unsigned short* po = a.part_o + ((long long)sp.part_begin * H + rh) * 64 + d8 * 8;
-  for (int s0 = 0; s0 < n; s0 += 4) {
-    float t[4];
-    bf16x8 v[4];
+  if (n <= 8) {
+    // up to eight splits (every schedule of one frame's queries): all sixteen loads - the
+    // log-sum-exps and the partial rows - are issued before the first use of any of them, one
+    // round trip of memory latency instead of three
+    float t[8];
+    bf16x8 v[8];
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const long long s = min(s0 + j, n - 1);
+    for (int j = 0; j < 8; ++j) {
+      const long long s = min(j, n - 1);
       t[j] = lse[s * split_stride];
       v[j] = *(const bf16x8*)(po + s * split_stride * 64);
     }
+    float mx = -INFINITY;
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const float w = s0 + j < n ? __builtin_amdgcn_exp2f(t[j] - mx) : 0.f;
+    for (int j = 0; j < 8; ++j) mx = fmaxf(mx, t[j]);
+    if (mx == -INFINITY) mx = 0.f;  // every split empty (no visible token): weights 0, output 0
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const float w = j < n ? __builtin_amdgcn_exp2f(t[j] - mx) : 0.f;
       const f32x8 vf = __builtin_convertvector(v[j], f32x8);
       wsum += w;
 #pragma unroll
       for (int e = 0; e < 8; ++e) acc[e] += w * vf[e];
+    }
+  } else {
+    // loads are issued in batches (the split count is a run-time value, a plain loop would
+    // wait for each load in turn)
+    float mx = -INFINITY;
+    for (int s0 = 0; s0 < n; s0 += 8) {
+      float t[8];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) t[j] = lse[min(s0 + j, n - 1) * split_stride];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) mx = fmaxf(mx, t[j]);
+    }
+    if (mx == -INFINITY) mx = 0.f;
+    for (int s0 = 0; s0 < n; s0 += 4) {
+      float t[4];
+      bf16x8 v[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const long long s = min(s0 + j, n - 1);
+        t[j] = lse[s * split_stride];
+        v[j] = *(const bf16x8*)(po + s * split_stride * 64);
+      }
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const float w = s0 + j < n ? __builtin_amdgcn_exp2f(t[j] - mx) : 0.f;
+        const f32x8 vf = __builtin_convertvector(v[j], f32x8);
+        wsum += w;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) acc[e] += w * vf[e];
+      }
     }
   }
   const float inv = wsum > 0.f ? 1.0f / wsum : 0.f;
