@@ -24,7 +24,7 @@
 extern "C" {
 #endif
 
-#define LBM_ABI_VERSION 4
+#define LBM_ABI_VERSION 5
 
 #define LBM_OK 0
 #define LBM_ERR_INVALID 1     /* bad argument (null pointer, negative size, bad enum)      */
@@ -196,6 +196,20 @@ int lbm_residual_norm(const void* x, const void* y, int32_t dtype, const float* 
 int lbm_linear(const void* a, const void* w, const float* bias, const float* gamma,
                const void* residual, void* out, int32_t M, int32_t N, int32_t K, int32_t epilogue,
                void* stream);
+
+/* The qkv projection with the fused pre-attention producer as its epilogue: lbm_linear
+ * (LBM_LINEAR_BIAS) followed by lbm_qkv_prepare on its bf16 output, as one launch - the
+ * projection's output never goes to memory.  Replaces self.qkv(x) (attention.py:413) together
+ * with everything lbm_qkv_prepare replaces.  Results are bit-identical to the two calls.
+ *   a     [M][K] bf16, w [3 * num_heads * 64][K] bf16, bias [3 * num_heads * 64] float32 or NULL
+ *   every other argument as in lbm_qkv_prepare, with bf16 activations and a bf16 cache;
+ *   head_dim is 64, K a multiple of 128. */
+int lbm_qkv_linear_prepare(const void* a, const void* w, const float* bias, int32_t M, int32_t K,
+                           const float* q_norm_w, const float* q_norm_b, const float* k_norm_w,
+                           const float* k_norm_b, float norm_eps, const float* rope_cs,
+                           int32_t rope_layout, void* q_out, void* k_out, void* v_out, void* pool,
+                           const int32_t* append_rows, int32_t num_heads, int32_t head_dim,
+                           int32_t page_size, void* stream);
 
 /* lbm_attn_run with the token counts read on the device: stream i attends to
  * live_kv_tokens[streams[i].live_at] entries of its row table instead of streams[i].kv_tokens,

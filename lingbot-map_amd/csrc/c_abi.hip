@@ -133,6 +133,25 @@ int lbm_linear(const void* a, const void* w, const float* bias, const float* gam
   return lbm_launch_linear(a, w, bias, gamma, residual, out, M, N, K, epilogue, (hipStream_t)stream);
 }
 
+int lbm_qkv_linear_prepare(const void* a, const void* w, const float* bias, int32_t M, int32_t K,
+                           const float* q_norm_w, const float* q_norm_b, const float* k_norm_w,
+                           const float* k_norm_b, float norm_eps, const float* rope_cs, int32_t rope_layout,
+                           void* q_out, void* k_out, void* v_out, void* pool, const int32_t* append_rows,
+                           int32_t num_heads, int32_t head_dim, int32_t page_size, void* stream) {
+  if (!a || !w || !q_out) return lbm_fail(LBM_ERR_INVALID, "lbm_qkv_linear_prepare: null a, w or q_out");
+  if (M < 0 || K <= 0 || num_heads <= 0) return lbm_fail(LBM_ERR_INVALID, "lbm_qkv_linear_prepare: bad shape");
+  if (head_dim != 64) return lbm_fail(LBM_ERR_UNSUPPORTED, "lbm_qkv_linear_prepare: head_dim must be 64 (got %d)", head_dim);
+  const int n_norm = (q_norm_w != nullptr) + (q_norm_b != nullptr) + (k_norm_w != nullptr) + (k_norm_b != nullptr);
+  if (n_norm != 0 && n_norm != 4) return lbm_fail(LBM_ERR_INVALID, "lbm_qkv_linear_prepare: give all four LayerNorm parameters or none");
+  if (rope_cs && rope_layout != LBM_ROPE_INTERLEAVED && rope_layout != LBM_ROPE_HALF_SPLIT)
+    return lbm_fail(LBM_ERR_INVALID, "lbm_qkv_linear_prepare: unknown rope_layout %d", rope_layout);
+  if (append_rows && !pool) return lbm_fail(LBM_ERR_INVALID, "lbm_qkv_linear_prepare: append_rows without a pool");
+  if (append_rows && page_size <= 0) return lbm_fail(LBM_ERR_INVALID, "lbm_qkv_linear_prepare: bad page_size");
+  return lbm_launch_qkv_linear_prepare(a, w, bias, M, K, q_norm_w, q_norm_b, k_norm_w, k_norm_b, norm_eps, rope_cs,
+                                       rope_layout, q_out, k_out, v_out, pool, append_rows, num_heads, page_size,
+                                       (hipStream_t)stream);
+}
+
 int lbm_residual_norm(const void* x, const void* y, int32_t dtype, const float* gamma, const float* norm_w,
                       const float* norm_b, float norm_eps, void* x_out, void* n_out, int32_t rows, int32_t cols,
                       void* stream) {

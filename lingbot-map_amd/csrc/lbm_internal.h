@@ -36,6 +36,12 @@ int lbm_launch_residual_norm(const void* x, const void* y, int dtype, const floa
 int lbm_launch_linear(const void* a, const void* w, const float* bias, const float* gamma, const void* residual,
                       void* out, int M, int N, int K, int epilogue, hipStream_t stream);
 
+int lbm_launch_qkv_linear_prepare(const void* a, const void* w, const float* bias, int M, int K,
+                                  const float* q_norm_w, const float* q_norm_b, const float* k_norm_w,
+                                  const float* k_norm_b, float norm_eps, const float* rope_cs, int rope_layout,
+                                  void* q_out, void* k_out, void* v_out, void* pool, const int32_t* append_rows,
+                                  int num_heads, int page_size, hipStream_t stream);
+
 // Split-KV schedule of one attention call, computed on the host from token counts only.
 struct LbmAttnStreamPlan {
   int32_t q_begin, q_rows, kv_row_begin, kv_tokens, live_at;

@@ -27,6 +27,7 @@
 // leaves through LDS as whole rows: 16-byte stores, and the residual is read the same way.
 #include <hip/hip_runtime.h>
 #include "lbm_internal.h"
+#include "qkv_math.h"
 
 #pragma clang fp contract(off)
 
@@ -53,7 +54,20 @@ struct LinearArgs {
   unsigned short* out;           // [M, N]
   int M, N, K;
   int m_tiles, n_tiles;
+  // LBM_LINEAR_QKV_PREPARE: the fused pre-attention producer as the epilogue of the qkv projection
+  const float* q_norm_w;         // all four null: no qk-norm
+  const float* q_norm_b;
+  const float* k_norm_w;
+  const float* k_norm_b;
+  const float* rope_cs;
+  unsigned short* k_out;         // out is q_out; k_out / v_out may be null
+  unsigned short* v_out;
+  unsigned short* pool;
+  const int32_t* append_rows;    // null: nothing is appended
+  float eps;
+  int num_heads, page_size;
 };
+constexpr int kEpiQkvPrepare = 3;   // internal: reached through lbm_qkv_linear_prepare only
 
 __device__ __forceinline__ float round_bf16(float f) { return (float)(__bf16)f; }
 // Exact (erf) GELU as torch evaluates it in fp32, 0.5 v (1 + erf(v / sqrt 2)).  erf comes from the
@@ -89,7 +103,9 @@ __device__ __forceinline__ float gelu_erf(float v) {
 __device__ __forceinline__ float bf16_bits_to_f32(unsigned v) { return __builtin_bit_cast(float, v << 16); }
 
 // TN: output columns per tile (128 or 64); a wavefront owns 64 x (TN / 2) of the tile.
-template <int EPI, int TN>
+// ROPE / NORM: rotary layout (0 none, 1 interleaved, 2 half-split) and qk-LayerNorm of the
+// kEpiQkvPrepare epilogue; 0 / false otherwise.
+template <int EPI, int TN, int ROPE = 0, bool NORM = false>
 __global__ __launch_bounds__(kGThreads, 1) void lbm_linear_bf16_kernel(LinearArgs p) {
   constexpr int NT = TN / 64;   // 32-column blocks of W per wavefront
   // [buffer][k half][row][64 + pad]
@@ -259,6 +275,63 @@ __global__ __launch_bounds__(kGThreads, 1) void lbm_linear_bf16_kernel(LinearArg
   __syncthreads();
   constexpr int kPieces = TN / 8;                 // 16-byte pieces per row
   constexpr int kRowsPerPass = kGThreads / kPieces;
+  if (EPI == kEpiQkvPrepare) {
+    // The staged tile holds the projection's output rounded to bf16, 8 consecutive columns per
+    // thread: exactly the producer's layout (8 lanes per (token, q|k|v, head) row of 64), so its
+    // LayerNorm, rotary embedding and scatter run here instead of in a pass of their own
+    // (lingbot_map/layers/attention.py:402-426, rope.py:438-461, flashinfer_cache.py:215-218).
+    const int H = p.num_heads;
+    const int c = (tid % kPieces) * 8;
+    const int col = n0 + c;                       // column of the projection: [q|k|v][head][64]
+    const int which = col / (H * 64);             // uniform over the workgroup (H * 64 is a multiple of TN)
+    const int h = (col - which * H * 64) >> 6;
+    const int c8 = (col & 63) >> 3;               // = tid % 8: the lane's place in its row of 64
+    typedef lbm_qkv::f32x4 qf4;
+    qf4 w4[2] = {}, b4[2] = {};
+    if (NORM && which < 2) {
+      const qf4* wp = (const qf4*)((which == 0 ? p.q_norm_w : p.k_norm_w) + c8 * 8);
+      const qf4* bp = (const qf4*)((which == 0 ? p.q_norm_b : p.k_norm_b) + c8 * 8);
+      w4[0] = wp[0]; w4[1] = wp[1];
+      b4[0] = bp[0]; b4[1] = bp[1];
+    }
+    unsigned short* dst_plain = which == 0 ? p.out : (which == 1 ? p.k_out : p.v_out);
+#pragma unroll
+    for (int r0 = 0; r0 < kGM; r0 += kRowsPerPass) {
+      const int r = r0 + tid / kPieces;
+      const int t = min(m0 + r, p.M - 1);         // rows past M compute on (and never store) the last token's entries
+      const bool valid = m0 + r < p.M;
+      qf4 cs4[4] = {};
+      if (ROPE == 1 && which < 2) {
+        const qf4* cs = (const qf4*)(p.rope_cs + ((long long)t * 32 + c8 * 4) * 2);
+        cs4[0] = cs[0]; cs4[1] = cs[1];
+      } else if (ROPE == 2 && which < 2) {
+        const qf4* cs = (const qf4*)(p.rope_cs + ((long long)t * 64 + c8 * 8) * 2);
+        cs4[0] = cs[0]; cs4[1] = cs[1]; cs4[2] = cs[2]; cs4[3] = cs[3];
+      }
+      int pool_row = -1;
+      if (which > 0 && p.append_rows) pool_row = p.append_rows[t];
+      const u32x2 lo = *(const u32x2*)&stage[r * kCStride + c], hi = *(const u32x2*)&stage[r * kCStride + c + 4];
+      const u32x4 raw = {lo[0], lo[1], hi[0], hi[1]};
+      float x[8];
+#pragma unroll
+      for (int i = 0; i < 8; ++i) x[i] = __builtin_bit_cast(float, (i & 1) ? (raw[i >> 1] & 0xffff0000u) : (raw[i >> 1] << 16));
+      if (which < 2) lbm_qkv::norm_rope<0, ROPE, NORM>(x, w4, b4, cs4, c8, p.eps);
+      bf16x8 o8;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) o8[i] = (__bf16)x[i];
+      if (valid) {
+        const long long nhd = ((long long)(m0 + r) * H + h) * 64 + c8 * 8;
+        if (dst_plain) *(bf16x8*)(dst_plain + nhd) = o8;
+        if (which > 0 && pool_row >= 0) {
+          const long long row_elems = (long long)H * 64;
+          const long long d = (long long)pool_row * row_elems + (which == 2 ? (long long)p.page_size * row_elems : 0) +
+                              h * 64 + c8 * 8;
+          *(bf16x8*)(p.pool + d) = o8;
+        }
+      }
+    }
+    return;
+  }
 #pragma unroll
   for (int r0 = 0; r0 < kGM; r0 += kRowsPerPass) {
     const int r = r0 + tid / kPieces, c = (tid % kPieces) * 8;
@@ -286,12 +359,25 @@ __global__ __launch_bounds__(kGThreads, 1) void lbm_linear_bf16_kernel(LinearArg
 
 }  // namespace
 
+namespace {
+// tile width: 128 columns when that gives the 256 CUs at least most of a round of workgroups (and
+// N splits into 128s), 64 otherwise (N = 1024 at one frame: 128 tiles of 128 x 64 instead of 64
+// of 128 x 128)
+int lbm_linear_tiles(LinearArgs& p) {
+  p.m_tiles = (p.M + kGM - 1) / kGM;
+  const bool wide = (p.N % 128 == 0) && ((long long)p.m_tiles * (p.N / 128) >= 160);
+  const int tn = wide ? 128 : 64;
+  p.n_tiles = p.N / tn;
+  return tn;
+}
+}  // namespace
+
 int lbm_launch_linear(const void* a, const void* w, const float* bias, const float* gamma, const void* residual,
                       void* out, int M, int N, int K, int epilogue, hipStream_t stream) {
   if (M == 0) return LBM_OK;
   if (K % kGK != 0 || N % 64 != 0)
     return lbm_fail(LBM_ERR_UNSUPPORTED, "lbm_linear: K must be a multiple of 128 and N of 64 (got K %d, N %d)", K, N);
-  LinearArgs p;
+  LinearArgs p = {};
   p.a = (const unsigned short*)a;
   p.w = (const unsigned short*)w;
   p.bias = bias;
@@ -299,13 +385,7 @@ int lbm_launch_linear(const void* a, const void* w, const float* bias, const flo
   p.res = (const unsigned short*)residual;
   p.out = (unsigned short*)out;
   p.M = M; p.N = N; p.K = K;
-  p.m_tiles = (M + kGM - 1) / kGM;
-  // 128-column tiles when they give the 256 CUs at least most of a round of workgroups (or N
-  // does not split into 64s evenly); 64-column tiles otherwise (N = 1024 at one frame: 128 tiles
-  // of 128 x 64 instead of 64 of 128 x 128)
-  const bool wide = (N % 128 == 0) && ((long long)p.m_tiles * (N / 128) >= 160);
-  const int tn = wide ? 128 : 64;
-  p.n_tiles = N / tn;
+  const bool wide = lbm_linear_tiles(p) == 128;
   const dim3 grid((unsigned)(p.m_tiles * p.n_tiles)), block(kGThreads);
 #define LBM_LINEAR_LAUNCH(E)                                                                         \
   {                                                                                                  \
@@ -318,4 +398,49 @@ int lbm_launch_linear(const void* a, const void* w, const float* bias, const flo
   else return lbm_fail(LBM_ERR_INVALID, "lbm_linear: unknown epilogue %d", epilogue);
 #undef LBM_LINEAR_LAUNCH
   return lbm_check_launch("lbm_linear_bf16_kernel");
+}
+
+int lbm_launch_qkv_linear_prepare(const void* a, const void* w, const float* bias, int M, int K,
+                                  const float* q_norm_w, const float* q_norm_b, const float* k_norm_w,
+                                  const float* k_norm_b, float norm_eps, const float* rope_cs, int rope_layout,
+                                  void* q_out, void* k_out, void* v_out, void* pool, const int32_t* append_rows,
+                                  int num_heads, int page_size, hipStream_t stream) {
+  if (M == 0) return LBM_OK;
+  const int N = 3 * num_heads * 64;
+  if (K % kGK != 0) return lbm_fail(LBM_ERR_UNSUPPORTED, "lbm_qkv_linear_prepare: K must be a multiple of 128 (got %d)", K);
+  LinearArgs p = {};
+  p.a = (const unsigned short*)a;
+  p.w = (const unsigned short*)w;
+  p.bias = bias;
+  p.out = (unsigned short*)q_out;
+  p.M = M; p.N = N; p.K = K;
+  p.q_norm_w = q_norm_w; p.q_norm_b = q_norm_b; p.k_norm_w = k_norm_w; p.k_norm_b = k_norm_b;
+  p.rope_cs = rope_cs;
+  p.k_out = (unsigned short*)k_out; p.v_out = (unsigned short*)v_out;
+  p.pool = (unsigned short*)pool;
+  p.append_rows = append_rows;
+  p.eps = norm_eps;
+  p.num_heads = num_heads; p.page_size = page_size;
+  // a tile must not straddle q | k | v: 128-wide tiles need an even number of heads
+  bool wide = lbm_linear_tiles(p) == 128;
+  if (wide && (num_heads & 1)) {
+    wide = false;
+    p.n_tiles = N / 64;
+  }
+  const dim3 grid((unsigned)(p.m_tiles * p.n_tiles)), block(kGThreads);
+  const int rope = !rope_cs ? 0 : (rope_layout == LBM_ROPE_INTERLEAVED ? 1 : 2);
+  const bool norm = q_norm_w != nullptr;
+#define LBM_QKV_LAUNCH(R, NRM)                                                                                        \
+  {                                                                                                                   \
+    if (wide) hipLaunchKernelGGL((lbm_linear_bf16_kernel<kEpiQkvPrepare, 128, R, NRM>), grid, block, 0, stream, p);   \
+    else hipLaunchKernelGGL((lbm_linear_bf16_kernel<kEpiQkvPrepare, 64, R, NRM>), grid, block, 0, stream, p);         \
+  }
+  if (rope == 0 && !norm) LBM_QKV_LAUNCH(0, false)
+  else if (rope == 0) LBM_QKV_LAUNCH(0, true)
+  else if (rope == 1 && !norm) LBM_QKV_LAUNCH(1, false)
+  else if (rope == 1) LBM_QKV_LAUNCH(1, true)
+  else if (!norm) LBM_QKV_LAUNCH(2, false)
+  else LBM_QKV_LAUNCH(2, true)
+#undef LBM_QKV_LAUNCH
+  return lbm_check_launch("lbm_linear_bf16_kernel<qkv prepare>");
 }

@@ -1,0 +1,106 @@
+// Arithmetic shared by the fused pre-attention producer (qkv_prepare_gfx950.hip) and the qkv
+// projection that carries the producer as its epilogue (linear_gfx950.hip): per-head LayerNorm
+// and rotary embedding of one q or k row of 64 elements held by 8 consecutive lanes, 8 elements
+// each (lingbot_map/layers/attention.py:402-426, lingbot_map/layers/rope.py:123-198,438-461).
+// Compiled with floating-point contraction off: every product and sum is rounded on its own, as
+// the reference's separate torch ops are.
+#ifndef LBM_QKV_MATH_H
+#define LBM_QKV_MATH_H
+
+#include <hip/hip_runtime.h>
+
+#pragma clang fp contract(off)
+
+namespace lbm_qkv {
+
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+
+// (the math header's __fmul_rn / __fadd_rn are plain operators compiled with contraction allowed)
+__device__ __forceinline__ float mul_rn(float a, float b) { return a * b; }
+__device__ __forceinline__ float add_rn(float a, float b) { return a + b; }
+__device__ __forceinline__ float sub_rn(float a, float b) { return a - b; }
+// round-to-nearest-even to bf16 and back (torch's .to(bfloat16)); the hardware conversion
+// v_cvt_pk_bf16_f32 rounds the same way
+__device__ __forceinline__ float round_bf16(float f) { return (float)(__bf16)f; }
+
+// x: this lane's elements 8 c .. 8 c + 7 of the row (c = lane % 8; the row's 8 lanes are
+// consecutive and aligned, so the shuffles below stay inside it).  SRC 0: bf16 activations
+// (roundings after the LayerNorm, of cos and sin, and after every product and sum), 1: fp32.
+// ROPE 0 none, 1 interleaved pairs (cs4[0..1] = (cos, sin) of this lane's four pairs), 2
+// half-split pairs (cs4[0..3] = (cos, sin) of its eight elements).  w4 / b4: LayerNorm weight
+// and bias of the lane's eight elements.
+template <int SRC, int ROPE, bool NORM>
+__device__ __forceinline__ void norm_rope(float (&x)[8], const f32x4 (&w4)[2], const f32x4 (&b4)[2],
+                                          const f32x4 (&cs4)[4], int c, float eps) {
+  if (NORM) {
+    float s = 0.f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) s += x[i];
+    s += __shfl_xor(s, 1);
+    s += __shfl_xor(s, 2);
+    s += __shfl_xor(s, 4);
+    const float mean = s * (1.0f / 64.0f);
+    float v = 0.f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) v += (x[i] - mean) * (x[i] - mean);
+    v += __shfl_xor(v, 1);
+    v += __shfl_xor(v, 2);
+    v += __shfl_xor(v, 4);
+    const float rstd = __builtin_amdgcn_rsqf(v * (1.0f / 64.0f) + eps);  // torch's LayerNorm uses rsqrt too
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const float y = add_rn(mul_rn(mul_rn(x[i] - mean, rstd), w4[i >> 2][i & 3]), b4[i >> 2][i & 3]);
+      x[i] = SRC == 0 ? round_bf16(y) : y;
+    }
+  }
+  if (ROPE == 1) {
+#pragma unroll
+    for (int p = 0; p < 2; ++p) {
+      const f32x4 q4 = cs4[p];  // (cos, sin) of two pairs
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        const int i = 4 * p + 2 * j;
+        float co = q4[2 * j], si = q4[2 * j + 1];
+        const float x1 = x[i], x2 = x[i + 1];
+        if (SRC == 0) {
+          co = round_bf16(co);
+          si = round_bf16(si);
+          x[i] = round_bf16(sub_rn(round_bf16(mul_rn(x1, co)), round_bf16(mul_rn(x2, si))));
+          x[i + 1] = round_bf16(add_rn(round_bf16(mul_rn(x1, si)), round_bf16(mul_rn(x2, co))));
+        } else {
+          x[i] = sub_rn(mul_rn(x1, co), mul_rn(x2, si));
+          x[i + 1] = add_rn(mul_rn(x1, si), mul_rn(x2, co));
+        }
+      }
+    }
+  } else if (ROPE != 0) {
+    // half-split pairs: in each 32-element half, element j < 16 rotates with element j + 16
+    // (x * cos + rotate(x) * sin with rotate = (-second, first), rope.py:123-152); the partner
+    // sits two lanes away in the 8-lane group
+    const bool first = (c & 2) == 0;
+#pragma unroll
+    for (int p = 0; p < 4; ++p) {
+      const f32x4 q4 = cs4[p];  // (cos, sin) of two elements
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        const int i = 2 * p + j;
+        float co = q4[2 * j], si = q4[2 * j + 1];
+        const float own = x[i];
+        const float other = __shfl_xor(own, 2);
+        if (SRC == 0) {
+          co = round_bf16(co);
+          si = round_bf16(si);
+          const float a0 = round_bf16(mul_rn(own, co)), b0 = round_bf16(mul_rn(other, si));
+          x[i] = round_bf16(first ? sub_rn(a0, b0) : add_rn(a0, b0));
+        } else {
+          const float a0 = mul_rn(own, co), b0 = mul_rn(other, si);
+          x[i] = first ? sub_rn(a0, b0) : add_rn(a0, b0);
+        }
+      }
+    }
+  }
+}
+
+}  // namespace lbm_qkv
+
+#endif  // LBM_QKV_MATH_H

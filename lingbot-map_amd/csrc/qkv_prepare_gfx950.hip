@@ -25,18 +25,13 @@
 // (the compiler fuses them into FMAs), so the kernel uses its own, defined under this pragma.
 #pragma clang fp contract(off)
 
+#include "qkv_math.h"
+
 typedef __attribute__((ext_vector_type(4))) unsigned int u32x4;
 typedef __attribute__((ext_vector_type(4))) float f32x4;
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 
 namespace {
-
-// round-to-nearest-even to bf16 and back (torch's .to(bfloat16)); the hardware conversion
-// v_cvt_pk_bf16_f32 rounds the same way
-__device__ __forceinline__ float mul_rn(float a, float b) { return a * b; }
-__device__ __forceinline__ float add_rn(float a, float b) { return a + b; }
-__device__ __forceinline__ float sub_rn(float a, float b) { return a - b; }
-__device__ __forceinline__ float round_bf16(float f) { return (float)(__bf16)f; }
 
 template <int DT>  // 0 = bf16, 1 = f32
 __device__ __forceinline__ void load8(const void* base, long long elem, float (&x)[8]) {
@@ -164,75 +159,7 @@ __global__ __launch_bounds__(256) void lbm_qkv_prepare_d64_kernel(PrepareArgs a)
 
   // q and k rows: LayerNorm and rotary embedding
 #pragma unroll
-  for (int w = 0; w < 2; ++w) {
-    if (has_norm) {
-      float s = 0.f;
-#pragma unroll
-      for (int i = 0; i < 8; ++i) s += x[w][i];
-      s += __shfl_xor(s, 1);
-      s += __shfl_xor(s, 2);
-      s += __shfl_xor(s, 4);
-      const float mean = s * (1.0f / 64.0f);
-      float v = 0.f;
-#pragma unroll
-      for (int i = 0; i < 8; ++i) v += (x[w][i] - mean) * (x[w][i] - mean);
-      v += __shfl_xor(v, 1);
-      v += __shfl_xor(v, 2);
-      v += __shfl_xor(v, 4);
-      const float rstd = __builtin_amdgcn_rsqf(v * (1.0f / 64.0f) + a.eps);  // torch's LayerNorm uses rsqrt too
-#pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        const float y = add_rn(mul_rn(mul_rn(x[w][i] - mean, rstd), w4[w][i >> 2][i & 3]), b4[w][i >> 2][i & 3]);
-        x[w][i] = SRC == 0 ? round_bf16(y) : y;
-      }
-    }
-    if (interleaved) {
-#pragma unroll
-      for (int p = 0; p < 2; ++p) {
-        const f32x4 q4 = cs4[p];  // (cos, sin) of two pairs
-#pragma unroll
-        for (int j = 0; j < 2; ++j) {
-          const int i = 4 * p + 2 * j;
-          float co = q4[2 * j], si = q4[2 * j + 1];
-          const float x1 = x[w][i], x2 = x[w][i + 1];
-          if (SRC == 0) {
-            co = round_bf16(co);
-            si = round_bf16(si);
-            x[w][i] = round_bf16(sub_rn(round_bf16(mul_rn(x1, co)), round_bf16(mul_rn(x2, si))));
-            x[w][i + 1] = round_bf16(add_rn(round_bf16(mul_rn(x1, si)), round_bf16(mul_rn(x2, co))));
-          } else {
-            x[w][i] = sub_rn(mul_rn(x1, co), mul_rn(x2, si));
-            x[w][i + 1] = add_rn(mul_rn(x1, si), mul_rn(x2, co));
-          }
-        }
-      }
-    } else if (has_rope) {
-      // half-split pairs: in each 32-element half, element j < 16 rotates with element j + 16
-      // (x * cos + rotate(x) * sin with rotate = (-second, first), rope.py:123-152); the partner
-      // sits two lanes away in the 8-lane group
-      const bool first = (c & 2) == 0;
-#pragma unroll
-      for (int p = 0; p < 4; ++p) {
-        const f32x4 q4 = cs4[p];  // (cos, sin) of two elements
-#pragma unroll
-        for (int j = 0; j < 2; ++j) {
-          const int i = 2 * p + j;
-          float co = q4[2 * j], si = q4[2 * j + 1];
-          const float own = x[w][i];
-          const float other = __shfl_xor(own, 2);
-          if (SRC == 0) {
-            co = round_bf16(co);
-            si = round_bf16(si);
-            const float a0 = round_bf16(mul_rn(own, co)), b0 = round_bf16(mul_rn(other, si));
-            x[w][i] = round_bf16(first ? sub_rn(a0, b0) : add_rn(a0, b0));
-          } else {
-            const float a0 = mul_rn(own, co), b0 = mul_rn(other, si);
-            x[w][i] = first ? sub_rn(a0, b0) : add_rn(a0, b0);
-          }
-        }
-      }
-    }
-  }
+  for (int w = 0; w < 2; ++w) lbm_qkv::norm_rope<SRC, ROPE, NORM>(x[w], w4[w], b4[w], cs4, c, a.eps);
 
   const long long nhd = ((long long)t * H + h) * 64 + c * 8;
   store8<DST>(a.q_out, nhd, x[0]);

@@ -338,7 +338,8 @@ class HipPagedAttention(nn.Module):
         """qkv projection, then one kernel for q/k LayerNorm + rotary embedding + layout +
         paged append, then the paged attention (attention.py:402-426 and block.py:256-278)."""
         B, N, _ = x.shape
-        qkv = self.qkv(x).reshape(B * N, -1)
+        proj = self._fused_projection(x, manager.dtype)
+        qkv = None if proj is not None else self.qkv(x).reshape(B * N, -1)
         has_norm = isinstance(self.q_norm, nn.LayerNorm)
         rope_cs = None
         if self.rope is not None:
@@ -350,7 +351,31 @@ class HipPagedAttention(nn.Module):
                                 self._norm_f32(self.k_norm) if has_norm else None, rope_cs,
                                 norm_eps=self.q_norm.eps if has_norm else 1e-5, keyframe=None,
                                 cross_frame_special=self.kv_cache_cross_frame_special,
-                                camera_only=self.kv_cache_camera_only)
+                                camera_only=self.kv_cache_camera_only, proj=proj)
+
+    #: rows up to which the projection with the producer as its epilogue is used (one frame per
+    #: call; at several streams' rows the library GEMM's larger tiles win)
+    FUSED_PROJ_MAX_ROWS = 1280
+
+    def _fused_projection(self, x: Tensor, cache_dtype) -> Optional[tuple]:
+        """(x [rows, K], weight, float32 bias) for ``lbm_qkv_linear_prepare`` when the projection
+        can run in the producer's kernel: bf16 activations, weights and cache, head_dim 64, K a
+        multiple of 128, one frame's worth of rows; None otherwise (the caller projects first)."""
+        w = self.qkv.weight
+        rows = x.numel() // x.shape[-1]
+        if not (x.is_cuda and x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and cache_dtype == torch.bfloat16
+                and self.head_dim == 64 and x.shape[-1] % 128 == 0 and rows <= self.FUSED_PROJ_MAX_ROWS
+                and not (torch.is_grad_enabled() and (x.requires_grad or w.requires_grad))):
+            return None
+        bias = None
+        if self.qkv.bias is not None:
+            b = self.qkv.bias
+            key = (b._version, b.data_ptr(), b.device)
+            hit = self.__dict__.get("_qkv_bias_f32")
+            if hit is None or hit[0] != key:
+                hit = self.__dict__["_qkv_bias_f32"] = (key, b.detach().float().contiguous())
+            bias = hit[1]
+        return x.reshape(rows, x.shape[-1]).contiguous(), (w if w.is_contiguous() else w.contiguous()), bias
 
     def can_fuse_dense(self, x: Tensor, pos, enable_3d_rope: bool) -> bool:
         """Whether the cache-less attention of a batch of frames can run as fused producer +
@@ -379,7 +404,8 @@ class HipPagedAttention(nn.Module):
         from .dense import dense_attention
         B, n, _ = x.shape
         H, D = self.num_heads, self.head_dim
-        qkv = self.qkv(x).reshape(B * n, -1).contiguous()
+        proj = self._fused_projection(x, x.dtype)
+        qkv = None if proj is not None else self.qkv(x).reshape(B * n, -1).contiguous()
         has_norm = isinstance(self.q_norm, nn.LayerNorm)
         norm = (self._norm_f32(self.q_norm) + self._norm_f32(self.k_norm)) if has_norm else (None,) * 4
         table, layout = None, N.ROPE_INTERLEAVED
@@ -396,10 +422,16 @@ class HipPagedAttention(nn.Module):
         q, k, v = (torch.empty(B * n, H, D, dtype=x.dtype, device=x.device) for _ in range(3))
         p = lambda t: None if t is None else C.c_void_p(t.data_ptr())
         dt = N.DTYPE_BF16 if x.dtype == torch.bfloat16 else N.DTYPE_F32
-        N.check(N.lib.lbm_qkv_prepare(
-            p(qkv), dt, p(norm[0]), p(norm[1]), p(norm[2]), p(norm[3]),
-            float(self.q_norm.eps) if has_norm else 1e-5, p(table), layout, p(q), p(k), p(v), dt, None, None,
-            B * n, H, D, 16, C.c_void_p(torch.cuda.current_stream(x.device).cuda_stream)))
+        eps = float(self.q_norm.eps) if has_norm else 1e-5
+        stream = C.c_void_p(torch.cuda.current_stream(x.device).cuda_stream)
+        if proj is not None:
+            N.check(N.lib.lbm_qkv_linear_prepare(
+                p(proj[0]), p(proj[1]), p(proj[2]), B * n, proj[0].shape[1], p(norm[0]), p(norm[1]), p(norm[2]), p(norm[3]),
+                eps, p(table), layout, p(q), p(k), p(v), None, None, H, D, 16, stream))
+        else:
+            N.check(N.lib.lbm_qkv_prepare(
+                p(qkv), dt, p(norm[0]), p(norm[1]), p(norm[2]), p(norm[3]), eps, p(table), layout, p(q), p(k), p(v), dt,
+                None, None, B * n, H, D, 16, stream))
         return dense_attention(q, k, v, num_streams=B).reshape(B, n, H * D)
 
     def forward(self, x: Tensor, pos=None, num_patches=None, num_special=None, num_frames=None,

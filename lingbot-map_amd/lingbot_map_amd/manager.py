@@ -458,23 +458,36 @@ class HipPagedKVCacheManager:
             self._n_appends[block_idx] += 1
         return self._attend_planned(block_idx, q, k if any(tail) else None, v if any(tail) else None)
 
-    def step_qkv(self, block_idx: int, qkv: Tensor, q_norm=None, k_norm=None, rope_cs: Optional[Tensor] = None,
+    def step_qkv(self, block_idx: int, qkv: Optional[Tensor], q_norm=None, k_norm=None, rope_cs: Optional[Tensor] = None,
                  norm_eps: float = 1e-5, keyframe: Optional[Sequence[bool]] = None,
-                 cross_frame_special: bool = True, camera_only: bool = False) -> Tensor:
+                 cross_frame_special: bool = True, camera_only: bool = False, proj=None) -> Tensor:
         """`step` fed with the output of the qkv projection instead of finished q, k, v: one
         kernel applies the per-head LayerNorm of q and k, the rotary embedding, lays q out as
         [token, head, dim] and writes k and v straight into the page pool (attention.py:402-426
         plus append_frame).  ``qkv``: [streams * tokens_per_frame, 3 * heads * head_dim];
         ``q_norm`` / ``k_norm``: (weight, bias) float32 tensors of [head_dim] or None;
         ``rope_cs``: float32 [streams * tokens_per_frame, head_dim / 2, 2] holding (cos, sin),
-        i.e. ``torch.view_as_real`` of the reference's complex ``freqs``, or None."""
+        i.e. ``torch.view_as_real`` of the reference's complex ``freqs``, or None.
+
+        ``proj = (x, weight, bias)`` instead of ``qkv`` (then None): the projection itself runs in
+        the same kernel (``x`` [rows, K] bf16, ``weight`` [3 * heads * head_dim, K] bf16, ``bias``
+        float32 or None; bf16 cache, head_dim 64) and its output never goes to memory; the results
+        are bit-identical to projecting first."""
         rows, H, D = self.num_streams * self.tokens_per_frame, self.num_heads, self.head_dim
-        assert qkv.shape[0] == rows and qkv.numel() == rows * 3 * H * D, (
-            f"qkv: expected [{rows}, {3 * H * D}], got {tuple(qkv.shape)}")
+        if proj is None:
+            assert qkv.shape[0] == rows and qkv.numel() == rows * 3 * H * D, (
+                f"qkv: expected [{rows}, {3 * H * D}], got {tuple(qkv.shape)}")
+            if qkv.dtype not in (torch.bfloat16, torch.float32):
+                qkv = qkv.to(self.dtype)
+            qkv = qkv.contiguous()
+        else:
+            px, pw, pb = proj
+            assert qkv is None and self.dtype == torch.bfloat16 and D == 64, "proj: bf16 cache with head_dim 64"
+            assert px.dtype == pw.dtype == torch.bfloat16 and px.is_contiguous() and pw.is_contiguous()
+            assert px.shape[0] == rows and pw.shape == (3 * H * D, px.shape[1]) and px.shape[1] % 128 == 0, (
+                f"proj: x [{rows}, K] and weight [{3 * H * D}, K] with K a multiple of 128, got {tuple(px.shape)}, {tuple(pw.shape)}")
+            assert pb is None or (pb.dtype == torch.float32 and pb.numel() == 3 * H * D)
         assert (q_norm is None) == (k_norm is None), "q_norm and k_norm go together"
-        if qkv.dtype not in (torch.bfloat16, torch.float32):
-            qkv = qkv.to(self.dtype)
-        qkv = qkv.contiguous()
         ts, keyframe, tail = self._step_tables(block_idx, keyframe, cross_frame_special, camera_only)
         q = torch.empty(rows, H, D, dtype=self.dtype, device=self.device)
         k = torch.empty_like(q) if any(tail) else None
@@ -487,15 +500,19 @@ class HipPagedKVCacheManager:
                 f"rope_cs: expected float32 [{rows}, {D // 2}, 2], got {rope_cs.dtype} {tuple(rope_cs.shape)}")
             rope_cs = rope_cs.contiguous()
         dt = lambda d: N.DTYPE_BF16 if d == torch.bfloat16 else N.DTYPE_F32
-        N.check(N.lib.lbm_qkv_prepare(
-            C.c_void_p(qkv.data_ptr()), dt(qkv.dtype),
-            norm_ptr[0], norm_ptr[1], norm_ptr[2], norm_ptr[3], float(norm_eps),
-            C.c_void_p(rope_cs.data_ptr()) if rope_cs is not None else None, N.ROPE_INTERLEAVED,
-            C.c_void_p(q.data_ptr()), C.c_void_p(k.data_ptr()) if k is not None else None,
-            C.c_void_p(v.data_ptr()) if v is not None else None, dt(self.dtype),
-            C.c_void_p(self.kv_caches[block_idx].data_ptr()),
-            C.c_void_p(self._append_rows[ts].data_ptr()) if any(keyframe) else None,
-            rows, H, D, self.page_size, self._stream_handle()))
+        vp = lambda t: None if t is None else C.c_void_p(t.data_ptr())
+        rope_ptr = vp(rope_cs)
+        append_ptr = vp(self._append_rows[ts]) if any(keyframe) else None
+        if proj is None:
+            N.check(N.lib.lbm_qkv_prepare(
+                vp(qkv), dt(qkv.dtype), norm_ptr[0], norm_ptr[1], norm_ptr[2], norm_ptr[3], float(norm_eps),
+                rope_ptr, N.ROPE_INTERLEAVED, vp(q), vp(k), vp(v), dt(self.dtype),
+                vp(self.kv_caches[block_idx]), append_ptr, rows, H, D, self.page_size, self._stream_handle()))
+        else:
+            N.check(N.lib.lbm_qkv_linear_prepare(
+                vp(px), vp(pw), vp(pb), rows, px.shape[1], norm_ptr[0], norm_ptr[1], norm_ptr[2], norm_ptr[3],
+                float(norm_eps), rope_ptr, N.ROPE_INTERLEAVED, vp(q), vp(k), vp(v),
+                vp(self.kv_caches[block_idx]), append_ptr, H, D, self.page_size, self._stream_handle()))
         if any(keyframe):
             self.frame_count[block_idx] += 1
             self._n_appends[block_idx] += 1

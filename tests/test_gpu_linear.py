@@ -136,3 +136,61 @@ def test_mlp_with_fused_fc1_gelu_equals_the_unfused_module():
         assert not mlp._can_fuse_fc1(x.float())
         assert not Mlp(256, 1024, act_layer=lambda: torch.nn.GELU(approximate="tanh")).to(dev).to(torch.bfloat16)._can_fuse_fc1(x)
         assert not mlp._can_fuse_fc1(torch.zeros(4, 1004, 256, device=dev, dtype=torch.bfloat16))
+
+
+@pytest.mark.parametrize("rope", ["none", "interleaved", "half_split"])
+@pytest.mark.parametrize("norm", [False, True])
+@pytest.mark.parametrize("M,H,K", [(1004, 16, 1024), (70, 3, 128)])
+def test_qkv_projection_with_the_producer_as_its_epilogue(M, H, K, norm, rope):
+    """lbm_qkv_linear_prepare against lbm_linear (bias) followed by lbm_qkv_prepare on its output:
+    the same arithmetic on the same rounded projection, so q, k, v and the pool rows are bit-equal.
+    Keyframe-gated pool writes (some rows -1), k_out / v_out present and absent, an odd number of
+    heads (64-column tiles)."""
+    N = _native()
+    dev = torch.device("cuda:0")
+    D, S = 64, 16
+    g = torch.Generator().manual_seed(M + H + K + norm + len(rope))
+    a = torch.randn(M, K, generator=g).to(torch.bfloat16).to(dev)
+    w = (torch.randn(3 * H * D, K, generator=g) / K ** 0.5).to(torch.bfloat16).to(dev)
+    bias = (0.1 * torch.randn(3 * H * D, generator=g)).to(dev)
+    ln = [(1 + 0.2 * torch.randn(D, generator=g)).to(dev) if i % 2 == 0 else (0.1 * torch.randn(D, generator=g)).to(dev)
+          for i in range(4)] if norm else [None] * 4
+    cs, layout = None, N.ROPE_INTERLEAVED
+    if rope == "interleaved":
+        ang = torch.rand(M, D // 2, generator=g) * 6.283185
+        cs = torch.stack([ang.cos(), ang.sin()], dim=-1).contiguous().to(dev)
+    elif rope == "half_split":
+        ang = torch.rand(M, D, generator=g) * 6.283185
+        cs, layout = torch.stack([ang.cos(), ang.sin()], dim=-1).contiguous().to(dev), N.ROPE_HALF_SPLIT
+    n_pages = -(-M // S) + 3
+    rows = torch.randperm(n_pages * S, generator=g)[:M]
+    rows = ((rows // S) * 2 * S + rows % S).to(torch.int32)
+    rows[::7] = -1                                            # gated off
+    rows = rows.to(dev)
+    for with_kv, with_pool in ((True, True), (False, True), (True, False)):
+        def outputs():
+            q = torch.full((M, H, D), float("nan"), dtype=torch.bfloat16, device=dev)
+            k = torch.full_like(q, float("nan")) if with_kv else None
+            v = torch.full_like(q, float("nan")) if with_kv else None
+            pool = torch.zeros(n_pages, 2, S, H, D, dtype=torch.bfloat16, device=dev) if with_pool else None
+            return q, k, v, pool
+        q0, k0, v0, pool0 = outputs()
+        qkv = torch.empty(M, 3 * H * D, dtype=torch.bfloat16, device=dev)
+        N.check(N.lib.lbm_linear(ptr(a), ptr(w), ptr(bias), None, None, ptr(qkv), M, 3 * H * D, K, N.LINEAR_BIAS, None))
+        N.check(N.lib.lbm_qkv_prepare(ptr(qkv), N.DTYPE_BF16, *[ptr(t) for t in ln], 1e-5, ptr(cs), layout, ptr(q0), ptr(k0), ptr(v0),
+                                      N.DTYPE_BF16, ptr(pool0), ptr(rows) if with_pool else None, M, H, D, S, None))
+        q1, k1, v1, pool1 = outputs()
+        N.check(N.lib.lbm_qkv_linear_prepare(ptr(a), ptr(w), ptr(bias), M, K, *[ptr(t) for t in ln], 1e-5, ptr(cs), layout,
+                                             ptr(q1), ptr(k1), ptr(v1), ptr(pool1), ptr(rows) if with_pool else None, H, D, S, None))
+        torch.cuda.synchronize()
+        assert torch.isfinite(q1.float()).all() and torch.equal(q0, q1)
+        if with_kv:
+            assert torch.equal(k0, k1) and torch.equal(v0, v1)
+        if with_pool:
+            assert torch.equal(pool0, pool1) and pool1.float().abs().sum().item() > 0
+    # argument checks
+    bad = lambda *args: N.lib.lbm_qkv_linear_prepare(*args) != N.OK
+    q1 = torch.empty(M, H, D, dtype=torch.bfloat16, device=dev)
+    assert bad(ptr(a), ptr(w), None, M, K, None, None, None, None, 1e-5, None, 0, ptr(q1), None, None, None, None, H, 128, S, None)   # head_dim
+    assert bad(ptr(a), ptr(w), None, M, K, ptr(bias), None, None, None, 1e-5, None, 0, ptr(q1), None, None, None, None, H, D, S, None)  # one norm parameter
+    assert bad(ptr(a), ptr(w), None, M, K, None, None, None, None, 1e-5, None, 0, ptr(q1), None, None, None, ptr(rows), H, D, S, None)  # rows without pool
