@@ -217,9 +217,11 @@ __device__ __forceinline__ void lbm_attn_split(const AttnArgs& a) {
     u32x4 raw[kQPerWave / 8];
 #pragma unroll
     for (int k = 0; k < kQPerWave / 8; ++k) {
-      const int r = q_row0 + k * 8 + (lane >> 3);
-      raw[k] = u32x4{0u, 0u, 0u, 0u};
-      if (r < sp.q_rows) raw[k] = *(const u32x4*)(a.q + ((size_t)(sp.q_begin + r) * H + head) * 64 + (lane & 7) * 8);
+      // rows past the stream's last query row re-read that row: their results are never stored,
+      // and eight unconditional loads go out back to back (a load inside a conditional block
+      // ends up with a wait for everything in flight behind it)
+      const int r = max(min(q_row0 + k * 8 + (lane >> 3), sp.q_rows - 1), 0);
+      raw[k] = *(const u32x4*)(a.q + ((size_t)(sp.q_begin + r) * H + head) * 64 + (lane & 7) * 8);
     }
 #pragma unroll
     for (int k = 0; k < kQPerWave / 8; ++k)
@@ -767,9 +769,8 @@ __global__ __launch_bounds__(kSmThreads, 1) void lbm_attn_bf16_d64_small_kernel(
   bf16x8 qf[2][4];
   {
     unsigned short* patch_q = (unsigned short*)lds_raw;
-    const int r = q_row0 + (tid >> 3);
-    u32x4 raw = {0u, 0u, 0u, 0u};
-    if (r < sp.q_rows) raw = *(const u32x4*)(a.q + ((size_t)(sp.q_begin + r) * H + head) * 64 + (tid & 7) * 8);
+    const int r = max(min(q_row0 + (tid >> 3), sp.q_rows - 1), 0);   // rows past the last one re-read it (never stored)
+    const u32x4 raw = *(const u32x4*)(a.q + ((size_t)(sp.q_begin + r) * H + head) * 64 + (tid & 7) * 8);
     *(u32x4*)&patch_q[(tid >> 3) * kKStride + (tid & 7) * 8] = raw;
     __syncthreads();
 #pragma unroll
