@@ -65,7 +65,7 @@ constexpr int kKStride = 72;            // bf16 per LDS row of K: 144 B, b128 re
 constexpr int kVStride = 96;            // bf16 per LDS row of V: 192 B, 4-row transpose reads conflict-free
 constexpr float kHeadroom = 11.0f;      // the softmax reference is set this far above the row maxima (log2 units)
 
-struct AttnArgs {
+struct AttnCore {
   const unsigned short* q;
   const unsigned short* pool;
   unsigned short* out;
@@ -78,6 +78,8 @@ struct AttnArgs {
   int num_heads;
   int page_size;
   float scale_log2;
+};
+struct AttnArgs : AttnCore {
   LbmAttnSchedule sch;
 };
 
@@ -119,7 +121,9 @@ __shared__ __attribute__((aligned(16))) unsigned short lds_q[kWaves][kQPerWave *
 // The repeat pass is a function of its own, not inlined: it is entered once in a blue moon,
 // and compiled into the kernel body its registers would push the common path into scratch
 // memory (spill stores and reloads on every launch, tens of MB of HBM traffic).
-__device__ __noinline__ void lbm_attn_split_safe(AttnArgs a);
+// (it takes the 130 bytes it needs, not the whole argument block with its sixteen stream plans:
+// what is passed by value sizes the kernel's scratch frame)
+__device__ __noinline__ void lbm_attn_split_safe(AttnCore a, LbmAttnStreamPlan sp);
 
 // One workgroup's share of the split-KV attention: 512 query rows of one head over one run of
 // KV tiles, start to finish.  SAFE = false is the common path (no softmax reference, range
@@ -127,15 +131,11 @@ __device__ __noinline__ void lbm_attn_split_safe(AttnArgs a);
 // repeat pass and ends the program there, so that nothing of the common path is live across
 // the call.  SAFE = true is the repeat with a reference that follows the row maxima.
 template <bool SAFE>
-__device__ __forceinline__ void lbm_attn_split(const AttnArgs& a) {
+__device__ __forceinline__ void lbm_attn_split(const AttnCore& a, const LbmAttnStreamPlan& sp) {
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int n32 = lane & 31, g = lane >> 5;
 
-  // ---- which piece of work is this workgroup
-  int b = 0;
-  for (int i = 1; i < a.sch.n_streams; ++i)
-    if ((int)blockIdx.x >= a.sch.s[i].wg_begin) b = i;
-  const LbmAttnStreamPlan sp = a.sch.s[b];
+  // ---- which piece of this stream's work is this workgroup
   const int H = a.num_heads;
   const int local = (int)blockIdx.x - sp.wg_begin;
   const int n_hs = H * sp.n_splits;
@@ -646,7 +646,7 @@ __device__ __forceinline__ void lbm_attn_split(const AttnArgs& a) {
       }
     }
     if (!safe && __builtin_amdgcn_readfirstlane(__syncthreads_or(bad))) {
-      lbm_attn_split_safe(a);
+      lbm_attn_split_safe(a, sp);
       __builtin_amdgcn_endpgm();
     }
   }
@@ -699,12 +699,16 @@ __device__ __forceinline__ void lbm_attn_split(const AttnArgs& a) {
   }
 }
 
-__device__ __noinline__ void lbm_attn_split_safe(AttnArgs a) { lbm_attn_split<true>(a); }
+__device__ __noinline__ void lbm_attn_split_safe(AttnCore a, LbmAttnStreamPlan sp) { lbm_attn_split<true>(a, sp); }
 
 }  // namespace
 
 __global__ __launch_bounds__(kThreads, 1) void lbm_attn_bf16_d64_kernel(AttnArgs a) {
-  lbm_attn_split<false>(a);
+  int b = 0;   // which stream's work is this workgroup
+  for (int i = 1; i < a.sch.n_streams; ++i)
+    if ((int)blockIdx.x >= a.sch.s[i].wg_begin) b = i;
+  const LbmAttnStreamPlan sp = a.sch.s[b];
+  lbm_attn_split<false>(a, sp);
 }
 
 // ---------------------------------------------------------------------------- bf16, short KV
