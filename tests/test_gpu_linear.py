@@ -113,6 +113,13 @@ def test_linear_rows_past_m_are_not_written_and_arguments_are_checked():
     assert bad(ptr(ad), ptr(wd), None, None, None, ptr(o), 200, 128, 128, N.LINEAR_BIAS_RESIDUAL, None)  # no residual
     assert bad(ptr(ad), ptr(wd), None, None, ptr(o), ptr(o), 200, 128, 128, N.LINEAR_BIAS, None)    # residual without the epilogue
     assert bad(ptr(ad), ptr(wd), None, None, None, ptr(o), 200, 128, 128, 9, None)
+    # no rows: accepted, nothing written
+    o.fill_(3.0)
+    N.check(N.lib.lbm_linear(ptr(ad), ptr(wd), None, None, None, ptr(o), 0, 128, 128, N.LINEAR_BIAS, None))
+    N.check(N.lib.lbm_qkv_linear_prepare(ptr(ad), ptr(wd), None, 0, 128, None, None, None, None, 1e-5, None, 0, ptr(o), None, None,
+                                         None, None, 2, 64, 16, None))
+    torch.cuda.synchronize()
+    assert bool((o == 3.0).all())
 
 
 def test_mlp_with_fused_fc1_gelu_equals_the_unfused_module():
