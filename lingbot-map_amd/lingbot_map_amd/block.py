@@ -233,7 +233,7 @@ class Mlp(nn.Module):
         out = torch.empty(a.shape[0], fc1.out_features, dtype=x.dtype, device=x.device)
         p = lambda t: None if t is None else C.c_void_p(t.data_ptr())
         N.check(N.lib.lbm_linear(p(a), p(w), p(bias), None, None, p(out), a.shape[0], fc1.out_features, fc1.in_features,
-                                 N.LINEAR_BIAS_GELU, C.c_void_p(torch.cuda.current_stream(x.device).cuda_stream)))
+                                 N.LINEAR_BIAS_GELU, N.stream_ptr(x.device)))
         return out.reshape(*x.shape[:-1], fc1.out_features)
 
     def forward(self, x: Tensor) -> Tensor:
@@ -423,7 +423,7 @@ class HipPagedAttention(nn.Module):
         p = lambda t: None if t is None else C.c_void_p(t.data_ptr())
         dt = N.DTYPE_BF16 if x.dtype == torch.bfloat16 else N.DTYPE_F32
         eps = float(self.q_norm.eps) if has_norm else 1e-5
-        stream = C.c_void_p(torch.cuda.current_stream(x.device).cuda_stream)
+        stream = N.stream_ptr(x.device)
         if proj is not None:
             N.check(N.lib.lbm_qkv_linear_prepare(
                 p(proj[0]), p(proj[1]), p(proj[2]), B * n, proj[0].shape[1], p(norm[0]), p(norm[1]), p(norm[2]), p(norm[3]),
@@ -524,7 +524,7 @@ class HipPagedBlock(nn.Module):
         N.check(N.lib.lbm_residual_norm(
             p(x), p(y), N.DTYPE_BF16 if x.dtype == torch.bfloat16 else N.DTYPE_F32, p(gamma), p(w), p(b),
             float(norm.eps) if norm is not None else 0.0, p(x_out), p(n_out), x.numel() // x.shape[-1], x.shape[-1],
-            C.c_void_p(torch.cuda.current_stream(x.device).cuda_stream)))
+            N.stream_ptr(x.device)))
         return x_out, n_out
 
     def _finish(self, x: Tensor, attn_out: Tensor, next_norm: Optional[nn.LayerNorm] = None):

@@ -16,8 +16,8 @@ from torch import Tensor
 
 from . import _native as N
 
-_rows_cache: Dict[Tuple[int, int, str], Tensor] = {}
-_workspace: Dict[str, Tensor] = {}
+_plans: Dict[tuple, tuple] = {}          # (rows, streams, H, D, device) -> (row table, stream descriptors, workspace bytes)
+_workspace: Dict[object, Tensor] = {}
 
 
 def dense_attention(q: Tensor, k: Tensor, v: Tensor, num_streams: int = 1) -> Tensor:
@@ -32,22 +32,23 @@ def dense_attention(q: Tensor, k: Tensor, v: Tensor, num_streams: int = 1) -> Te
     assert 1 <= num_streams <= N.MAX_STREAMS and rows % num_streams == 0
     n = rows // num_streams
     q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
-    key = (rows, num_streams, str(q.device))
-    kv_rows = _rows_cache.get(key)
-    if kv_rows is None:
+    key = (rows, num_streams, H, D, q.device)
+    plan = _plans.get(key)
+    if plan is None:
         # entry -1 - r names row r of the caller's own K/V
         kv_rows = (-1 - torch.arange(rows, dtype=torch.int32)).to(q.device)
-        _rows_cache[key] = kv_rows
-    streams = (N.AttnStream * num_streams)(*[N.AttnStream(s * n, n, s * n, n) for s in range(num_streams)])
-    need = int(N.lib.lbm_attn_workspace_bytes(streams, num_streams, H, D))
-    ws = _workspace.get(str(q.device))
+        streams = (N.AttnStream * num_streams)(*[N.AttnStream(s * n, n, s * n, n) for s in range(num_streams)])
+        need = int(N.lib.lbm_attn_workspace_bytes(streams, num_streams, H, D))
+        plan = _plans[key] = (kv_rows, streams, need)
+    kv_rows, streams, need = plan
+    ws = _workspace.get(q.device)
     if ws is None or ws.numel() < max(need, 16):
         ws = torch.empty(max(int(need * 1.25), 1 << 20), dtype=torch.uint8, device=q.device)
-        _workspace[str(q.device)] = ws
+        _workspace[q.device] = ws
     out = torch.empty_like(q)
     p = lambda t: C.c_void_p(t.data_ptr())
     N.check(N.lib.lbm_attn_run(
         p(q), p(k), p(out), p(k), p(v), p(kv_rows), streams, num_streams, H, D, 16,
         N.DTYPE_BF16 if q.dtype == torch.bfloat16 else N.DTYPE_F32, 1.0 / math.sqrt(D),
-        p(ws), ws.numel(), C.c_void_p(torch.cuda.current_stream(q.device).cuda_stream)))
+        p(ws), ws.numel(), N.stream_ptr(q.device)))
     return out

@@ -187,7 +187,7 @@ class HipPagedKVCacheManager:
     # helpers
     # =========================================================================
     def _stream_handle(self):
-        return C.c_void_p(torch.cuda.current_stream(self.device).cuda_stream)
+        return N.stream_ptr(self.device)
 
     def _set(self, block_idx: int) -> int:
         return block_idx if self.per_block_tables else 0
