@@ -767,27 +767,13 @@ __global__ __launch_bounds__(kSmThreads, 1) void lbm_attn_bf16_d64_small_kernel(
   const int p0 = wave * pps, p1 = min(p0 + pps, n_pieces);   // this wavefront's pieces (possibly none)
   const unsigned row_bytes = (unsigned)H * 128u;
   const int q_row0 = qb64 * kQPerWave;
-
-  // ---- Q: the workgroup reads the 64 rows once as whole rows, every wavefront picks its
-  // fragments up from LDS; scale * log2(e) folded in (as in the main kernel)
-  bf16x8 qf[2][4];
-  {
-    unsigned short* patch_q = (unsigned short*)lds_raw;
-    const int r = max(min(q_row0 + (tid >> 3), sp.q_rows - 1), 0);   // rows past the last one re-read it (never stored)
-    const u32x4 raw = *(const u32x4*)(a.q + ((size_t)(sp.q_begin + r) * H + head) * 64 + (tid & 7) * 8);
-    *(u32x4*)&patch_q[(tid >> 3) * kKStride + (tid & 7) * 8] = raw;
-    __syncthreads();
-#pragma unroll
-    for (int qb = 0; qb < 2; ++qb)
-#pragma unroll
-      for (int ks = 0; ks < 4; ++ks) {
-        const bf16x8 rawf = __builtin_bit_cast(bf16x8, *(const u32x4*)&patch_q[(qb * 32 + n32) * kKStride + ks * 16 + g * 8]);
-        f32x8 f = __builtin_convertvector(rawf, f32x8);
-#pragma unroll
-        for (int j = 0; j < 8; ++j) f[j] *= a.scale_log2;
-        qf[qb][ks] = __builtin_convertvector(f, bf16x8);
-      }
-    __syncthreads();   // the patches below overlay the Q rows
+  if (n_pieces == 0) {
+    // nothing visible: the reference returns zeros (lingbot_map/layers/flashinfer_cache.py:368-370).
+    // Decided before the first load, so that every load below is unconditional.
+    const int r = q_row0 + (tid >> 3);
+    if (r < sp.q_rows)
+      *(u32x4*)(a.out + ((size_t)(sp.q_begin + r) * H + head) * 64 + (tid & 7) * 8) = u32x4{0u, 0u, 0u, 0u};
+    return;
   }
 
   // ---- K/V rows of a piece: lane l takes the 16-byte part (l & 7) of rows (l >> 3) + 8 j
@@ -813,6 +799,36 @@ __global__ __launch_bounds__(kSmThreads, 1) void lbm_attn_bf16_d64_small_kernel(
       vv[j] = fetch(e, pool_v, own_v);
     }
   };
+  // Loads in the order their data is needed and their chains are long: this thread's piece of a
+  // Q row first (the load counter retires in order, so the wait for it must not sit behind the
+  // K/V rows), then the first piece's row entries and, once those are back, its K/V rows.
+  const int q_r = max(min(q_row0 + (tid >> 3), sp.q_rows - 1), 0);   // rows past the last one re-read it (never stored)
+  const u32x4 q_raw = *(const u32x4*)(a.q + ((size_t)(sp.q_begin + q_r) * H + head) * 64 + (tid & 7) * 8);
+  // (a wavefront without pieces loads the last piece and drops it: a load inside a conditional
+  // block would make the wait for the Q row a wait for everything in flight)
+  u32x4 kk[kPasses], vv[kPasses];
+  load_piece(min(p0, n_pieces - 1), kk, vv);
+
+  // ---- Q: the workgroup reads the 64 rows once as whole rows, every wavefront picks its
+  // fragments up from LDS; scale * log2(e) folded in (as in the main kernel)
+  bf16x8 qf[2][4];
+  {
+    unsigned short* patch_q = (unsigned short*)lds_raw;
+    *(u32x4*)&patch_q[(tid >> 3) * kKStride + (tid & 7) * 8] = q_raw;
+    __syncthreads();
+#pragma unroll
+    for (int qb = 0; qb < 2; ++qb)
+#pragma unroll
+      for (int ks = 0; ks < 4; ++ks) {
+        const bf16x8 rawf = __builtin_bit_cast(bf16x8, *(const u32x4*)&patch_q[(qb * 32 + n32) * kKStride + ks * 16 + g * 8]);
+        f32x8 f = __builtin_convertvector(rawf, f32x8);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) f[j] *= a.scale_log2;
+        qf[qb][ks] = __builtin_convertvector(f, bf16x8);
+      }
+    __syncthreads();   // the patches below overlay the Q rows
+  }
+
   auto store_piece = [&](const u32x4 (&kk)[kPasses], const u32x4 (&vv)[kPasses]) {
 #pragma unroll
     for (int j = 0; j < kPasses; ++j) {
@@ -854,8 +870,7 @@ __global__ __launch_bounds__(kSmThreads, 1) void lbm_attn_bf16_d64_small_kernel(
       m_run[qb] = safe ? -INFINITY : 0.f;
       l_lane[qb] = 0.f;
     }
-    u32x4 kk[kPasses], vv[kPasses];
-    if (p0 < p1) load_piece(p0, kk, vv);
+    if (pass > 0 && p0 < p1) load_piece(p0, kk, vv);   // (the first pass's first piece is already on its way)
     for (int pc = p0; pc < p1; ++pc) {
       store_piece(kk, vv);
       if (pc + 1 < p1) load_piece(pc + 1, kk, vv);   // in flight while this piece is computed
