@@ -739,7 +739,9 @@ static_assert(kSmLdsBytes >= kSmQBytes && kSmLdsBytes <= 160 * 1024, "LDS budget
 
 __global__ __launch_bounds__(kSmThreads, 1) void lbm_attn_bf16_d64_small_kernel(AttnArgs a) {
   __shared__ __attribute__((aligned(16))) unsigned char lds_raw[kSmLdsBytes];
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  // (the wavefront index is uniform by construction; said so, or the loop over this wavefront's
+  // pieces is compiled as divergent control flow)
+  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int n32 = lane & 31, g = lane >> 5;
   unsigned short* patch_k = (unsigned short*)(lds_raw + wave * kSmPatchBytes);
   unsigned short* patch_v = patch_k + kSmPiece * kKStride;
