@@ -101,6 +101,17 @@ __device__ __forceinline__ float gelu_erf(float v) {
   return 0.5f * v * (1.0f + erf_x);
 }
 __device__ __forceinline__ float bf16_bits_to_f32(unsigned v) { return __builtin_bit_cast(float, v << 16); }
+// The GELU of the fused fc1 epilogue acts on a value already rounded to bf16 and is rounded to
+// bf16 again: a function from 16 bits to 16 bits.  Evaluating it costs about 32 vector
+// instructions per element (more where the negative tail calls erff), 4 us of a 20 us launch;
+// the workgroup instead tabulates it in LDS for |v| in [2^-12, 2^3) - 15 binades x 128 mantissas
+// x 2 signs, 7.5 KB, filled from gelu_erf while the first operand tiles are on their way - and
+// looks the elements up.  Values outside the table (tiny, huge, inf, NaN: a handful per
+// million behind a LayerNorm) are evaluated directly behind a wave-uniform branch, so every
+// result is gelu_erf's, bit for bit.
+constexpr int kGeluE0 = 127 - 12;              // biased exponent of the first tabulated binade
+constexpr int kGeluHalf = 15 * 128;            // entries per sign
+constexpr int kGeluEntries = 2 * kGeluHalf;
 
 // TN: output columns per tile (128 or 64); a wavefront owns 64 x (TN / 2) of the tile.
 // ROPE / NORM: rotary layout (0 none, 1 interleaved, 2 half-split) and qk-LayerNorm of the
@@ -111,6 +122,7 @@ __global__ __launch_bounds__(kGThreads, 1) void lbm_linear_bf16_kernel(LinearArg
   // [buffer][k half][row][64 + pad]
   __shared__ __attribute__((aligned(16))) unsigned short lds_a[2][kGM * kGStride];
   __shared__ __attribute__((aligned(16))) unsigned short lds_w[2][TN * kGStride];
+  __shared__ unsigned short gelu_tab[EPI == LBM_LINEAR_BIAS_GELU ? kGeluEntries : 1];
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int n32 = lane & 31, g = lane >> 5;
@@ -213,6 +225,14 @@ __global__ __launch_bounds__(kGThreads, 1) void lbm_linear_bf16_kernel(LinearArg
   const int last = nk - 1;                       // steps past the end re-read the last one (never multiplied)
   load_step(0, ra0, rw0);
   load_step(min(1, last), ra1, rw1);
+  if (EPI == LBM_LINEAR_BIAS_GELU) {
+    // (under the latency of the loads above; the barrier before the first multiply publishes it)
+    for (int i = tid; i < kGeluEntries; i += kGThreads) {
+      const unsigned neg = i >= kGeluHalf ? 1u : 0u;
+      const unsigned bits = (neg << 15) | (unsigned)((kGeluE0 << 7) + (i - (int)neg * kGeluHalf));
+      gelu_tab[i] = __builtin_bit_cast(unsigned short, (__bf16)gelu_erf(bf16_bits_to_f32(bits)));
+    }
+  }
   store_step(0, ra0, rw0);
   load_step(min(2, last), ra0, rw0);
   __syncthreads();
@@ -266,7 +286,18 @@ __global__ __launch_bounds__(kGThreads, 1) void lbm_linear_bf16_kernel(LinearArg
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
         float v = round_bf16(fin[a][c4 * 4 + e] + bias4[e]);
-        if (EPI == LBM_LINEAR_BIAS_GELU) v = gelu_erf(v);
+        if (EPI == LBM_LINEAR_BIAS_GELU) {
+          const unsigned b16 = __builtin_bit_cast(unsigned, v) >> 16;
+          const unsigned rel = (b16 & 0x7fffu) - (unsigned)(kGeluE0 << 7);
+          const bool tabulated = rel < (unsigned)kGeluHalf;
+          const unsigned looked_up = gelu_tab[min(rel, (unsigned)(kGeluHalf - 1)) + (b16 >> 15) * kGeluHalf];
+          float r = bf16_bits_to_f32(looked_up);
+          if (__builtin_amdgcn_ballot_w64(!tabulated)) {
+            const float direct = gelu_erf(v);
+            r = tabulated ? r : direct;
+          }
+          v = r;
+        }
         if (EPI == LBM_LINEAR_BIAS_RESIDUAL && p.gamma) v = v * gamma4[e];
         y[e] = v;
       }

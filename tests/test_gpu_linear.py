@@ -68,6 +68,28 @@ def test_linear_bias(M, K, Nn):
     check(run_linear(a, w, None, N.LINEAR_BIAS), expected(a, w, None, N.LINEAR_BIAS))
 
 
+def test_gelu_epilogue_on_every_bf16_pre_activation():
+    """One-hot activations make the pre-activation of output (i, n) the weight w[n, i] itself, so
+    a 512 x 128 weight matrix puts every finite bf16 bit pattern through the epilogue: the
+    tabulated range, the values below and above it, both zeros, the negative tail.  torch's GELU
+    of the same bf16 values is the expectation: bit-equal from -3 up (zeros compare equal whatever
+    their sign), within one bf16 ulp of the pre-activation's scale below -3, where the result is
+    the last bits of an erff."""
+    N = _native()
+    bits = torch.arange(65536, dtype=torch.int32)
+    exp_field = (bits >> 7) & 0xFF
+    bits = torch.where(exp_field == 0xFF, torch.zeros_like(bits), bits)      # inf / NaN would poison the other columns' sums
+    w = bits.to(torch.uint16).view(torch.bfloat16).reshape(512, 128)
+    a = torch.eye(128, dtype=torch.bfloat16)
+    got = run_linear(a, w, None, N.LINEAR_BIAS_GELU)                          # [128, 512]: got[i, n] = gelu(w[n, i])
+    pre = w.t().contiguous()
+    ref = torch.nn.functional.gelu(pre.to("cuda:0")).cpu()
+    head = pre.float() >= -3.0
+    assert torch.equal(got.float()[head], ref.float()[head])
+    tail = ~head
+    assert ((got.float() - ref.float()).abs()[tail] <= 2.0 ** -8 * 2.0 ** -7 * pre.float().abs()[tail] + 1e-30).all()
+
+
 @pytest.mark.parametrize("M,K,Nn", [(1004, 1024, 4096), (257, 256, 320)])
 def test_linear_bias_gelu(M, K, Nn):
     N = _native()
