@@ -24,7 +24,7 @@
 extern "C" {
 #endif
 
-#define LBM_ABI_VERSION 5
+#define LBM_ABI_VERSION 6
 
 #define LBM_OK 0
 #define LBM_ERR_INVALID 1     /* bad argument (null pointer, negative size, bad enum)      */
@@ -210,6 +210,43 @@ int lbm_qkv_linear_prepare(const void* a, const void* w, const float* bias, int3
                            int32_t rope_layout, void* q_out, void* k_out, void* v_out, void* pool,
                            const int32_t* append_rows, int32_t num_heads, int32_t head_dim,
                            int32_t page_size, void* stream);
+
+/* A LayerNorm folded into the launch that consumes its output.  lbm_linear with the residual
+ * epilogue can leave behind, for every row of its output, one (mean, M2 = sum of squared
+ * deviations from that mean) pair per column tile of the launch: out_stats [M][tiles][2] float32
+ * with tiles = lbm_linear_stats_tiles(M, N).  A following launch that takes the output as its
+ * activations normalises each row on the way into the multiply - LayerNorm(a) @ w^T - from those
+ * pairs (merged as Chan et al.: equal-sized parts), so the normalised rows never go to memory and
+ * the LayerNorm is no launch of its own.  Replaces norm2(x) in front of the MLP (block.py:194-195)
+ * and norm1(x) of the block that follows (block.py:217).  The normalised value is
+ * ((x * rstd - mean * rstd) * weight + bias) rounded to bf16.
+ *   weight, bias  [K] bf16        stats  [M][stats_tiles][2] float32, stats_tiles divides K */
+typedef struct lbm_row_norm {
+  const void* weight;
+  const void* bias;
+  const float* stats;
+  int32_t stats_tiles;
+  float eps;
+} lbm_row_norm;
+
+/* Column tiles per row of the statistics lbm_linear_norm writes for an M x N output. */
+int32_t lbm_linear_stats_tiles(int32_t M, int32_t N);
+
+/* lbm_linear with a_norm (NULL = none; not with the residual epilogue) applied to the
+ * activations and / or out_stats (NULL = none; residual epilogue only) written. */
+int lbm_linear_norm(const void* a, const lbm_row_norm* a_norm, const void* w, const float* bias,
+                    const float* gamma, const void* residual, void* out, float* out_stats,
+                    int32_t M, int32_t N, int32_t K, int32_t epilogue, void* stream);
+
+/* lbm_qkv_linear_prepare with a_norm (NULL = none) applied to the activations: norm1 of the
+ * block, its qkv projection and the pre-attention producer as one launch. */
+int lbm_qkv_linear_prepare_norm(const void* a, const lbm_row_norm* a_norm, const void* w,
+                                const float* bias, int32_t M, int32_t K, const float* q_norm_w,
+                                const float* q_norm_b, const float* k_norm_w, const float* k_norm_b,
+                                float norm_eps, const float* rope_cs, int32_t rope_layout,
+                                void* q_out, void* k_out, void* v_out, void* pool,
+                                const int32_t* append_rows, int32_t num_heads, int32_t head_dim,
+                                int32_t page_size, void* stream);
 
 /* lbm_attn_run with the token counts read on the device: stream i attends to
  * live_kv_tokens[streams[i].live_at] entries of its row table instead of streams[i].kv_tokens,

@@ -122,15 +122,26 @@ int lbm_qkv_prepare(const void* qkv, int32_t src_dtype, const float* q_norm_w, c
                                 (hipStream_t)stream);
 }
 
-int lbm_linear(const void* a, const void* w, const float* bias, const float* gamma, const void* residual,
-               void* out, int32_t M, int32_t N, int32_t K, int32_t epilogue, void* stream) {
+int lbm_linear_norm(const void* a, const lbm_row_norm* a_norm, const void* w, const float* bias, const float* gamma,
+                    const void* residual, void* out, float* out_stats, int32_t M, int32_t N, int32_t K,
+                    int32_t epilogue, void* stream) {
   if (!a || !w || !out) return lbm_fail(LBM_ERR_INVALID, "lbm_linear: null a, w or out");
   if (M < 0 || N <= 0 || K <= 0) return lbm_fail(LBM_ERR_INVALID, "lbm_linear: bad shape %d x %d x %d", M, N, K);
   if (epilogue == LBM_LINEAR_BIAS_RESIDUAL && !residual)
     return lbm_fail(LBM_ERR_INVALID, "lbm_linear: the residual epilogue needs a residual");
   if (epilogue != LBM_LINEAR_BIAS_RESIDUAL && (residual || gamma))
     return lbm_fail(LBM_ERR_INVALID, "lbm_linear: residual / gamma given without the residual epilogue");
-  return lbm_launch_linear(a, w, bias, gamma, residual, out, M, N, K, epilogue, (hipStream_t)stream);
+  return lbm_launch_linear(a, a_norm, w, bias, gamma, residual, out, out_stats, M, N, K, epilogue, (hipStream_t)stream);
+}
+
+int lbm_linear(const void* a, const void* w, const float* bias, const float* gamma, const void* residual,
+               void* out, int32_t M, int32_t N, int32_t K, int32_t epilogue, void* stream) {
+  return lbm_linear_norm(a, nullptr, w, bias, gamma, residual, out, nullptr, M, N, K, epilogue, stream);
+}
+
+int32_t lbm_linear_stats_tiles(int32_t M, int32_t N) {
+  if (M < 0 || N <= 0 || N % 64 != 0) return 0;
+  return lbm_linear_stats_tiles_for(M, N);
 }
 
 int lbm_qkv_linear_prepare(const void* a, const void* w, const float* bias, int32_t M, int32_t K,
@@ -138,6 +149,16 @@ int lbm_qkv_linear_prepare(const void* a, const void* w, const float* bias, int3
                            const float* k_norm_b, float norm_eps, const float* rope_cs, int32_t rope_layout,
                            void* q_out, void* k_out, void* v_out, void* pool, const int32_t* append_rows,
                            int32_t num_heads, int32_t head_dim, int32_t page_size, void* stream) {
+  return lbm_qkv_linear_prepare_norm(a, nullptr, w, bias, M, K, q_norm_w, q_norm_b, k_norm_w, k_norm_b, norm_eps, rope_cs,
+                                     rope_layout, q_out, k_out, v_out, pool, append_rows, num_heads, head_dim, page_size,
+                                     stream);
+}
+
+int lbm_qkv_linear_prepare_norm(const void* a, const lbm_row_norm* a_norm, const void* w, const float* bias, int32_t M,
+                                int32_t K, const float* q_norm_w, const float* q_norm_b, const float* k_norm_w,
+                                const float* k_norm_b, float norm_eps, const float* rope_cs, int32_t rope_layout,
+                                void* q_out, void* k_out, void* v_out, void* pool, const int32_t* append_rows,
+                                int32_t num_heads, int32_t head_dim, int32_t page_size, void* stream) {
   if (!a || !w || !q_out) return lbm_fail(LBM_ERR_INVALID, "lbm_qkv_linear_prepare: null a, w or q_out");
   if (M < 0 || K <= 0 || num_heads <= 0) return lbm_fail(LBM_ERR_INVALID, "lbm_qkv_linear_prepare: bad shape");
   if (head_dim != 64) return lbm_fail(LBM_ERR_UNSUPPORTED, "lbm_qkv_linear_prepare: head_dim must be 64 (got %d)", head_dim);
@@ -147,7 +168,7 @@ int lbm_qkv_linear_prepare(const void* a, const void* w, const float* bias, int3
     return lbm_fail(LBM_ERR_INVALID, "lbm_qkv_linear_prepare: unknown rope_layout %d", rope_layout);
   if (append_rows && !pool) return lbm_fail(LBM_ERR_INVALID, "lbm_qkv_linear_prepare: append_rows without a pool");
   if (append_rows && page_size <= 0) return lbm_fail(LBM_ERR_INVALID, "lbm_qkv_linear_prepare: bad page_size");
-  return lbm_launch_qkv_linear_prepare(a, w, bias, M, K, q_norm_w, q_norm_b, k_norm_w, k_norm_b, norm_eps, rope_cs,
+  return lbm_launch_qkv_linear_prepare(a, a_norm, w, bias, M, K, q_norm_w, q_norm_b, k_norm_w, k_norm_b, norm_eps, rope_cs,
                                        rope_layout, q_out, k_out, v_out, pool, append_rows, num_heads, page_size,
                                        (hipStream_t)stream);
 }

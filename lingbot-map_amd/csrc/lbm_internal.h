@@ -33,10 +33,12 @@ int lbm_launch_residual_norm(const void* x, const void* y, int dtype, const floa
                              const float* norm_b, float eps, void* x_out, void* n_out, int rows, int cols,
                              hipStream_t stream);
 
-int lbm_launch_linear(const void* a, const void* w, const float* bias, const float* gamma, const void* residual,
-                      void* out, int M, int N, int K, int epilogue, hipStream_t stream);
+int lbm_launch_linear(const void* a, const lbm_row_norm* a_norm, const void* w, const float* bias, const float* gamma,
+                      const void* residual, void* out, float* out_stats, int M, int N, int K, int epilogue,
+                      hipStream_t stream);
+int lbm_linear_stats_tiles_for(int M, int N);
 
-int lbm_launch_qkv_linear_prepare(const void* a, const void* w, const float* bias, int M, int K,
+int lbm_launch_qkv_linear_prepare(const void* a, const lbm_row_norm* a_norm, const void* w, const float* bias, int M, int K,
                                   const float* q_norm_w, const float* q_norm_b, const float* k_norm_w,
                                   const float* k_norm_b, float norm_eps, const float* rope_cs, int rope_layout,
                                   void* q_out, void* k_out, void* v_out, void* pool, const int32_t* append_rows,

@@ -37,6 +37,7 @@ typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
 typedef __attribute__((ext_vector_type(16))) float f32x16;
 typedef __attribute__((ext_vector_type(4))) float f32x4;
+typedef __attribute__((ext_vector_type(2))) float f32x2;
 typedef __attribute__((ext_vector_type(4))) unsigned int u32x4;
 typedef __attribute__((ext_vector_type(2))) unsigned int u32x2;
 
@@ -44,6 +45,7 @@ constexpr int kGK = 128;         // k-step of the workgroup (64 per wave group)
 constexpr int kGStride = 136;    // bf16 per LDS row of a k-step (128 elements + 16 bytes: 272 B)
 constexpr int kGM = 128;         // activation rows per tile
 constexpr int kGThreads = 512;
+constexpr int kLnMaxK = 2048;    // widest input a folded LayerNorm is accepted for (its parameters sit in LDS)
 
 struct LinearArgs {
   const unsigned short* a;       // [M, K]
@@ -66,6 +68,17 @@ struct LinearArgs {
   const int32_t* append_rows;    // null: nothing is appended
   float eps;
   int num_heads, page_size;
+  // LNA kernels: the activations are LayerNorm'ed over K on their way into LDS, from row
+  // statistics the launch that produced them left behind (one (mean, M2) pair per row and
+  // column tile of that launch)
+  const unsigned short* ln_w;    // [K] bf16
+  const unsigned short* ln_b;    // [K] bf16
+  const float* ln_stats;         // [M][ln_tiles][2]
+  int ln_tiles;
+  float ln_eps;
+  // LBM_LINEAR_BIAS_RESIDUAL: (mean, M2) of every output row over this tile's columns,
+  // [M][n_tiles][2], or null
+  float* stats_out;
 };
 constexpr int kEpiQkvPrepare = 3;   // internal: reached through lbm_qkv_linear_prepare only
 
@@ -116,13 +129,16 @@ constexpr int kGeluEntries = 2 * kGeluHalf;
 // TN: output columns per tile (128 or 64); a wavefront owns 64 x (TN / 2) of the tile.
 // ROPE / NORM: rotary layout (0 none, 1 interleaved, 2 half-split) and qk-LayerNorm of the
 // kEpiQkvPrepare epilogue; 0 / false otherwise.
-template <int EPI, int TN, int ROPE = 0, bool NORM = false>
+// LNA: LayerNorm of the activations folded into their staging (see LinearArgs).
+template <int EPI, int TN, int ROPE = 0, bool NORM = false, bool LNA = false>
 __global__ __launch_bounds__(kGThreads, 1) void lbm_linear_bf16_kernel(LinearArgs p) {
   constexpr int NT = TN / 64;   // 32-column blocks of W per wavefront
   // [buffer][k half][row][64 + pad]
   __shared__ __attribute__((aligned(16))) unsigned short lds_a[2][kGM * kGStride];
   __shared__ __attribute__((aligned(16))) unsigned short lds_w[2][TN * kGStride];
   __shared__ unsigned short gelu_tab[EPI == LBM_LINEAR_BIAS_GELU ? kGeluEntries : 1];
+  __shared__ __attribute__((aligned(8))) float ln_rows[LNA ? kGM * 2 : 2];   // per row of the tile: rstd, -mean * rstd
+  __shared__ __attribute__((aligned(16))) unsigned short ln_wb[LNA ? 2 * kLnMaxK : 8];   // LayerNorm weight, then bias
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int n32 = lane & 31, g = lane >> 5;
@@ -146,25 +162,53 @@ __global__ __launch_bounds__(kGThreads, 1) void lbm_linear_bf16_kernel(LinearArg
   // ---- staging: thread t moves the 16-byte piece (t & 15) of rows (t >> 4) + 32 j of a k-step
   constexpr int kPassA = kGM / 32, kPassW = TN / 32;
   const int ld_r = tid >> 4, ld_c = (tid & 15) * 8;          // ld_c: element within the 128 of the k-step
-  const unsigned short* ga[kPassA];
-  const unsigned short* gw[kPassW];
+  // 32-bit byte offsets from uniform bases (a scalar base + a vector offset per load instead of a
+  // 64-bit vector address per row pass: 11 registers less)
+  unsigned a_off[kPassA];
 #pragma unroll
-  for (int j = 0; j < kPassA; ++j) ga[j] = p.a + (size_t)min(m0 + ld_r + 32 * j, p.M - 1) * p.K + ld_c;   // rows past M re-read the last row
-#pragma unroll
-  for (int j = 0; j < kPassW; ++j) gw[j] = p.w + (size_t)(n0 + ld_r + 32 * j) * p.K + ld_c;
+  for (int j = 0; j < kPassA; ++j) a_off[j] = ((unsigned)min(m0 + ld_r + 32 * j, p.M - 1) * (unsigned)p.K + ld_c) * 2u;   // rows past M re-read the last row
+  const unsigned w_off = ((unsigned)ld_r * (unsigned)p.K + ld_c) * 2u;
+  const char* a_base = (const char*)p.a;
+  const char* w_base = (const char*)(p.w + (size_t)n0 * p.K);
+  auto load_a = [&](int j, int ks) -> u32x4 { return *(const u32x4*)(a_base + ks * (kGK * 2) + a_off[j]); };
+  auto load_w = [&](int j, int ks) -> u32x4 {
+    return *(const u32x4*)(w_base + ((size_t)(32 * j) * p.K + (size_t)ks * kGK) * 2 + w_off);
+  };
   // Two register sets: the rows of k-step s are asked for at the top of iteration s - 2 and
   // written into the LDS buffer at the end of iteration s - 1, so a load has two multiply
   // phases to arrive before anything waits for it.
   u32x4 ra0[kPassA], rw0[kPassW], ra1[kPassA], rw1[kPassW];
+  // LNA: every staged piece of the activations is normalised before it goes to LDS:
+  // (x * rstd - mean * rstd) * w + b, the row's two factors and the weight and bias of the
+  // thread's 8 columns of k-step ks read from LDS
+  auto norm_piece = [&](const u32x4& raw, int j, int ks) -> u32x4 {
+    if (!LNA) return raw;
+    const f32x2 row = *(const f32x2*)&ln_rows[2 * (ld_r + 32 * j)];
+    const float ln_sc_j = row[0], ln_sh_j = row[1];
+    u32x4 ln[2];
+    ln[0] = *(const u32x4*)&ln_wb[ks * kGK + ld_c];
+    ln[1] = *(const u32x4*)&ln_wb[kLnMaxK + ks * kGK + ld_c];
+    u32x4 o;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const float x0 = bf16_bits_to_f32(raw[e] & 0xffffu), x1 = __builtin_bit_cast(float, raw[e] & 0xffff0000u);
+      const float w0 = bf16_bits_to_f32(ln[0][e] & 0xffffu), w1 = __builtin_bit_cast(float, ln[0][e] & 0xffff0000u);
+      const float b0 = bf16_bits_to_f32(ln[1][e] & 0xffffu), b1 = __builtin_bit_cast(float, ln[1][e] & 0xffff0000u);
+      const float y0 = __builtin_fmaf(__builtin_fmaf(x0, ln_sc_j, ln_sh_j), w0, b0);
+      const float y1 = __builtin_fmaf(__builtin_fmaf(x1, ln_sc_j, ln_sh_j), w1, b1);
+      o[e] = (unsigned)__builtin_bit_cast(unsigned short, (__bf16)y0) | ((unsigned)__builtin_bit_cast(unsigned short, (__bf16)y1) << 16);
+    }
+    return o;
+  };
   auto load_step = [&](int ks, u32x4 (&ra)[kPassA], u32x4 (&rw)[kPassW]) {
 #pragma unroll
-    for (int j = 0; j < kPassA; ++j) ra[j] = *(const u32x4*)(ga[j] + ks * kGK);
+    for (int j = 0; j < kPassA; ++j) ra[j] = load_a(j, ks);
 #pragma unroll
-    for (int j = 0; j < kPassW; ++j) rw[j] = *(const u32x4*)(gw[j] + ks * kGK);
+    for (int j = 0; j < kPassW; ++j) rw[j] = load_w(j, ks);
   };
-  auto store_step = [&](int buf, const u32x4 (&ra)[kPassA], const u32x4 (&rw)[kPassW]) {
+  auto store_step = [&](int buf, const u32x4 (&ra)[kPassA], const u32x4 (&rw)[kPassW], int ks) {
 #pragma unroll
-    for (int j = 0; j < kPassA; ++j) *(u32x4*)&lds_a[buf][(ld_r + 32 * j) * kGStride + ld_c] = ra[j];
+    for (int j = 0; j < kPassA; ++j) *(u32x4*)&lds_a[buf][(ld_r + 32 * j) * kGStride + ld_c] = norm_piece(ra[j], j, ks);
 #pragma unroll
     for (int j = 0; j < kPassW; ++j) *(u32x4*)&lds_w[buf][(ld_r + 32 * j) * kGStride + ld_c] = rw[j];
   };
@@ -181,7 +225,8 @@ __global__ __launch_bounds__(kGThreads, 1) void lbm_linear_bf16_kernel(LinearArg
   // and the rows of the step after next (held in `ra`, `rw` since the previous iteration) go
   // into the other LDS buffer two stores per slice, in the shadow of the MFMAs, followed by the
   // loads that refill the set.  sched_barrier keeps the slices as written.
-  auto step = [&](int buf, u32x4 (&ra)[kPassA], u32x4 (&rw)[kPassW], bool write, int next_ks) {
+  // (`held_ks`: the k-step whose rows `ra`, `rw` hold on entry)
+  auto step = [&](int buf, u32x4 (&ra)[kPassA], u32x4 (&rw)[kPassW], int held_ks, int next_ks) {
     const unsigned short* la = &lds_a[buf][kh * 64];
     const unsigned short* lw = &lds_w[buf][kh * 64];
     bf16x8 wf[2][NT], af[2][2];
@@ -202,21 +247,20 @@ __global__ __launch_bounds__(kGThreads, 1) void lbm_linear_bf16_kernel(LinearArg
 #pragma unroll
         for (int b = 0; b < 2; ++b)
           acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wf[k16 & 1][a], af[k16 & 1][b], acc[a][b], 0, 0, 0);
-      if (write) {
-        // this slice's share of the stores: the passes j with j % 4 == k16
-#pragma unroll
-        for (int j = 0; j < kPassA; ++j)
-          if ((j & 3) == k16) *(u32x4*)&lds_a[buf ^ 1][(ld_r + 32 * j) * kGStride + ld_c] = ra[j];
-#pragma unroll
-        for (int j = 0; j < kPassW; ++j)
-          if ((j & 3) == k16) *(u32x4*)&lds_w[buf ^ 1][(ld_r + 32 * j) * kGStride + ld_c] = rw[j];
-      }
+      // this slice's share of the stores: the passes j with j % 4 == k16 (after the last k-step
+      // they put a repeat of it into a buffer nobody reads any more: cheaper than a branch per slice)
 #pragma unroll
       for (int j = 0; j < kPassA; ++j)
-        if ((j & 3) == k16) ra[j] = *(const u32x4*)(ga[j] + next_ks * kGK);
+        if ((j & 3) == k16) *(u32x4*)&lds_a[buf ^ 1][(ld_r + 32 * j) * kGStride + ld_c] = norm_piece(ra[j], j, held_ks);
 #pragma unroll
       for (int j = 0; j < kPassW; ++j)
-        if ((j & 3) == k16) rw[j] = *(const u32x4*)(gw[j] + next_ks * kGK);
+        if ((j & 3) == k16) *(u32x4*)&lds_w[buf ^ 1][(ld_r + 32 * j) * kGStride + ld_c] = rw[j];
+#pragma unroll
+      for (int j = 0; j < kPassA; ++j)
+        if ((j & 3) == k16) ra[j] = load_a(j, next_ks);
+#pragma unroll
+      for (int j = 0; j < kPassW; ++j)
+        if ((j & 3) == k16) rw[j] = load_w(j, next_ks);
       __builtin_amdgcn_sched_barrier(0);
     }
   };
@@ -225,6 +269,36 @@ __global__ __launch_bounds__(kGThreads, 1) void lbm_linear_bf16_kernel(LinearArg
   const int last = nk - 1;                       // steps past the end re-read the last one (never multiplied)
   load_step(0, ra0, rw0);
   load_step(min(1, last), ra1, rw1);
+  if (LNA) {
+    for (int i = tid * 8; i < p.K; i += kGThreads * 8) {
+      *(u32x4*)&ln_wb[i] = *(const u32x4*)(p.ln_w + i);
+      *(u32x4*)&ln_wb[kLnMaxK + i] = *(const u32x4*)(p.ln_b + i);
+    }
+    // Row statistics: row r of the tile is handled by threads 4 r .. 4 r + 3, each taking every
+    // fourth (mean, M2) partial; equal-sized partials merge as mean = avg(mean_i),
+    // M2 = sum(M2_i) + n_i * sum((mean_i - mean)^2) (Chan et al.), variance = M2 / K.
+    const int r = tid >> 2, part = tid & 3;
+    const float* st = p.ln_stats + (size_t)min(m0 + r, p.M - 1) * p.ln_tiles * 2;
+    float sm = 0.f;
+    for (int i = part; i < p.ln_tiles; i += 4) sm += st[2 * i];
+    sm += __shfl_xor(sm, 1);
+    sm += __shfl_xor(sm, 2);
+    const float mean = sm / (float)p.ln_tiles;
+    const float n_i = (float)p.K / (float)p.ln_tiles;
+    float m2 = 0.f;
+    for (int i = part; i < p.ln_tiles; i += 4) {
+      const float d = st[2 * i] - mean;
+      m2 += st[2 * i + 1] + n_i * d * d;
+    }
+    m2 += __shfl_xor(m2, 1);
+    m2 += __shfl_xor(m2, 2);
+    const float rstd = __builtin_amdgcn_rsqf(m2 / (float)p.K + p.ln_eps);
+    if (part == 0) {
+      ln_rows[2 * r] = rstd;
+      ln_rows[2 * r + 1] = -mean * rstd;
+    }
+    __syncthreads();
+  }
   if (EPI == LBM_LINEAR_BIAS_GELU) {
     // (under the latency of the loads above; the barrier before the first multiply publishes it)
     for (int i = tid; i < kGeluEntries; i += kGThreads) {
@@ -233,16 +307,16 @@ __global__ __launch_bounds__(kGThreads, 1) void lbm_linear_bf16_kernel(LinearArg
       gelu_tab[i] = __builtin_bit_cast(unsigned short, (__bf16)gelu_erf(bf16_bits_to_f32(bits)));
     }
   }
-  store_step(0, ra0, rw0);
+  store_step(0, ra0, rw0, 0);
   load_step(min(2, last), ra0, rw0);
   __syncthreads();
   // iteration ks multiplies buffer ks & 1 and moves the set holding step ks + 1 into the other
   // buffer, then refills that set with step ks + 3
   for (int ks = 0; ks < nk; ks += 2) {
-    step(0, ra1, rw1, ks + 1 < nk, min(ks + 3, last));
+    step(0, ra1, rw1, min(ks + 1, last), min(ks + 3, last));
     __syncthreads();
     if (ks + 1 >= nk) break;
-    step(1, ra0, rw0, ks + 2 < nk, min(ks + 4, last));
+    step(1, ra0, rw0, min(ks + 2, last), min(ks + 4, last));
     __syncthreads();
   }
 
@@ -385,6 +459,30 @@ __global__ __launch_bounds__(kGThreads, 1) void lbm_linear_bf16_kernel(LinearArg
       }
       *(u32x4*)dst = v;
     }
+    if (EPI == LBM_LINEAR_BIAS_RESIDUAL && p.stats_out) {
+      // (mean, M2) of the row's TN stored values: the kPieces lanes that hold the row are
+      // neighbours inside one 16-lane group
+      float x[8];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        x[2 * e] = bf16_bits_to_f32(v[e] & 0xffffu);
+        x[2 * e + 1] = bf16_bits_to_f32(v[e] >> 16);
+      }
+      float sm = ((x[0] + x[1]) + (x[2] + x[3])) + ((x[4] + x[5]) + (x[6] + x[7]));
+#pragma unroll
+      for (int m = 1; m < kPieces; m <<= 1) sm += __shfl_xor(sm, m);
+      const float mean = sm / (float)TN;
+      float m2 = 0.f;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) m2 += (x[e] - mean) * (x[e] - mean);
+#pragma unroll
+      for (int m = 1; m < kPieces; m <<= 1) m2 += __shfl_xor(m2, m);
+      if (row < p.M && (tid % kPieces) == 0) {
+        float* so = p.stats_out + ((size_t)row * p.n_tiles + nt) * 2;
+        so[0] = mean;
+        so[1] = m2;
+      }
+    }
   }
 }
 
@@ -403,12 +501,43 @@ int lbm_linear_tiles(LinearArgs& p) {
 }
 }  // namespace
 
-int lbm_launch_linear(const void* a, const void* w, const float* bias, const float* gamma, const void* residual,
-                      void* out, int M, int N, int K, int epilogue, hipStream_t stream) {
+namespace {
+// the folded LayerNorm of the activations, checked and copied into the kernel arguments
+int lbm_set_row_norm(LinearArgs& p, const lbm_row_norm* ln, const char* who) {
+  if (!ln) return LBM_OK;
+  if (p.K > kLnMaxK)
+    return lbm_fail(LBM_ERR_UNSUPPORTED, "%s: a folded LayerNorm takes inputs up to %d wide (got %d)", who, kLnMaxK, p.K);
+  if (!ln->weight || !ln->bias || !ln->stats || ln->stats_tiles <= 0 || p.K % ln->stats_tiles != 0)
+    return lbm_fail(LBM_ERR_INVALID, "%s: the folded LayerNorm needs weight, bias, stats and a tile count that divides K (got %d for K %d)",
+                    who, ln->stats_tiles, p.K);
+  p.ln_w = (const unsigned short*)ln->weight;
+  p.ln_b = (const unsigned short*)ln->bias;
+  p.ln_stats = ln->stats;
+  p.ln_tiles = ln->stats_tiles;
+  p.ln_eps = ln->eps;
+  return LBM_OK;
+}
+}  // namespace
+
+int lbm_linear_stats_tiles_for(int M, int N) {
+  LinearArgs p = {};
+  p.M = M; p.N = N;
+  lbm_linear_tiles(p);
+  return p.n_tiles;
+}
+
+int lbm_launch_linear(const void* a, const lbm_row_norm* a_norm, const void* w, const float* bias, const float* gamma,
+                      const void* residual, void* out, float* out_stats, int M, int N, int K, int epilogue,
+                      hipStream_t stream) {
   if (M == 0) return LBM_OK;
   if (K % kGK != 0 || N % 64 != 0)
     return lbm_fail(LBM_ERR_UNSUPPORTED, "lbm_linear: K must be a multiple of 128 and N of 64 (got K %d, N %d)", K, N);
+  if (a_norm && epilogue == LBM_LINEAR_BIAS_RESIDUAL)
+    return lbm_fail(LBM_ERR_UNSUPPORTED, "lbm_linear: no folded LayerNorm with the residual epilogue");
+  if (out_stats && epilogue != LBM_LINEAR_BIAS_RESIDUAL)
+    return lbm_fail(LBM_ERR_UNSUPPORTED, "lbm_linear: row statistics come with the residual epilogue only");
   LinearArgs p = {};
+  p.stats_out = out_stats;
   p.a = (const unsigned short*)a;
   p.w = (const unsigned short*)w;
   p.bias = bias;
@@ -416,22 +545,26 @@ int lbm_launch_linear(const void* a, const void* w, const float* bias, const flo
   p.res = (const unsigned short*)residual;
   p.out = (unsigned short*)out;
   p.M = M; p.N = N; p.K = K;
+  if (int rc = lbm_set_row_norm(p, a_norm, "lbm_linear_norm")) return rc;
   const bool wide = lbm_linear_tiles(p) == 128;
+  const bool lna = a_norm != nullptr;
   const dim3 grid((unsigned)(p.m_tiles * p.n_tiles)), block(kGThreads);
-#define LBM_LINEAR_LAUNCH(E)                                                                         \
-  {                                                                                                  \
-    if (wide) hipLaunchKernelGGL((lbm_linear_bf16_kernel<E, 128>), grid, block, 0, stream, p);       \
-    else hipLaunchKernelGGL((lbm_linear_bf16_kernel<E, 64>), grid, block, 0, stream, p);             \
+#define LBM_LINEAR_LAUNCH(E, L)                                                                                  \
+  {                                                                                                              \
+    if (wide) hipLaunchKernelGGL((lbm_linear_bf16_kernel<E, 128, 0, false, L>), grid, block, 0, stream, p);      \
+    else hipLaunchKernelGGL((lbm_linear_bf16_kernel<E, 64, 0, false, L>), grid, block, 0, stream, p);            \
   }
-  if (epilogue == LBM_LINEAR_BIAS) LBM_LINEAR_LAUNCH(LBM_LINEAR_BIAS)
-  else if (epilogue == LBM_LINEAR_BIAS_GELU) LBM_LINEAR_LAUNCH(LBM_LINEAR_BIAS_GELU)
-  else if (epilogue == LBM_LINEAR_BIAS_RESIDUAL) LBM_LINEAR_LAUNCH(LBM_LINEAR_BIAS_RESIDUAL)
+  if (epilogue == LBM_LINEAR_BIAS && lna) LBM_LINEAR_LAUNCH(LBM_LINEAR_BIAS, true)
+  else if (epilogue == LBM_LINEAR_BIAS) LBM_LINEAR_LAUNCH(LBM_LINEAR_BIAS, false)
+  else if (epilogue == LBM_LINEAR_BIAS_GELU && lna) LBM_LINEAR_LAUNCH(LBM_LINEAR_BIAS_GELU, true)
+  else if (epilogue == LBM_LINEAR_BIAS_GELU) LBM_LINEAR_LAUNCH(LBM_LINEAR_BIAS_GELU, false)
+  else if (epilogue == LBM_LINEAR_BIAS_RESIDUAL) LBM_LINEAR_LAUNCH(LBM_LINEAR_BIAS_RESIDUAL, false)
   else return lbm_fail(LBM_ERR_INVALID, "lbm_linear: unknown epilogue %d", epilogue);
 #undef LBM_LINEAR_LAUNCH
   return lbm_check_launch("lbm_linear_bf16_kernel");
 }
 
-int lbm_launch_qkv_linear_prepare(const void* a, const void* w, const float* bias, int M, int K,
+int lbm_launch_qkv_linear_prepare(const void* a, const lbm_row_norm* a_norm, const void* w, const float* bias, int M, int K,
                                   const float* q_norm_w, const float* q_norm_b, const float* k_norm_w,
                                   const float* k_norm_b, float norm_eps, const float* rope_cs, int rope_layout,
                                   void* q_out, void* k_out, void* v_out, void* pool, const int32_t* append_rows,
@@ -452,6 +585,8 @@ int lbm_launch_qkv_linear_prepare(const void* a, const void* w, const float* bia
   p.append_rows = append_rows;
   p.eps = norm_eps;
   p.num_heads = num_heads; p.page_size = page_size;
+  if (int rc = lbm_set_row_norm(p, a_norm, "lbm_qkv_linear_prepare_norm")) return rc;
+  const bool lna = a_norm != nullptr;
   // a tile must not straddle q | k | v: 128-wide tiles need an even number of heads
   bool wide = lbm_linear_tiles(p) == 128;
   if (wide && (num_heads & 1)) {
@@ -461,10 +596,14 @@ int lbm_launch_qkv_linear_prepare(const void* a, const void* w, const float* bia
   const dim3 grid((unsigned)(p.m_tiles * p.n_tiles)), block(kGThreads);
   const int rope = !rope_cs ? 0 : (rope_layout == LBM_ROPE_INTERLEAVED ? 1 : 2);
   const bool norm = q_norm_w != nullptr;
+#define LBM_QKV_LAUNCH_L(R, NRM, L)                                                                                   \
+  {                                                                                                                   \
+    if (wide) hipLaunchKernelGGL((lbm_linear_bf16_kernel<kEpiQkvPrepare, 128, R, NRM, L>), grid, block, 0, stream, p); \
+    else hipLaunchKernelGGL((lbm_linear_bf16_kernel<kEpiQkvPrepare, 64, R, NRM, L>), grid, block, 0, stream, p);       \
+  }
 #define LBM_QKV_LAUNCH(R, NRM)                                                                                        \
   {                                                                                                                   \
-    if (wide) hipLaunchKernelGGL((lbm_linear_bf16_kernel<kEpiQkvPrepare, 128, R, NRM>), grid, block, 0, stream, p);   \
-    else hipLaunchKernelGGL((lbm_linear_bf16_kernel<kEpiQkvPrepare, 64, R, NRM>), grid, block, 0, stream, p);         \
+    if (lna) LBM_QKV_LAUNCH_L(R, NRM, true) else LBM_QKV_LAUNCH_L(R, NRM, false)                                      \
   }
   if (rope == 0 && !norm) LBM_QKV_LAUNCH(0, false)
   else if (rope == 0) LBM_QKV_LAUNCH(0, true)
@@ -472,6 +611,7 @@ int lbm_launch_qkv_linear_prepare(const void* a, const void* w, const float* bia
   else if (rope == 1) LBM_QKV_LAUNCH(1, true)
   else if (!norm) LBM_QKV_LAUNCH(2, false)
   else LBM_QKV_LAUNCH(2, true)
+#undef LBM_QKV_LAUNCH_L
 #undef LBM_QKV_LAUNCH
   return lbm_check_launch("lbm_linear_bf16_kernel<qkv prepare>");
 }

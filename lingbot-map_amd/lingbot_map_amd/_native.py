@@ -22,7 +22,7 @@ HDR = {"frame_count": 0, "n_anchor": 1, "win_head": 2, "win_count": 3, "n_free_p
        "n_free_special": 5, "n_special_pages": 6, "special_tokens": 7, "n_memory": 8,
        "n_memory_pages": 9, "error": 10, "plan_kv_tokens": 11, "plan_n_pages": 12}
 HDR_WORDS = 16
-ABI_VERSION = 5
+ABI_VERSION = 6
 
 
 class CacheGeom(C.Structure):
@@ -41,8 +41,14 @@ class AttnStream(C.Structure):
     _fields_ = [(n, C.c_int32) for n in ("q_begin", "q_rows", "kv_row_begin", "kv_tokens", "live_at")]
 
 
+class RowNorm(C.Structure):
+    """``lbm_row_norm``: a LayerNorm folded into the launch that consumes its output."""
+    _fields_ = [("weight", C.c_void_p), ("bias", C.c_void_p), ("stats", C.c_void_p),
+                ("stats_tiles", C.c_int32), ("eps", C.c_float)]
+
+
 SYMBOLS = ("lbm_abi_version", "lbm_last_error", "lbm_tables_words", "lbm_tables_step",
-           "lbm_rows_from_pages", "lbm_kv_append", "lbm_qkv_prepare", "lbm_residual_norm", "lbm_linear", "lbm_qkv_linear_prepare", "lbm_attn_workspace_bytes", "lbm_attn_run", "lbm_attn_run_live",
+           "lbm_rows_from_pages", "lbm_kv_append", "lbm_qkv_prepare", "lbm_residual_norm", "lbm_linear", "lbm_linear_norm", "lbm_linear_stats_tiles", "lbm_qkv_linear_prepare", "lbm_qkv_linear_prepare_norm", "lbm_attn_workspace_bytes", "lbm_attn_run", "lbm_attn_run_live",
            "lbm_attn_run_static")
 
 
@@ -69,6 +75,12 @@ def _load():
     lib.lbm_residual_norm.argtypes = [vp, vp, i32, vp, vp, vp, C.c_float, vp, vp, i32, i32, vp]
     lib.lbm_linear.restype = C.c_int
     lib.lbm_linear.argtypes = [vp, vp, vp, vp, vp, vp, i32, i32, i32, i32, vp]
+    lib.lbm_linear_norm.restype = C.c_int
+    lib.lbm_linear_norm.argtypes = [vp, p(RowNorm), vp, vp, vp, vp, vp, vp, i32, i32, i32, i32, vp]
+    lib.lbm_linear_stats_tiles.restype = i32
+    lib.lbm_linear_stats_tiles.argtypes = [i32, i32]
+    lib.lbm_qkv_linear_prepare_norm.restype = C.c_int
+    lib.lbm_qkv_linear_prepare_norm.argtypes = [vp, p(RowNorm), vp, vp, i32, i32, vp, vp, vp, vp, C.c_float, vp, i32, vp, vp, vp, vp, vp, i32, i32, i32, vp]
     lib.lbm_qkv_linear_prepare.restype = C.c_int
     lib.lbm_qkv_linear_prepare.argtypes = [vp, vp, vp, i32, i32, vp, vp, vp, vp, C.c_float, vp, i32, vp, vp, vp, vp, vp, i32, i32, i32, vp]
     lib.lbm_attn_workspace_bytes.restype = C.c_size_t

@@ -211,6 +211,16 @@ class HipAggregatorStream(nn.Module):
         frames are counted from the number already cached (stream.py:297-368)."""
         scale_frames = self.num_frame_for_scale if num_frame_for_scale is None else num_frame_for_scale
         cached = self.kv_cache_manager.num_frames if self.kv_cache_manager is not None else 0
+        # which frames of the call are "first" is host knowledge; the assembled tokens of a pattern
+        # are kept until a parameter changes (every steady-state frame asks for the same ones)
+        first = tuple(cached + i < 1 for i in range(S))
+        first_scale = tuple(cached + i < max(min(scale_frames, cached + S), 1) for i in range(S))
+        params = [self.camera_token] + ([self.register_token] if self.num_register_tokens > 0 else []) + \
+                 ([self.scale_token] if self.use_scale_token else [])
+        key = (B, first, first_scale, tuple((t._version, t.data_ptr(), t.dtype) for t in params))
+        hit = self.__dict__.get("_special_cache")
+        if hit is not None and hit[0] == key and not torch.is_grad_enabled():
+            return hit[1]
         index = cached + torch.arange(S, device=self.camera_token.device)
         parts = [_first_then_rest(self.camera_token, index < 1)]
         if self.num_register_tokens > 0:
@@ -219,6 +229,8 @@ class HipAggregatorStream(nn.Module):
             parts.append(_first_then_rest(self.scale_token, index < max(min(scale_frames, cached + S), 1)))
         tokens = torch.cat(parts, dim=1)                                   # [S, n, C]
         tokens = tokens.unsqueeze(0).expand(B, -1, -1, -1).reshape(B * S, self.num_special_tokens, C)
+        if not torch.is_grad_enabled():
+            self.__dict__["_special_cache"] = (key, tokens)
         return tokens
 
     def _embed_images(self, images: Tensor, num_frame_for_scale: Optional[int] = None):
@@ -241,9 +253,15 @@ class HipAggregatorStream(nn.Module):
         shifted by one (base.py:416-440)."""
         if self.rope is None:
             return None
+        key = (frames, H, W, str(device))
+        hit = self.__dict__.get("_positions_cache")
+        if hit is not None and hit[0] == key:      # the same tensor again: the rotary table derived from it is reused too
+            return hit[1]
         pos = self.position_getter(frames, H // self.patch_size, W // self.patch_size, device=device) + 1
         zeros = torch.zeros(frames, self.patch_start_idx, 2, dtype=pos.dtype, device=device)
-        return torch.cat([zeros, pos], dim=1)
+        pos = torch.cat([zeros, pos], dim=1)
+        self.__dict__["_positions_cache"] = (key, pos)
+        return pos
 
     # ------------------------------------------------------------------ forward
     def stream_table(self, frames: int, H: int, W: int, device, first_frame: Optional[int] = None) -> Optional[Tensor]:
