@@ -214,17 +214,21 @@ int lbm_qkv_linear_prepare(const void* a, const void* w, const float* bias, int3
 /* A LayerNorm folded into the launch that consumes its output.  lbm_linear with the residual
  * epilogue can leave behind, for every row of its output, one (mean, M2 = sum of squared
  * deviations from that mean) pair per column tile of the launch: out_stats [M][tiles][2] float32
- * with tiles = lbm_linear_stats_tiles(M, N).  A following launch that takes the output as its
- * activations normalises each row on the way into the multiply - LayerNorm(a) @ w^T - from those
- * pairs (merged as Chan et al.: equal-sized parts), so the normalised rows never go to memory and
- * the LayerNorm is no launch of its own.  Replaces norm2(x) in front of the MLP (block.py:194-195)
- * and norm1(x) of the block that follows (block.py:217).  The normalised value is
- * ((x * rstd - mean * rstd) * weight + bias) rounded to bf16.
- *   weight, bias  [K] bf16        stats  [M][stats_tiles][2] float32, stats_tiles divides K */
+ * with tiles = lbm_linear_stats_tiles(M, N).  A following launch that takes that output as its
+ * activations standardises each row, (x - mean) * rstd with rstd = 1 / sqrt(M2 / K + eps) merged
+ * from the pairs (Chan et al., equal-sized parts), without rewriting it: the product runs on the
+ * raw rows and the store applies  rstd * (a @ w^T - mean * w_colsum) + bias.  With the
+ * LayerNorm's weight g and bias c folded into the linear layer by the caller,
+ *     w[n][k] = W[n][k] * g[k] (rounded to bf16),  w_colsum[n] = sum_k w[n][k] (of the rounded
+ *     values),  bias[n] = B[n] + sum_k W[n][k] * c[k],
+ * that is LayerNorm(a) @ W^T + B with no launch and no memory traffic for the LayerNorm:
+ * norm2(x) in front of the MLP (block.py:194-195) and norm1(x) of the block that follows
+ * (block.py:217).  Unlike the separate ops the normalised rows are never rounded to bf16 (the
+ * weights' fold is instead): results agree with them to the last bf16 step or two.
+ *   stats  [M][stats_tiles][2] float32, stats_tiles divides K        w_colsum  [N] float32 */
 typedef struct lbm_row_norm {
-  const void* weight;
-  const void* bias;
   const float* stats;
+  const float* w_colsum;
   int32_t stats_tiles;
   float eps;
 } lbm_row_norm;
@@ -239,7 +243,8 @@ int lbm_linear_norm(const void* a, const lbm_row_norm* a_norm, const void* w, co
                     int32_t M, int32_t N, int32_t K, int32_t epilogue, void* stream);
 
 /* lbm_qkv_linear_prepare with a_norm (NULL = none) applied to the activations: norm1 of the
- * block, its qkv projection and the pre-attention producer as one launch. */
+ * block (folded as described at lbm_row_norm), its qkv projection and the pre-attention producer
+ * as one launch. */
 int lbm_qkv_linear_prepare_norm(const void* a, const lbm_row_norm* a_norm, const void* w,
                                 const float* bias, int32_t M, int32_t K, const float* q_norm_w,
                                 const float* q_norm_b, const float* k_norm_w, const float* k_norm_b,

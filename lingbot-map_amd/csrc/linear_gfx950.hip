@@ -45,7 +45,6 @@ constexpr int kGK = 128;         // k-step of the workgroup (64 per wave group)
 constexpr int kGStride = 136;    // bf16 per LDS row of a k-step (128 elements + 16 bytes: 272 B)
 constexpr int kGM = 128;         // activation rows per tile
 constexpr int kGThreads = 512;
-constexpr int kLnMaxK = 2048;    // widest input a folded LayerNorm is accepted for (its parameters sit in LDS)
 
 struct LinearArgs {
   const unsigned short* a;       // [M, K]
@@ -68,11 +67,11 @@ struct LinearArgs {
   const int32_t* append_rows;    // null: nothing is appended
   float eps;
   int num_heads, page_size;
-  // LNA kernels: the activations are LayerNorm'ed over K on their way into LDS, from row
-  // statistics the launch that produced them left behind (one (mean, M2) pair per row and
-  // column tile of that launch)
-  const unsigned short* ln_w;    // [K] bf16
-  const unsigned short* ln_b;    // [K] bf16
+  // LNA kernels: the rows of the activations are standardised, (x - mean) * rstd, without ever
+  // being rewritten: the product runs on the raw rows and the store applies
+  // rstd * (a @ w^T - mean * colsum(w)) + bias.  The statistics come from the launch that
+  // produced the activations (one (mean, M2) pair per row and column tile of that launch).
+  const float* ln_colsum;        // [N]: sum over k of w[n][k]
   const float* ln_stats;         // [M][ln_tiles][2]
   int ln_tiles;
   float ln_eps;
@@ -129,7 +128,7 @@ constexpr int kGeluEntries = 2 * kGeluHalf;
 // TN: output columns per tile (128 or 64); a wavefront owns 64 x (TN / 2) of the tile.
 // ROPE / NORM: rotary layout (0 none, 1 interleaved, 2 half-split) and qk-LayerNorm of the
 // kEpiQkvPrepare epilogue; 0 / false otherwise.
-// LNA: LayerNorm of the activations folded into their staging (see LinearArgs).
+// LNA: the activations' rows are standardised by the store (see LinearArgs).
 template <int EPI, int TN, int ROPE = 0, bool NORM = false, bool LNA = false>
 __global__ __launch_bounds__(kGThreads, 1) void lbm_linear_bf16_kernel(LinearArgs p) {
   constexpr int NT = TN / 64;   // 32-column blocks of W per wavefront
@@ -138,7 +137,6 @@ __global__ __launch_bounds__(kGThreads, 1) void lbm_linear_bf16_kernel(LinearArg
   __shared__ __attribute__((aligned(16))) unsigned short lds_w[2][TN * kGStride];
   __shared__ unsigned short gelu_tab[EPI == LBM_LINEAR_BIAS_GELU ? kGeluEntries : 1];
   __shared__ __attribute__((aligned(8))) float ln_rows[LNA ? kGM * 2 : 2];   // per row of the tile: rstd, -mean * rstd
-  __shared__ __attribute__((aligned(16))) unsigned short ln_wb[LNA ? 2 * kLnMaxK : 8];   // LayerNorm weight, then bias
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int n32 = lane & 31, g = lane >> 5;
@@ -178,37 +176,15 @@ __global__ __launch_bounds__(kGThreads, 1) void lbm_linear_bf16_kernel(LinearArg
   // written into the LDS buffer at the end of iteration s - 1, so a load has two multiply
   // phases to arrive before anything waits for it.
   u32x4 ra0[kPassA], rw0[kPassW], ra1[kPassA], rw1[kPassW];
-  // LNA: every staged piece of the activations is normalised before it goes to LDS:
-  // (x * rstd - mean * rstd) * w + b, the row's two factors and the weight and bias of the
-  // thread's 8 columns of k-step ks read from LDS
-  auto norm_piece = [&](const u32x4& raw, int j, int ks) -> u32x4 {
-    if (!LNA) return raw;
-    const f32x2 row = *(const f32x2*)&ln_rows[2 * (ld_r + 32 * j)];
-    const float ln_sc_j = row[0], ln_sh_j = row[1];
-    u32x4 ln[2];
-    ln[0] = *(const u32x4*)&ln_wb[ks * kGK + ld_c];
-    ln[1] = *(const u32x4*)&ln_wb[kLnMaxK + ks * kGK + ld_c];
-    u32x4 o;
-#pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      const float x0 = bf16_bits_to_f32(raw[e] & 0xffffu), x1 = __builtin_bit_cast(float, raw[e] & 0xffff0000u);
-      const float w0 = bf16_bits_to_f32(ln[0][e] & 0xffffu), w1 = __builtin_bit_cast(float, ln[0][e] & 0xffff0000u);
-      const float b0 = bf16_bits_to_f32(ln[1][e] & 0xffffu), b1 = __builtin_bit_cast(float, ln[1][e] & 0xffff0000u);
-      const float y0 = __builtin_fmaf(__builtin_fmaf(x0, ln_sc_j, ln_sh_j), w0, b0);
-      const float y1 = __builtin_fmaf(__builtin_fmaf(x1, ln_sc_j, ln_sh_j), w1, b1);
-      o[e] = (unsigned)__builtin_bit_cast(unsigned short, (__bf16)y0) | ((unsigned)__builtin_bit_cast(unsigned short, (__bf16)y1) << 16);
-    }
-    return o;
-  };
   auto load_step = [&](int ks, u32x4 (&ra)[kPassA], u32x4 (&rw)[kPassW]) {
 #pragma unroll
     for (int j = 0; j < kPassA; ++j) ra[j] = load_a(j, ks);
 #pragma unroll
     for (int j = 0; j < kPassW; ++j) rw[j] = load_w(j, ks);
   };
-  auto store_step = [&](int buf, const u32x4 (&ra)[kPassA], const u32x4 (&rw)[kPassW], int ks) {
+  auto store_step = [&](int buf, const u32x4 (&ra)[kPassA], const u32x4 (&rw)[kPassW]) {
 #pragma unroll
-    for (int j = 0; j < kPassA; ++j) *(u32x4*)&lds_a[buf][(ld_r + 32 * j) * kGStride + ld_c] = norm_piece(ra[j], j, ks);
+    for (int j = 0; j < kPassA; ++j) *(u32x4*)&lds_a[buf][(ld_r + 32 * j) * kGStride + ld_c] = ra[j];
 #pragma unroll
     for (int j = 0; j < kPassW; ++j) *(u32x4*)&lds_w[buf][(ld_r + 32 * j) * kGStride + ld_c] = rw[j];
   };
@@ -225,8 +201,7 @@ __global__ __launch_bounds__(kGThreads, 1) void lbm_linear_bf16_kernel(LinearArg
   // and the rows of the step after next (held in `ra`, `rw` since the previous iteration) go
   // into the other LDS buffer two stores per slice, in the shadow of the MFMAs, followed by the
   // loads that refill the set.  sched_barrier keeps the slices as written.
-  // (`held_ks`: the k-step whose rows `ra`, `rw` hold on entry)
-  auto step = [&](int buf, u32x4 (&ra)[kPassA], u32x4 (&rw)[kPassW], int held_ks, int next_ks) {
+  auto step = [&](int buf, u32x4 (&ra)[kPassA], u32x4 (&rw)[kPassW], int next_ks) {
     const unsigned short* la = &lds_a[buf][kh * 64];
     const unsigned short* lw = &lds_w[buf][kh * 64];
     bf16x8 wf[2][NT], af[2][2];
@@ -251,7 +226,7 @@ __global__ __launch_bounds__(kGThreads, 1) void lbm_linear_bf16_kernel(LinearArg
       // they put a repeat of it into a buffer nobody reads any more: cheaper than a branch per slice)
 #pragma unroll
       for (int j = 0; j < kPassA; ++j)
-        if ((j & 3) == k16) *(u32x4*)&lds_a[buf ^ 1][(ld_r + 32 * j) * kGStride + ld_c] = norm_piece(ra[j], j, held_ks);
+        if ((j & 3) == k16) *(u32x4*)&lds_a[buf ^ 1][(ld_r + 32 * j) * kGStride + ld_c] = ra[j];
 #pragma unroll
       for (int j = 0; j < kPassW; ++j)
         if ((j & 3) == k16) *(u32x4*)&lds_w[buf ^ 1][(ld_r + 32 * j) * kGStride + ld_c] = rw[j];
@@ -270,10 +245,6 @@ __global__ __launch_bounds__(kGThreads, 1) void lbm_linear_bf16_kernel(LinearArg
   load_step(0, ra0, rw0);
   load_step(min(1, last), ra1, rw1);
   if (LNA) {
-    for (int i = tid * 8; i < p.K; i += kGThreads * 8) {
-      *(u32x4*)&ln_wb[i] = *(const u32x4*)(p.ln_w + i);
-      *(u32x4*)&ln_wb[kLnMaxK + i] = *(const u32x4*)(p.ln_b + i);
-    }
     // Row statistics: row r of the tile is handled by threads 4 r .. 4 r + 3, each taking every
     // fourth (mean, M2) partial; equal-sized partials merge as mean = avg(mean_i),
     // M2 = sum(M2_i) + n_i * sum((mean_i - mean)^2) (Chan et al.), variance = M2 / K.
@@ -297,7 +268,7 @@ __global__ __launch_bounds__(kGThreads, 1) void lbm_linear_bf16_kernel(LinearArg
       ln_rows[2 * r] = rstd;
       ln_rows[2 * r + 1] = -mean * rstd;
     }
-    __syncthreads();
+    // (read in the epilogue, many barriers from here)
   }
   if (EPI == LBM_LINEAR_BIAS_GELU) {
     // (under the latency of the loads above; the barrier before the first multiply publishes it)
@@ -307,16 +278,16 @@ __global__ __launch_bounds__(kGThreads, 1) void lbm_linear_bf16_kernel(LinearArg
       gelu_tab[i] = __builtin_bit_cast(unsigned short, (__bf16)gelu_erf(bf16_bits_to_f32(bits)));
     }
   }
-  store_step(0, ra0, rw0, 0);
+  store_step(0, ra0, rw0);
   load_step(min(2, last), ra0, rw0);
   __syncthreads();
   // iteration ks multiplies buffer ks & 1 and moves the set holding step ks + 1 into the other
   // buffer, then refills that set with step ks + 3
   for (int ks = 0; ks < nk; ks += 2) {
-    step(0, ra1, rw1, min(ks + 1, last), min(ks + 3, last));
+    step(0, ra1, rw1, min(ks + 3, last));
     __syncthreads();
     if (ks + 1 >= nk) break;
-    step(1, ra0, rw0, min(ks + 2, last), min(ks + 4, last));
+    step(1, ra0, rw0, min(ks + 4, last));
     __syncthreads();
   }
 
@@ -347,19 +318,24 @@ __global__ __launch_bounds__(kGThreads, 1) void lbm_linear_bf16_kernel(LinearArg
   // Then the tile goes through LDS and leaves as whole rows.
   constexpr int kCStride = TN + 4;   // bf16 per staged row: 8-byte writes of 32 rows hit 64 distinct banks
   unsigned short* stage = (unsigned short*)&lds_w[0][0];
+  f32x2 row_f = {1.f, 0.f};   // this lane's output row: rstd, -mean * rstd
+  if (LNA) row_f = *(const f32x2*)&ln_rows[2 * (wm + b * 32 + n32)];
   static_assert(kGM * kCStride * 2 <= (int)sizeof(lds_w), "the staged tile fits the weight buffers");
 #pragma unroll
   for (int a = 0; a < NT; ++a)
 #pragma unroll
     for (int c4 = 0; c4 < 4; ++c4) {
       const int col = wn + a * 32 + c4 * 8 + g * 4;     // four consecutive output columns
-      f32x4 bias4 = {0.f, 0.f, 0.f, 0.f}, gamma4 = {1.f, 1.f, 1.f, 1.f};
+      f32x4 bias4 = {0.f, 0.f, 0.f, 0.f}, gamma4 = {1.f, 1.f, 1.f, 1.f}, colsum4 = {0.f, 0.f, 0.f, 0.f};
       if (p.bias) bias4 = *(const f32x4*)(p.bias + n0 + col);
+      if (LNA) colsum4 = *(const f32x4*)(p.ln_colsum + n0 + col);
       if (EPI == LBM_LINEAR_BIAS_RESIDUAL && p.gamma) gamma4 = *(const f32x4*)(p.gamma + n0 + col);
       f32x4 y;
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
-        float v = round_bf16(fin[a][c4 * 4 + e] + bias4[e]);
+        float lin = fin[a][c4 * 4 + e];
+        if (LNA) lin = __builtin_fmaf(lin, row_f[0], row_f[1] * colsum4[e]);   // rstd * acc - mean * rstd * colsum
+        float v = round_bf16(lin + bias4[e]);
         if (EPI == LBM_LINEAR_BIAS_GELU) {
           const unsigned b16 = __builtin_bit_cast(unsigned, v) >> 16;
           const unsigned rel = (b16 & 0x7fffu) - (unsigned)(kGeluE0 << 7);
@@ -505,13 +481,10 @@ namespace {
 // the folded LayerNorm of the activations, checked and copied into the kernel arguments
 int lbm_set_row_norm(LinearArgs& p, const lbm_row_norm* ln, const char* who) {
   if (!ln) return LBM_OK;
-  if (p.K > kLnMaxK)
-    return lbm_fail(LBM_ERR_UNSUPPORTED, "%s: a folded LayerNorm takes inputs up to %d wide (got %d)", who, kLnMaxK, p.K);
-  if (!ln->weight || !ln->bias || !ln->stats || ln->stats_tiles <= 0 || p.K % ln->stats_tiles != 0)
-    return lbm_fail(LBM_ERR_INVALID, "%s: the folded LayerNorm needs weight, bias, stats and a tile count that divides K (got %d for K %d)",
+  if (!ln->w_colsum || !ln->stats || ln->stats_tiles <= 0 || p.K % ln->stats_tiles != 0)
+    return lbm_fail(LBM_ERR_INVALID, "%s: standardised rows need w_colsum, stats and a tile count that divides K (got %d for K %d)",
                     who, ln->stats_tiles, p.K);
-  p.ln_w = (const unsigned short*)ln->weight;
-  p.ln_b = (const unsigned short*)ln->bias;
+  p.ln_colsum = ln->w_colsum;
   p.ln_stats = ln->stats;
   p.ln_tiles = ln->stats_tiles;
   p.ln_eps = ln->eps;
@@ -533,7 +506,7 @@ int lbm_launch_linear(const void* a, const lbm_row_norm* a_norm, const void* w, 
   if (K % kGK != 0 || N % 64 != 0)
     return lbm_fail(LBM_ERR_UNSUPPORTED, "lbm_linear: K must be a multiple of 128 and N of 64 (got K %d, N %d)", K, N);
   if (a_norm && epilogue == LBM_LINEAR_BIAS_RESIDUAL)
-    return lbm_fail(LBM_ERR_UNSUPPORTED, "lbm_linear: no folded LayerNorm with the residual epilogue");
+    return lbm_fail(LBM_ERR_UNSUPPORTED, "lbm_linear: no row standardisation with the residual epilogue");
   if (out_stats && epilogue != LBM_LINEAR_BIAS_RESIDUAL)
     return lbm_fail(LBM_ERR_UNSUPPORTED, "lbm_linear: row statistics come with the residual epilogue only");
   LinearArgs p = {};

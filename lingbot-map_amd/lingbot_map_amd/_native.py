@@ -43,8 +43,7 @@ class AttnStream(C.Structure):
 
 class RowNorm(C.Structure):
     """``lbm_row_norm``: a LayerNorm folded into the launch that consumes its output."""
-    _fields_ = [("weight", C.c_void_p), ("bias", C.c_void_p), ("stats", C.c_void_p),
-                ("stats_tiles", C.c_int32), ("eps", C.c_float)]
+    _fields_ = [("stats", C.c_void_p), ("w_colsum", C.c_void_p), ("stats_tiles", C.c_int32), ("eps", C.c_float)]
 
 
 SYMBOLS = ("lbm_abi_version", "lbm_last_error", "lbm_tables_words", "lbm_tables_step",

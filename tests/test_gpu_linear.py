@@ -225,9 +225,15 @@ def test_qkv_projection_with_the_producer_as_its_epilogue(M, H, K, norm, rope):
     assert bad(ptr(a), ptr(w), None, M, K, None, None, None, None, 1e-5, None, 0, ptr(q1), None, None, None, ptr(rows), H, D, S, None)  # rows without pool
 
 
-def _row_norm(N, weight, bias, stats, tiles, eps=1e-5):
-    import ctypes as C
-    return N.RowNorm(weight.data_ptr(), bias.data_ptr(), stats.data_ptr(), tiles, eps)
+def _row_norm(N, stats, colsum, tiles, eps=1e-5):
+    return N.RowNorm(stats.data_ptr(), colsum.data_ptr(), tiles, eps)
+
+
+def _fold(lw, lb, w, bias):
+    """The LayerNorm's weight and bias folded into a linear layer, as lbm_row_norm asks the caller
+    to: weight (bf16), its row sums (of the rounded values), bias."""
+    wf = (w.float() * lw.float()[None, :]).to(torch.bfloat16)
+    return wf, wf.float().sum(dim=1).contiguous(), (bias.float() + w.float() @ lb.float()).contiguous()
 
 
 @pytest.mark.parametrize("M,K,Nn", [(1004, 4096, 1024), (1004, 1024, 1024), (130, 256, 256), (1, 128, 64)])
@@ -258,7 +264,7 @@ def test_residual_epilogue_leaves_row_statistics(M, K, Nn):
     assert ((got[..., 1] - m2).abs() <= 1e-4 * m2.clamp_min(1e-3)).all()
     # statistics only come with the residual epilogue, a folded LayerNorm never with it
     assert N.lib.lbm_linear_norm(ptr(ad), None, ptr(wd), ptr(bd), None, None, ptr(out), ptr(stats), M, Nn, K, N.LINEAR_BIAS, None) != N.OK
-    ln = _row_norm(N, gd, gd, stats, tiles)
+    ln = _row_norm(N, stats, gd, tiles)
     assert N.lib.lbm_linear_norm(ptr(ad), ln, ptr(wd), ptr(bd), ptr(gd), ptr(rd), ptr(out), None, M, Nn, K, N.LINEAR_BIAS_RESIDUAL, None) != N.OK
 
 
@@ -272,9 +278,12 @@ def _stats_of(x, tiles):
 @pytest.mark.parametrize("M,K,Nn,tiles,epilogue", [(1004, 1024, 4096, 16, 1), (1004, 1024, 3072, 8, 0), (200, 256, 128, 4, 1),
                                                    (77, 2048, 64, 32, 0)])
 def test_layernorm_folded_into_the_linear(M, K, Nn, tiles, epilogue):
-    """lbm_linear_norm with a_norm against LayerNorm (torch, bf16 in and out) followed by the plain
-    lbm_linear arithmetic on the CPU: the normalised activations may land on the neighbouring bf16
-    value for a few elements in a hundred thousand (the statistics are merged from per-tile parts)."""
+    """lbm_linear_norm with a_norm (the LayerNorm's affine part folded into weight and bias by the
+    caller) against LayerNorm (torch, bf16 in and out) followed by the plain lbm_linear arithmetic
+    on the CPU.  The two round in different places - the normalised rows there, the folded weights
+    here - so the two differ by the accumulated rounding noise of 1,024 products (a few 1e-3, the worst
+    of millions of outputs 3e-2) on top of the output's own rounding; the mean difference stays a
+    fraction of a bf16 step, and against float64 arithmetic the folded form is the closer of the two."""
     N = _native()
     dev = torch.device("cuda:0")
     g = torch.Generator().manual_seed(M + K + Nn)
@@ -284,34 +293,33 @@ def test_layernorm_folded_into_the_linear(M, K, Nn, tiles, epilogue):
     w = (torch.randn(Nn, K, generator=g) / K ** 0.5).to(torch.bfloat16)
     bias = (0.1 * torch.randn(Nn, generator=g)).to(torch.bfloat16)
     normed = torch.nn.functional.layer_norm(x.float(), (K,), lw.float(), lb.float(), 1e-5).to(torch.bfloat16)
-    ref = expected(normed, w, bias, epilogue)
+    ref = expected(normed, w, bias, epilogue).float()
+    pre = expected(normed, w, bias, N.LINEAR_BIAS).float()
+    exact = torch.nn.functional.layer_norm(x.double(), (K,), lw.double(), lb.double(), 1e-5) @ w.double().t() + bias.double()
+    if epilogue == N.LINEAR_BIAS_GELU:
+        exact = torch.nn.functional.gelu(exact)
+    wf, colsum, bf = _fold(lw, lb, w, bias)
     stats = _stats_of(x, tiles).to(dev)
-    xd, lwd, lbd, wd, bd = x.to(dev), lw.to(dev), lb.to(dev), w.to(dev), bias.float().to(dev)
-    ln = _row_norm(N, lwd, lbd, stats, tiles)
+    xd, wd, cd, bd = x.to(dev), wf.to(dev), colsum.to(dev), bf.to(dev)
+    ln = _row_norm(N, stats, cd, tiles)
     out = torch.full((M, Nn), float("nan"), dtype=torch.bfloat16, device=dev)
     N.check(N.lib.lbm_linear_norm(ptr(xd), ln, ptr(wd), ptr(bd), None, None, ptr(out), None, M, Nn, K, epilogue, None))
     torch.cuda.synchronize()
-    # an activation on the neighbouring bf16 value moves a sum by up to ulp(activation) * |weight|
-    # (an absolute term), and a sum pushed over a rounding boundary that way can end two bf16
-    # steps of the pre-activation away after the GELU; nearly all elements are equal
-    got, pre = out.cpu().float(), expected(normed, w, bias, N.LINEAR_BIAS).float()
+    got = out.cpu().float()
     assert torch.isfinite(got).all()
-    err = (got - ref.float()).abs()
-    assert (err <= 2.0 ** -6 * pre.abs() + 2.0 ** -8 + 2e-3).all(), err.max().item()
-    assert (got != ref.float()).float().mean().item() < 0.03
-    assert err.mean().item() <= 2.0 ** -12 * pre.abs().mean().item()
-    # wider than the LDS copy of the LayerNorm parameters holds
-    big = torch.zeros(8, 4096, dtype=torch.bfloat16, device=dev)
-    st = torch.zeros(8, 8, 2, device=dev)
-    p4 = torch.zeros(4096, dtype=torch.bfloat16, device=dev)
-    w4 = torch.zeros(64, 4096, dtype=torch.bfloat16, device=dev)
-    o4 = torch.zeros(8, 64, dtype=torch.bfloat16, device=dev)
-    assert N.lib.lbm_linear_norm(ptr(big), _row_norm(N, p4, p4, st, 8), ptr(w4), None, None, None, ptr(o4), None, 8, 64, 4096, 0, None) != N.OK
+    err = (got - ref).abs()
+    assert (err <= 2.0 ** -6 * pre.abs() + 2.0 ** -5).all(), err.max().item()       # the worst of a few million
+    assert err.mean().item() <= 2.0 ** -8 * pre.abs().mean().item(), (err.mean().item(), pre.abs().mean().item())
+    assert (got.double() - exact).abs().mean().item() <= 1.05 * (ref.double() - exact).abs().mean().item()
+    # a tile count that does not divide K, missing column sums
+    assert N.lib.lbm_linear_norm(ptr(xd), _row_norm(N, stats, cd, 7), ptr(wd), ptr(bd), None, None, ptr(out), None, M, Nn, K, epilogue, None) != N.OK
+    assert N.lib.lbm_linear_norm(ptr(xd), N.RowNorm(stats.data_ptr(), None, tiles, 1e-5), ptr(wd), ptr(bd), None, None, ptr(out), None, M, Nn, K, epilogue, None) != N.OK
 
 
 def test_layernorm_folded_into_the_qkv_projection_and_producer():
-    """lbm_qkv_linear_prepare_norm against the same launch fed with the LayerNorm computed by
-    torch: q, k, v within one bf16 step, almost all equal."""
+    """lbm_qkv_linear_prepare_norm (norm1 folded into the projection) against the same launch fed
+    with the LayerNorm computed by torch: q, k, v agree to a bf16 step of the largest values, the
+    mean difference a small fraction of that."""
     N = _native()
     dev = torch.device("cuda:0")
     M, H, K, D, S, tiles = 1004, 16, 1024, 64, 16, 16
@@ -319,29 +327,30 @@ def test_layernorm_folded_into_the_qkv_projection_and_producer():
     x = (torch.randn(M, K, generator=g) * 1.7 + 0.2).to(torch.bfloat16)
     lw = (1 + 0.2 * torch.randn(K, generator=g)).to(torch.bfloat16)
     lb = (0.1 * torch.randn(K, generator=g)).to(torch.bfloat16)
-    w = (torch.randn(3 * H * D, K, generator=g) / K ** 0.5).to(torch.bfloat16).to(dev)
-    bias = (0.1 * torch.randn(3 * H * D, generator=g)).to(dev)
+    w = (torch.randn(3 * H * D, K, generator=g) / K ** 0.5).to(torch.bfloat16)
+    bias = 0.1 * torch.randn(3 * H * D, generator=g)
     qk = [(1 + 0.2 * torch.randn(D, generator=g)).to(dev) if i % 2 == 0 else (0.1 * torch.randn(D, generator=g)).to(dev) for i in range(4)]
     ang = torch.rand(M, D // 2, generator=g) * 6.283185
     cs = torch.stack([ang.cos(), ang.sin()], dim=-1).contiguous().to(dev)
     normed = torch.nn.functional.layer_norm(x.float(), (K,), lw.float(), lb.float(), 1e-5).to(torch.bfloat16).to(dev)
+    wf, colsum, bf = _fold(lw, lb, w, bias)
     outs = []
     for fold in (False, True):
         q, k, v = (torch.full((M, H, D), float("nan"), dtype=torch.bfloat16, device=dev) for _ in range(3))
         if fold:
-            xd, lwd, lbd, stats = x.to(dev), lw.to(dev), lb.to(dev), _stats_of(x, tiles).to(dev)
-            ln = _row_norm(N, lwd, lbd, stats, tiles)
-            N.check(N.lib.lbm_qkv_linear_prepare_norm(ptr(xd), ln, ptr(w), ptr(bias), M, K, *[ptr(t) for t in qk], 1e-5, ptr(cs),
+            xd, wd, cd, bd, stats = x.to(dev), wf.to(dev), colsum.to(dev), bf.to(dev), _stats_of(x, tiles).to(dev)
+            ln = _row_norm(N, stats, cd, tiles)
+            N.check(N.lib.lbm_qkv_linear_prepare_norm(ptr(xd), ln, ptr(wd), ptr(bd), M, K, *[ptr(t) for t in qk], 1e-5, ptr(cs),
                                                       N.ROPE_INTERLEAVED, ptr(q), ptr(k), ptr(v), None, None, H, D, S, None))
         else:
-            N.check(N.lib.lbm_qkv_linear_prepare(ptr(normed), ptr(w), ptr(bias), M, K, *[ptr(t) for t in qk], 1e-5, ptr(cs),
+            wd, bd = w.to(dev), bias.to(dev)
+            N.check(N.lib.lbm_qkv_linear_prepare(ptr(normed), ptr(wd), ptr(bd), M, K, *[ptr(t) for t in qk], 1e-5, ptr(cs),
                                                  N.ROPE_INTERLEAVED, ptr(q), ptr(k), ptr(v), None, None, H, D, S, None))
         torch.cuda.synchronize()
         outs.append([t.float().cpu() for t in (q, k, v)])
     for a0, a1 in zip(*outs):
         assert torch.isfinite(a1).all()
-        # q and k come out of a LayerNorm over the head: a projection that moved by one rounding
-        # moves every element of its head a little and the rotation mixes pairs, so the bar has an absolute part of one bf16
-        # step of the largest values (2 to 4)
-        assert ((a0 - a1).abs() <= 2.0 ** -7 * a0.abs() + 2.0 ** -6).all(), (a0 - a1).abs().max().item()
-        assert (a0 != a1).float().mean().item() < 0.05
+        # q and k come out of a LayerNorm over the head and a rotation that mixes pairs: the bar has
+        # an absolute part for the worst of three million elements (the noise of 1,024 products, 5 sigma)
+        assert ((a0 - a1).abs() <= 2.0 ** -6 * a0.abs() + 2.0 ** -4).all(), (a0 - a1).abs().max().item()
+        assert (a0 - a1).abs().mean().item() <= 2.0 ** -9 * a0.abs().mean().item() + 1e-3
