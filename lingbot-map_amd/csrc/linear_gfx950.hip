@@ -242,24 +242,42 @@ __global__ __launch_bounds__(kGThreads, 1) void lbm_linear_bf16_kernel(LinearArg
 
   const int nk = p.K / kGK;
   const int last = nk - 1;                       // steps past the end re-read the last one (never multiplied)
+  // LNA, row statistics: row r of the tile is handled by threads 4 r .. 4 r + 3, each taking every
+  // fourth (mean, M2) partial; equal-sized partials merge as mean = avg(mean_i),
+  // M2 = sum(M2_i) + n_i * sum((mean_i - mean)^2) (Chan et al.), variance = M2 / K.  The partials
+  // are asked for before the operand tiles (loads return in order) and merged while those travel.
+  constexpr int kLnHeld = 4;     // partials a thread keeps in registers (up to 16 column tiles)
+  f32x2 ln_part[kLnHeld] = {};
+  const float* ln_st = nullptr;
+  if (LNA) {
+    ln_st = p.ln_stats + (size_t)min(m0 + (tid >> 2), p.M - 1) * p.ln_tiles * 2;
+#pragma unroll
+    for (int i = 0; i < kLnHeld; ++i)
+      if ((tid & 3) + 4 * i < p.ln_tiles) ln_part[i] = *(const f32x2*)(ln_st + 2 * ((tid & 3) + 4 * i));
+  }
   load_step(0, ra0, rw0);
   load_step(min(1, last), ra1, rw1);
   if (LNA) {
-    // Row statistics: row r of the tile is handled by threads 4 r .. 4 r + 3, each taking every
-    // fourth (mean, M2) partial; equal-sized partials merge as mean = avg(mean_i),
-    // M2 = sum(M2_i) + n_i * sum((mean_i - mean)^2) (Chan et al.), variance = M2 / K.
     const int r = tid >> 2, part = tid & 3;
-    const float* st = p.ln_stats + (size_t)min(m0 + r, p.M - 1) * p.ln_tiles * 2;
     float sm = 0.f;
-    for (int i = part; i < p.ln_tiles; i += 4) sm += st[2 * i];
+#pragma unroll
+    for (int i = 0; i < kLnHeld; ++i)
+      if (part + 4 * i < p.ln_tiles) sm += ln_part[i][0];
+    for (int i = part + 4 * kLnHeld; i < p.ln_tiles; i += 4) sm += ln_st[2 * i];
     sm += __shfl_xor(sm, 1);
     sm += __shfl_xor(sm, 2);
     const float mean = sm / (float)p.ln_tiles;
     const float n_i = (float)p.K / (float)p.ln_tiles;
     float m2 = 0.f;
-    for (int i = part; i < p.ln_tiles; i += 4) {
-      const float d = st[2 * i] - mean;
-      m2 += st[2 * i + 1] + n_i * d * d;
+#pragma unroll
+    for (int i = 0; i < kLnHeld; ++i)
+      if (part + 4 * i < p.ln_tiles) {
+        const float d = ln_part[i][0] - mean;
+        m2 += ln_part[i][1] + n_i * d * d;
+      }
+    for (int i = part + 4 * kLnHeld; i < p.ln_tiles; i += 4) {
+      const float d = ln_st[2 * i] - mean;
+      m2 += ln_st[2 * i + 1] + n_i * d * d;
     }
     m2 += __shfl_xor(m2, 1);
     m2 += __shfl_xor(m2, 2);

@@ -64,7 +64,7 @@ class PatchTrunk(nn.Module):
         for i, blk in enumerate(self.blocks):   # each block hands the next one its norm1 (or the final norm)
             nxt = self.blocks[i + 1].norm1 if i + 1 < len(self.blocks) else self.norm
             x, normed = blk(x, normed=normed, next_norm=nxt)
-        return normed if len(self.blocks) else self.norm(x)
+        return normed if torch.is_tensor(normed) else self.norm(x)   # (row statistics: nobody left to fold them)
 
 
 def _first_then_rest(token: Tensor, first: Tensor) -> Tensor:
@@ -311,14 +311,14 @@ class HipAggregatorStream(nn.Module):
             for kind in self.aa_order:
                 if kind == "frame":
                     tokens = tokens.reshape(B * S, P, C)
-                    normed = normed.reshape(B * S, P, C) if normed is not None else None
+                    normed = normed.reshape(B * S, P, C) if torch.is_tensor(normed) else normed
                     for _ in range(self.aa_block_size):
                         tokens, normed = run(self.frame_blocks[frame_idx], tokens, normed, pos=pos)
                         frame_idx += 1
                         frame_out.append(tokens.view(B, S, P, C))
                 else:
                     tokens = tokens.reshape(B, S * P, C)
-                    normed = normed.reshape(B, S * P, C) if normed is not None else None
+                    normed = normed.reshape(B, S * P, C) if torch.is_tensor(normed) else normed
                     first_group = global_idx < self.aa_block_size
                     if self.rope3d is not None:     # frame index = frames streamed so far (stream.py:464-478)
                         if first_group:

@@ -189,6 +189,46 @@ class LayerScale(nn.Module):
         return x * self.gamma
 
 
+class RowStats:
+    """What a block hands the next one in place of ``norm1(x)``: per row of ``x`` and column tile of
+    the launch that wrote it, the mean and the sum of squared deviations (``lbm_linear_norm``'s
+    ``out_stats``).  The consumer folds its LayerNorm into its linear layer (``FoldedNorm``) and
+    reads ``x`` itself."""
+
+    def __init__(self, stats: Tensor, tiles: int) -> None:
+        self.stats, self.tiles = stats, tiles
+
+
+class FoldedNorm:
+    """A LayerNorm folded into the linear layer behind it: ``linear(norm(x))`` =
+    ``rstd * (x @ w^T - mean * colsum) + bias`` with ``w = W * g`` (bf16), ``colsum`` its row sums
+    and ``bias = B + W @ c`` for the LayerNorm's weight ``g`` and bias ``c``.  Kept per (norm,
+    linear) pair until one of the four parameters changes."""
+
+    @staticmethod
+    def possible(norm, linear: nn.Linear) -> bool:
+        return (type(norm) is nn.LayerNorm and norm.elementwise_affine and norm.bias is not None
+                and tuple(norm.normalized_shape) == (linear.in_features,) and linear.weight.dtype == torch.bfloat16
+                and linear.weight.is_cuda and linear.in_features % 128 == 0 and linear.out_features % 64 == 0)
+
+    @staticmethod
+    def of(owner: nn.Module, norm: nn.LayerNorm, linear: nn.Linear):
+        """(weight bf16 [N, K], colsum float32 [N], bias float32 [N])"""
+        ts = [norm.weight, norm.bias, linear.weight] + ([linear.bias] if linear.bias is not None else [])
+        key = tuple((t._version, t.data_ptr(), t.device) for t in ts)
+        cache = owner.__dict__.setdefault("_folded_norms", {})
+        hit = cache.get((id(norm), id(linear)))
+        if hit is None or hit[0] != key:
+            with torch.no_grad():
+                W = linear.weight.detach().float()
+                w = (W * norm.weight.detach().float()[None, :]).to(torch.bfloat16).contiguous()
+                bias = W @ norm.bias.detach().float()
+                if linear.bias is not None:
+                    bias = bias + linear.bias.detach().float()
+                hit = cache[(id(norm), id(linear))] = (key, (w, w.float().sum(dim=1).contiguous(), bias.contiguous()))
+        return hit[1]
+
+
 class Mlp(nn.Module):
     """lingbot_map/layers/mlp.py (dropout omitted: inference only)"""
 
@@ -221,19 +261,24 @@ class Mlp(nn.Module):
             cache[id(m)] = (key, m.bias.detach().float().contiguous())
         return cache[id(m)][1]
 
-    def fc1_gelu(self, x: Tensor) -> Tensor:
+    def fc1_gelu(self, x: Tensor, norm: Optional[nn.LayerNorm] = None, stats: Optional[RowStats] = None) -> Tensor:
         """``act(fc1(x))`` as one kernel: the GEMM with bias and the exact GELU in its store
-        (mlp.py:35-36), roundings as the two separate bf16 torch ops."""
+        (mlp.py:35-36), roundings as the two separate bf16 torch ops.  With ``norm`` and ``stats``:
+        ``act(fc1(norm(x)))``, the LayerNorm folded into the launch (block.py:194-195)."""
         import ctypes as C
         from . import _native as N
         fc1 = self.fc1
         a = x.reshape(-1, fc1.in_features).contiguous()
-        w = fc1.weight if fc1.weight.is_contiguous() else fc1.weight.contiguous()
-        bias = self._bias_f32(fc1)
         out = torch.empty(a.shape[0], fc1.out_features, dtype=x.dtype, device=x.device)
         p = lambda t: None if t is None else C.c_void_p(t.data_ptr())
-        N.check(N.lib.lbm_linear(p(a), p(w), p(bias), None, None, p(out), a.shape[0], fc1.out_features, fc1.in_features,
-                                 N.LINEAR_BIAS_GELU, N.stream_ptr(x.device)))
+        if norm is None:
+            w = fc1.weight if fc1.weight.is_contiguous() else fc1.weight.contiguous()
+            bias, row_norm = self._bias_f32(fc1), None
+        else:
+            w, colsum, bias = FoldedNorm.of(self, norm, fc1)
+            row_norm = N.RowNorm(stats.stats.data_ptr(), colsum.data_ptr(), stats.tiles, float(norm.eps))
+        N.check(N.lib.lbm_linear_norm(p(a), row_norm, p(w), p(bias), None, None, p(out), None, a.shape[0], fc1.out_features,
+                                      fc1.in_features, N.LINEAR_BIAS_GELU, N.stream_ptr(x.device)))
         return out.reshape(*x.shape[:-1], fc1.out_features)
 
     def forward(self, x: Tensor) -> Tensor:
@@ -334,11 +379,12 @@ class HipPagedAttention(nn.Module):
             cache[id(m)] = (key, (m.weight.detach().float().contiguous(), m.bias.detach().float().contiguous()))
         return cache[id(m)][1]
 
-    def stream_attend_fused(self, manager, global_idx: int, x: Tensor, pos=None) -> Tensor:
+    def stream_attend_fused(self, manager, global_idx: int, x: Tensor, pos=None, norm=None, stats=None) -> Tensor:
         """qkv projection, then one kernel for q/k LayerNorm + rotary embedding + layout +
-        paged append, then the paged attention (attention.py:402-426 and block.py:256-278)."""
+        paged append, then the paged attention (attention.py:402-426 and block.py:256-278).
+        ``norm``, ``stats``: ``x`` is the block's input and ``norm`` is folded into the projection."""
         B, N, _ = x.shape
-        proj = self._fused_projection(x, manager.dtype)
+        proj = self._fused_projection(x, manager.dtype, norm, stats)
         qkv = None if proj is not None else self.qkv(x).reshape(B * N, -1)
         has_norm = isinstance(self.q_norm, nn.LayerNorm)
         rope_cs = None
@@ -357,10 +403,19 @@ class HipPagedAttention(nn.Module):
     #: call; at several streams' rows the library GEMM's larger tiles win)
     FUSED_PROJ_MAX_ROWS = 1280
 
-    def _fused_projection(self, x: Tensor, cache_dtype) -> Optional[tuple]:
+    def _fused_projection(self, x: Tensor, cache_dtype, norm: Optional[nn.LayerNorm] = None,
+                          stats: Optional[RowStats] = None) -> Optional[tuple]:
         """(x [rows, K], weight, float32 bias) for ``lbm_qkv_linear_prepare`` when the projection
         can run in the producer's kernel: bf16 activations, weights and cache, head_dim 64, K a
-        multiple of 128, one frame's worth of rows; None otherwise (the caller projects first)."""
+        multiple of 128, one frame's worth of rows; None otherwise (the caller projects first).
+        With ``norm`` and ``stats`` (``x`` is then the block's input, not ``norm(x)``) a fourth
+        element: the ``lbm_row_norm`` of ``lbm_qkv_linear_prepare_norm``, weight and bias folded."""
+        if norm is not None:
+            from . import _native as N
+            rows = x.numel() // x.shape[-1]
+            w, colsum, bias = FoldedNorm.of(self, norm, self.qkv)
+            row_norm = N.RowNorm(stats.stats.data_ptr(), colsum.data_ptr(), stats.tiles, float(norm.eps))
+            return x.reshape(rows, x.shape[-1]).contiguous(), w, bias, row_norm, (stats, colsum)
         w = self.qkv.weight
         rows = x.numel() // x.shape[-1]
         if not (x.is_cuda and x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and cache_dtype == torch.bfloat16
@@ -376,6 +431,13 @@ class HipPagedAttention(nn.Module):
                 hit = self.__dict__["_qkv_bias_f32"] = (key, b.detach().float().contiguous())
             bias = hit[1]
         return x.reshape(rows, x.shape[-1]).contiguous(), (w if w.is_contiguous() else w.contiguous()), bias
+
+    def can_fold_norm(self, x: Tensor, norm, cache_dtype) -> bool:
+        """Whether ``norm`` (the block's ``norm1``) can be folded into the fused projection."""
+        rows = x.numel() // x.shape[-1]
+        return (FoldedNorm.possible(norm, self.qkv) and x.is_cuda and x.dtype == torch.bfloat16
+                and cache_dtype == torch.bfloat16 and self.head_dim == 64 and rows <= self.FUSED_PROJ_MAX_ROWS
+                and not torch.is_grad_enabled())
 
     def can_fuse_dense(self, x: Tensor, pos, enable_3d_rope: bool) -> bool:
         """Whether the cache-less attention of a batch of frames can run as fused producer +
@@ -396,18 +458,19 @@ class HipPagedAttention(nn.Module):
             return torch.is_tensor(pos) and pos.is_complex()
         return isinstance(self.rope, RotaryPositionEmbedding2D) and torch.is_tensor(pos) and pos.shape[0] in (1, x.shape[0])
 
-    def dense_attend_fused(self, x: Tensor, pos=None, enable_3d_rope: bool = False) -> Tensor:
+    def dense_attend_fused(self, x: Tensor, pos=None, enable_3d_rope: bool = False, norm=None, stats=None) -> Tensor:
         """Attention of every frame of the batch over its own tokens (attention.py:446-465):
-        qkv projection, one producer kernel, the paged kernel over a trivial row table."""
+        qkv projection, one producer kernel, the paged kernel over a trivial row table.
+        ``norm``, ``stats``: ``x`` is the block's input and ``norm`` is folded into the projection."""
         import ctypes as C
         from . import _native as N
         from .dense import dense_attention
         B, n, _ = x.shape
         H, D = self.num_heads, self.head_dim
-        proj = self._fused_projection(x, x.dtype)
+        proj = self._fused_projection(x, x.dtype, norm, stats)
         qkv = None if proj is not None else self.qkv(x).reshape(B * n, -1).contiguous()
         has_norm = isinstance(self.q_norm, nn.LayerNorm)
-        norm = (self._norm_f32(self.q_norm) + self._norm_f32(self.k_norm)) if has_norm else (None,) * 4
+        qk_norm = (self._norm_f32(self.q_norm) + self._norm_f32(self.k_norm)) if has_norm else (None,) * 4
         table, layout = None, N.ROPE_INTERLEAVED
         if self.rope is not None and enable_3d_rope:
             table = torch.view_as_real(pos.to(torch.complex64)).reshape(-1, D // 2, 2)
@@ -425,18 +488,21 @@ class HipPagedAttention(nn.Module):
         eps = float(self.q_norm.eps) if has_norm else 1e-5
         stream = N.stream_ptr(x.device)
         if proj is not None:
-            N.check(N.lib.lbm_qkv_linear_prepare(
-                p(proj[0]), p(proj[1]), p(proj[2]), B * n, proj[0].shape[1], p(norm[0]), p(norm[1]), p(norm[2]), p(norm[3]),
+            N.check(N.lib.lbm_qkv_linear_prepare_norm(
+                p(proj[0]), proj[3] if len(proj) > 3 else None, p(proj[1]), p(proj[2]), B * n, proj[0].shape[1],
+                p(qk_norm[0]), p(qk_norm[1]), p(qk_norm[2]), p(qk_norm[3]),
                 eps, p(table), layout, p(q), p(k), p(v), None, None, H, D, 16, stream))
         else:
             N.check(N.lib.lbm_qkv_prepare(
-                p(qkv), dt, p(norm[0]), p(norm[1]), p(norm[2]), p(norm[3]), eps, p(table), layout, p(q), p(k), p(v), dt,
+                p(qkv), dt, p(qk_norm[0]), p(qk_norm[1]), p(qk_norm[2]), p(qk_norm[3]), eps, p(table), layout, p(q), p(k), p(v), dt,
                 None, None, B * n, H, D, 16, stream))
         return dense_attention(q, k, v, num_streams=B).reshape(B, n, H * D)
 
     def forward(self, x: Tensor, pos=None, num_patches=None, num_special=None, num_frames=None,
                 enable_3d_rope=False, kv_cache=None, global_idx=0, num_frame_per_block=1,
-                num_frame_for_scale=-1, num_register_tokens=4) -> Tensor:
+                num_frame_for_scale=-1, num_register_tokens=4, project: bool = True) -> Tensor:
+        """The reference's arguments (attention.py:428-441); ``project=False`` returns the heads'
+        output before ``proj`` (for a caller that fuses the projection with what follows)."""
         B, N, _ = x.shape
         has_manager = kv_cache is not None and hasattr(kv_cache, "append_frame")
         if not has_manager:
@@ -465,7 +531,7 @@ class HipPagedAttention(nn.Module):
                 q, k, v = self.prepare_qkv(x, pos=pos, enable_3d_rope=enable_3d_rope)
                 out = self.stream_attend(kv_cache, global_idx, q, k, v, num_register_tokens)
             out = out.reshape(B, N, self.num_heads * self.head_dim).to(x.dtype)
-        return self.proj(out)
+        return self.proj(out) if project else out
 
 
 class HipPagedBlock(nn.Module):
@@ -542,6 +608,58 @@ class HipPagedBlock(nn.Module):
         x = self.ffn_residual(x + self.ls1(attn_out))
         return x if next_norm is None else (x, next_norm(x))
 
+    # ------------------------------------------------------------------ the block as a chain of fused launches
+    def _can_chain(self, x: Tensor, kv_cache, pos, enable_3d_rope: bool, streaming: bool) -> bool:
+        """Whether the block can run as: qkv projection (+ folded norm1) + producer, attention,
+        proj + LayerScale + residual (+ row statistics), fc1 (+ folded norm2) + GELU, fc2 +
+        LayerScale + residual (+ row statistics) - five GEMM launches and the attention, no
+        LayerNorm or residual kernel.  One frame's rows of bf16 on the GPU, inference."""
+        a, rows = self.attn, x.numel() // x.shape[-1]
+        if not (x.is_cuda and x.dtype == torch.bfloat16 and rows <= Mlp.FUSED_MAX_ROWS and not torch.is_grad_enabled()):
+            return False
+        if not (type(self.mlp) is Mlp and self.mlp._can_fuse_fc1(x) and FoldedNorm.possible(self.norm2, self.mlp.fc1)):
+            return False
+        if not all(isinstance(ls, (LayerScale, nn.Identity)) for ls in (self.ls1, self.ls2)):
+            return False
+        for lin in (a.proj, self.mlp.fc2):
+            if not (lin.weight.dtype == torch.bfloat16 and lin.weight.is_cuda and lin.in_features % 128 == 0
+                    and lin.out_features % 64 == 0):
+                return False
+        if streaming:
+            return a.can_fuse(kv_cache, pos, enable_3d_rope) and kv_cache.dtype == torch.bfloat16
+        return a.can_fuse_dense(x, pos, enable_3d_rope)
+
+    def _linear_residual(self, a: Tensor, linear: nn.Linear, ls, residual: Tensor, want_stats: bool):
+        """``residual + ls(linear(a))`` as one launch (attention.py:554 / mlp.py:38 with
+        layer_scale.py:21-22 and block.py:283-285), and the row statistics of the result for the
+        LayerNorm that reads it next."""
+        import ctypes as C
+        from . import _native as N
+        rows, n_out = a.numel() // a.shape[-1], linear.out_features
+        a2, res = a.reshape(rows, -1).contiguous(), residual.reshape(rows, n_out).contiguous()
+        out = torch.empty_like(res)
+        stats = None
+        if want_stats:
+            tiles = int(N.lib.lbm_linear_stats_tiles(rows, n_out))
+            stats = RowStats(torch.empty(rows, tiles, 2, dtype=torch.float32, device=a.device), tiles)
+        w = linear.weight if linear.weight.is_contiguous() else linear.weight.contiguous()
+        bias = self._f32(linear.bias) if linear.bias is not None else None
+        gamma = self._f32(ls.gamma) if isinstance(ls, LayerScale) else None
+        p = lambda t: None if t is None else C.c_void_p(t.data_ptr())
+        N.check(N.lib.lbm_linear_norm(p(a2), None, p(w), p(bias), p(gamma), p(res), p(out),
+                                      p(stats.stats) if stats is not None else None, rows, n_out, a2.shape[1],
+                                      N.LINEAR_BIAS_RESIDUAL, N.stream_ptr(a.device)))
+        return out.reshape(residual.shape), stats
+
+    def _finish_chain(self, x: Tensor, heads_out: Tensor, next_norm):
+        """Everything after the attention kernel (block.py:283-285) in three launches;
+        ``heads_out`` is the attention's output before ``proj``.  With ``next_norm`` the result is
+        ``(x, RowStats)``: the statistics the next block folds its ``norm1`` from."""
+        x, stats = self._linear_residual(heads_out, self.attn.proj, self.ls1, x, True)
+        hidden = self.mlp.fc1_gelu(x, self.norm2, stats)
+        x, stats = self._linear_residual(hidden, self.mlp.fc2, self.ls2, x, next_norm is not None)
+        return x if next_norm is None else (x, stats)
+
     def attn_pre(self, x: Tensor, pos=None, enable_3d_rope: bool = False):
         """norm1 + projections + qk-norm + RoPE, ready for the cache (block.py:217-227)."""
         return self.attn.prepare_qkv(self.norm1(x), pos=pos, enable_3d_rope=enable_3d_rope)
@@ -554,10 +672,26 @@ class HipPagedBlock(nn.Module):
                 num_frame_for_scale=-1, num_register_tokens=4, normed: Optional[Tensor] = None,
                 next_norm: Optional[nn.LayerNorm] = None):
         """The reference's arguments (block.py:229-243) plus two for a caller that chains blocks:
-        ``normed`` = ``self.norm1(x)`` if the caller already has it, ``next_norm`` = the ``norm1``
-        of the block that follows; with ``next_norm`` the result is ``(x, next_norm(x))``."""
-        n1 = self.norm1(x) if normed is None else normed
+        ``normed`` = ``self.norm1(x)`` if the caller already has it - or the ``RowStats`` of ``x``
+        the block before left behind - and ``next_norm`` = the ``norm1`` of the block that follows;
+        with ``next_norm`` the result is ``(x, next_norm(x))`` or ``(x, RowStats of x)``."""
         is_streaming = kv_cache is not None and (num_frames is None or num_frames <= 1)
+        is_dense = kv_cache is None or not hasattr(kv_cache, "append_frame")
+        stats = normed if isinstance(normed, RowStats) else None
+        if (is_streaming or is_dense) and self._can_chain(x, kv_cache, pos, enable_3d_rope, is_streaming):
+            cache_dtype = kv_cache.dtype if is_streaming else x.dtype
+            fold = stats is not None and self.attn.can_fold_norm(x, self.norm1, cache_dtype)
+            if fold:
+                a_in, kw = x, dict(norm=self.norm1, stats=stats)
+            else:
+                a_in, kw = (self.norm1(x) if (normed is None or stats is not None) else normed), {}
+            if is_streaming:
+                heads = self.attn.stream_attend_fused(kv_cache, global_idx, a_in, pos, **kw)
+            else:
+                heads = self.attn.dense_attend_fused(a_in, pos, enable_3d_rope, **kw)
+            heads = heads.reshape(x.shape[0], x.shape[1], self.attn.num_heads * self.attn.head_dim).to(x.dtype)
+            return self._finish_chain(x, heads, next_norm)
+        n1 = self.norm1(x) if (normed is None or stats is not None) else normed
         if is_streaming:
             if self.attn.can_fuse(kv_cache, pos, enable_3d_rope):
                 attn_x = self.attn.stream_attend_fused(kv_cache, global_idx, n1, pos)

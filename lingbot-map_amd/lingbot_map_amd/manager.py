@@ -481,7 +481,8 @@ class HipPagedKVCacheManager:
                 qkv = qkv.to(self.dtype)
             qkv = qkv.contiguous()
         else:
-            px, pw, pb = proj
+            px, pw, pb = proj[:3]
+            row_norm = proj[3] if len(proj) > 3 else None   # lbm_row_norm: norm1 folded into the projection
             assert qkv is None and self.dtype == torch.bfloat16 and D == 64, "proj: bf16 cache with head_dim 64"
             assert px.dtype == pw.dtype == torch.bfloat16 and px.is_contiguous() and pw.is_contiguous()
             assert px.shape[0] == rows and pw.shape == (3 * H * D, px.shape[1]) and px.shape[1] % 128 == 0, (
@@ -509,8 +510,8 @@ class HipPagedKVCacheManager:
                 rope_ptr, N.ROPE_INTERLEAVED, vp(q), vp(k), vp(v), dt(self.dtype),
                 vp(self.kv_caches[block_idx]), append_ptr, rows, H, D, self.page_size, self._stream_handle()))
         else:
-            N.check(N.lib.lbm_qkv_linear_prepare(
-                vp(px), vp(pw), vp(pb), rows, px.shape[1], norm_ptr[0], norm_ptr[1], norm_ptr[2], norm_ptr[3],
+            N.check(N.lib.lbm_qkv_linear_prepare_norm(
+                vp(px), row_norm, vp(pw), vp(pb), rows, px.shape[1], norm_ptr[0], norm_ptr[1], norm_ptr[2], norm_ptr[3],
                 float(norm_eps), rope_ptr, N.ROPE_INTERLEAVED, vp(q), vp(k), vp(v),
                 vp(self.kv_caches[block_idx]), append_ptr, H, D, self.page_size, self._stream_handle()))
         if any(keyframe):
