@@ -237,10 +237,22 @@ typedef struct lbm_row_norm {
 int32_t lbm_linear_stats_tiles(int32_t M, int32_t N);
 
 /* lbm_linear with a_norm (NULL = none; not with the residual epilogue) applied to the
- * activations and / or out_stats (NULL = none; residual epilogue only) written. */
+ * activations and / or out_stats (NULL = none; residual epilogue only) written.
+ * workspace (NULL = none): device memory of at least lbm_linear_workspace_bytes(M, N, K, epilogue)
+ * bytes that lets a launch with few tiles and a long K (fc2 of one frame: 128 tiles, K = 4096)
+ * put several workgroups on each tile, each over a slice of K; the one that finishes a tile last
+ * sums the slices in a fixed order, so results do not depend on timing.  The first 256-byte
+ * aligned part of the workspace holds one counter per tile: the caller zero-fills the workspace
+ * once, every launch leaves the counters at zero.  Launches that overlap in time on one GPU need
+ * workspaces of their own, and with a workspace the residual may not alias out. */
 int lbm_linear_norm(const void* a, const lbm_row_norm* a_norm, const void* w, const float* bias,
                     const float* gamma, const void* residual, void* out, float* out_stats,
-                    int32_t M, int32_t N, int32_t K, int32_t epilogue, void* stream);
+                    int32_t M, int32_t N, int32_t K, int32_t epilogue, void* workspace,
+                    size_t workspace_bytes, void* stream);
+
+/* Bytes of workspace with which lbm_linear_norm would split K for this shape and epilogue; 0 when
+ * it would not. */
+size_t lbm_linear_workspace_bytes(int32_t M, int32_t N, int32_t K, int32_t epilogue);
 
 /* lbm_qkv_linear_prepare with a_norm (NULL = none) applied to the activations: norm1 of the
  * block (folded as described at lbm_row_norm), its qkv projection and the pre-attention producer

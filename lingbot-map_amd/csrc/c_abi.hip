@@ -124,19 +124,25 @@ int lbm_qkv_prepare(const void* qkv, int32_t src_dtype, const float* q_norm_w, c
 
 int lbm_linear_norm(const void* a, const lbm_row_norm* a_norm, const void* w, const float* bias, const float* gamma,
                     const void* residual, void* out, float* out_stats, int32_t M, int32_t N, int32_t K,
-                    int32_t epilogue, void* stream) {
+                    int32_t epilogue, void* workspace, size_t workspace_bytes, void* stream) {
   if (!a || !w || !out) return lbm_fail(LBM_ERR_INVALID, "lbm_linear: null a, w or out");
   if (M < 0 || N <= 0 || K <= 0) return lbm_fail(LBM_ERR_INVALID, "lbm_linear: bad shape %d x %d x %d", M, N, K);
   if (epilogue == LBM_LINEAR_BIAS_RESIDUAL && !residual)
     return lbm_fail(LBM_ERR_INVALID, "lbm_linear: the residual epilogue needs a residual");
   if (epilogue != LBM_LINEAR_BIAS_RESIDUAL && (residual || gamma))
     return lbm_fail(LBM_ERR_INVALID, "lbm_linear: residual / gamma given without the residual epilogue");
-  return lbm_launch_linear(a, a_norm, w, bias, gamma, residual, out, out_stats, M, N, K, epilogue, (hipStream_t)stream);
+  return lbm_launch_linear(a, a_norm, w, bias, gamma, residual, out, out_stats, M, N, K, epilogue, workspace,
+                           workspace_bytes, (hipStream_t)stream);
+}
+
+size_t lbm_linear_workspace_bytes(int32_t M, int32_t N, int32_t K, int32_t epilogue) {
+  if (M <= 0 || N <= 0 || K <= 0 || N % 64 != 0 || K % 128 != 0) return 0;
+  return lbm_linear_workspace_for(M, N, K, epilogue);
 }
 
 int lbm_linear(const void* a, const void* w, const float* bias, const float* gamma, const void* residual,
                void* out, int32_t M, int32_t N, int32_t K, int32_t epilogue, void* stream) {
-  return lbm_linear_norm(a, nullptr, w, bias, gamma, residual, out, nullptr, M, N, K, epilogue, stream);
+  return lbm_linear_norm(a, nullptr, w, bias, gamma, residual, out, nullptr, M, N, K, epilogue, nullptr, 0, stream);
 }
 
 int32_t lbm_linear_stats_tiles(int32_t M, int32_t N) {

@@ -35,8 +35,9 @@ int lbm_launch_residual_norm(const void* x, const void* y, int dtype, const floa
 
 int lbm_launch_linear(const void* a, const lbm_row_norm* a_norm, const void* w, const float* bias, const float* gamma,
                       const void* residual, void* out, float* out_stats, int M, int N, int K, int epilogue,
-                      hipStream_t stream);
+                      void* workspace, size_t workspace_bytes, hipStream_t stream);
 int lbm_linear_stats_tiles_for(int M, int N);
+size_t lbm_linear_workspace_for(int M, int N, int K, int epilogue);
 
 int lbm_launch_qkv_linear_prepare(const void* a, const lbm_row_norm* a_norm, const void* w, const float* bias, int M, int K,
                                   const float* q_norm_w, const float* q_norm_b, const float* k_norm_w,

@@ -78,6 +78,13 @@ struct LinearArgs {
   // LBM_LINEAR_BIAS_RESIDUAL: (mean, M2) of every output row over this tile's columns,
   // [M][n_tiles][2], or null
   float* stats_out;
+  // SPLITK kernels: k_splits workgroups share a tile, each over its own slice of K.  Every one
+  // parks its fp32 partial tile in `split_part` and takes a ticket from the tile's counter; the
+  // one that draws the last ticket sums the partials in slice order (the same sum whoever is
+  // last) and runs the epilogue.  Counters start at zero and are left at zero.
+  int k_splits;
+  unsigned* split_counters;      // [m_tiles * n_tiles]
+  float* split_part;             // [m_tiles * n_tiles][k_splits][8 waves][NT * 16][64 lanes]
 };
 constexpr int kEpiQkvPrepare = 3;   // internal: reached through lbm_qkv_linear_prepare only
 
@@ -129,7 +136,8 @@ constexpr int kGeluEntries = 2 * kGeluHalf;
 // ROPE / NORM: rotary layout (0 none, 1 interleaved, 2 half-split) and qk-LayerNorm of the
 // kEpiQkvPrepare epilogue; 0 / false otherwise.
 // LNA: the activations' rows are standardised by the store (see LinearArgs).
-template <int EPI, int TN, int ROPE = 0, bool NORM = false, bool LNA = false>
+// SPLITK: several workgroups per tile, each over a slice of K (see LinearArgs).
+template <int EPI, int TN, int ROPE = 0, bool NORM = false, bool LNA = false, bool SPLITK = false>
 __global__ __launch_bounds__(kGThreads, 1) void lbm_linear_bf16_kernel(LinearArgs p) {
   constexpr int NT = TN / 64;   // 32-column blocks of W per wavefront
   // [buffer][k half][row][64 + pad]
@@ -143,15 +151,27 @@ __global__ __launch_bounds__(kGThreads, 1) void lbm_linear_bf16_kernel(LinearArg
   const int kh = wave >> 2, ws = wave & 3;    // k half of this wave's group, its sub-tile
   // Workgroups are dealt to the 8 XCDs round-robin: an XCD keeps its own column tiles of W (read
   // from HBM once, by it alone) and walks all row tiles of the activations with them.
-  int mt, nt;
+  // (the workgroups that share a tile under SPLITK land on the same XCD as well)
+  int mt, nt, split = 0;
   {
-    const int x = blockIdx.x & 7, i = blockIdx.x >> 3;
+    const int n_tiles_all = p.m_tiles * p.n_tiles;
     if ((p.n_tiles & 7) == 0) {
+      const int x = blockIdx.x & 7;
+      int i = blockIdx.x >> 3;
+      if (SPLITK) {
+        split = i / (n_tiles_all >> 3);
+        i -= split * (n_tiles_all >> 3);
+      }
       mt = i % p.m_tiles;
       nt = (i / p.m_tiles) * 8 + x;
     } else {
-      mt = (int)blockIdx.x % p.m_tiles;
-      nt = (int)blockIdx.x / p.m_tiles;
+      int i = (int)blockIdx.x;
+      if (SPLITK) {
+        split = i / n_tiles_all;
+        i -= split * n_tiles_all;
+      }
+      mt = i % p.m_tiles;
+      nt = i / p.m_tiles;
     }
   }
   const int m0 = mt * kGM, n0 = nt * TN;
@@ -166,8 +186,10 @@ __global__ __launch_bounds__(kGThreads, 1) void lbm_linear_bf16_kernel(LinearArg
 #pragma unroll
   for (int j = 0; j < kPassA; ++j) a_off[j] = ((unsigned)min(m0 + ld_r + 32 * j, p.M - 1) * (unsigned)p.K + ld_c) * 2u;   // rows past M re-read the last row
   const unsigned w_off = ((unsigned)ld_r * (unsigned)p.K + ld_c) * 2u;
-  const char* a_base = (const char*)p.a;
-  const char* w_base = (const char*)(p.w + (size_t)n0 * p.K);
+  const int nk = SPLITK ? p.K / kGK / p.k_splits : p.K / kGK;   // k-steps of this workgroup
+  const size_t k_first = SPLITK ? (size_t)split * nk * kGK : 0;
+  const char* a_base = (const char*)(p.a + k_first);
+  const char* w_base = (const char*)(p.w + (size_t)n0 * p.K + k_first);
   auto load_a = [&](int j, int ks) -> u32x4 { return *(const u32x4*)(a_base + ks * (kGK * 2) + a_off[j]); };
   auto load_w = [&](int j, int ks) -> u32x4 {
     return *(const u32x4*)(w_base + ((size_t)(32 * j) * p.K + (size_t)ks * kGK) * 2 + w_off);
@@ -240,7 +262,6 @@ __global__ __launch_bounds__(kGThreads, 1) void lbm_linear_bf16_kernel(LinearArg
     }
   };
 
-  const int nk = p.K / kGK;
   const int last = nk - 1;                       // steps past the end re-read the last one (never multiplied)
   // LNA, row statistics: row r of the tile is handled by threads 4 r .. 4 r + 3, each taking every
   // fourth (mean, M2) partial; equal-sized partials merge as mean = avg(mean_i),
@@ -331,6 +352,48 @@ __global__ __launch_bounds__(kGThreads, 1) void lbm_linear_bf16_kernel(LinearArg
       for (int i = 0; i < 16; ++i) fin[a][i] += xch[((peer * NT + a) * 16 + i) * 64 + lane];
   }
   const int b = kh;     // the row block this wave finishes
+  if (SPLITK) {
+    // Partials and counters travel as scope-qualified relaxed atomics, which go past the caches
+    // that are not coherent between workgroups (the CU's and, between XCDs, the L2) - a
+    // device-wide fence would write back and invalidate the whole L2 instead, once per
+    // workgroup (measured: 60 us on a 25 us launch).  Order: a thread's stores are complete
+    // (the workgroup-scope fence waits for their acknowledgements), the barrier collects all
+    // threads, thread 0 draws the ticket.
+    __shared__ unsigned ticket_lds;
+    const int tile = mt * p.n_tiles + nt;
+    constexpr int kPartFloats = 8 * NT * 16 * 64;                 // one workgroup's partial tile
+    float* tile_part = p.split_part + (size_t)tile * p.k_splits * kPartFloats;
+    float* mine = tile_part + (size_t)split * kPartFloats + (size_t)wave * (NT * 16 * 64);
+#pragma unroll
+    for (int a = 0; a < NT; ++a)
+#pragma unroll
+      for (int i = 0; i < 16; ++i)
+        __hip_atomic_store(&mine[(a * 16 + i) * 64 + lane], fin[a][i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    __syncthreads();
+    if (tid == 0) ticket_lds = __hip_atomic_fetch_add(&p.split_counters[tile], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __syncthreads();
+    if (ticket_lds != (unsigned)(p.k_splits - 1)) return;          // (uniform over the workgroup)
+    if (tid == 0) __hip_atomic_store(&p.split_counters[tile], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // as the next launch expects it
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+    // two slices: this workgroup's own sum is still in its registers and a + b = b + a; more
+    // slices: all of them from memory, in slice order, so the sum does not depend on who is last
+    const bool pair = p.k_splits == 2;
+    if (!pair) {
+#pragma unroll
+      for (int a = 0; a < NT; ++a)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) fin[a][i] = 0.f;
+    }
+    for (int sidx = pair ? 1 - split : 0; sidx < (pair ? 2 - split : p.k_splits); ++sidx) {
+      const float* src = tile_part + (size_t)sidx * kPartFloats + (size_t)wave * (NT * 16 * 64);
+#pragma unroll
+      for (int a = 0; a < NT; ++a)
+#pragma unroll
+        for (int i = 0; i < 16; ++i)
+          fin[a][i] += __hip_atomic_load(&src[(a * 16 + i) * 64 + lane], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+    }
+  }
 
   // ---- epilogue.  In registers: + bias, round (the linear's output), GELU or LayerScale, round.
   // Then the tile goes through LDS and leaves as whole rows.
@@ -510,6 +573,28 @@ int lbm_set_row_norm(LinearArgs& p, const lbm_row_norm* ln, const char* who) {
 }
 }  // namespace
 
+namespace {
+// K slices per tile: as many as still leave every workgroup eight k-steps and fit one round of
+// the 256 CUs (fc2 of one frame: 128 tiles x 2); the residual epilogue only
+int lbm_linear_splits(const LinearArgs& p, int epilogue) {
+  if (epilogue != LBM_LINEAR_BIAS_RESIDUAL) return 1;
+  const int tiles = p.m_tiles * p.n_tiles, nk = p.K / kGK;
+  for (int s = 4; s >= 2; s >>= 1)
+    if (tiles * s <= 256 && nk % s == 0 && nk / s >= 8) return s;
+  return 1;
+}
+size_t lbm_linear_counter_bytes(const LinearArgs& p) { return ((size_t)p.m_tiles * p.n_tiles * 4 + 255) & ~(size_t)255; }
+}  // namespace
+
+size_t lbm_linear_workspace_for(int M, int N, int K, int epilogue) {
+  LinearArgs p = {};
+  p.M = M; p.N = N; p.K = K;
+  const int tn = lbm_linear_tiles(p);
+  const int s = lbm_linear_splits(p, epilogue);
+  if (s == 1) return 0;
+  return lbm_linear_counter_bytes(p) + (size_t)p.m_tiles * p.n_tiles * s * kGM * tn * 4;
+}
+
 int lbm_linear_stats_tiles_for(int M, int N) {
   LinearArgs p = {};
   p.M = M; p.N = N;
@@ -519,7 +604,7 @@ int lbm_linear_stats_tiles_for(int M, int N) {
 
 int lbm_launch_linear(const void* a, const lbm_row_norm* a_norm, const void* w, const float* bias, const float* gamma,
                       const void* residual, void* out, float* out_stats, int M, int N, int K, int epilogue,
-                      hipStream_t stream) {
+                      void* workspace, size_t workspace_bytes, hipStream_t stream) {
   if (M == 0) return LBM_OK;
   if (K % kGK != 0 || N % 64 != 0)
     return lbm_fail(LBM_ERR_UNSUPPORTED, "lbm_linear: K must be a multiple of 128 and N of 64 (got K %d, N %d)", K, N);
@@ -539,7 +624,22 @@ int lbm_launch_linear(const void* a, const lbm_row_norm* a_norm, const void* w, 
   if (int rc = lbm_set_row_norm(p, a_norm, "lbm_linear_norm")) return rc;
   const bool wide = lbm_linear_tiles(p) == 128;
   const bool lna = a_norm != nullptr;
-  const dim3 grid((unsigned)(p.m_tiles * p.n_tiles)), block(kGThreads);
+  const dim3 block(kGThreads);
+  if (workspace) {
+    const int splits = lbm_linear_splits(p, epilogue);
+    if (splits > 1 && workspace_bytes >= lbm_linear_workspace_for(M, N, K, epilogue)) {
+      if (residual == out)   // a workgroup that is not the tile's last would see the other's store
+        return lbm_fail(LBM_ERR_INVALID, "lbm_linear_norm: with a workspace the residual may not alias out");
+      p.k_splits = splits;
+      p.split_counters = (unsigned*)workspace;
+      p.split_part = (float*)((char*)workspace + lbm_linear_counter_bytes(p));
+      const dim3 grid_s((unsigned)(p.m_tiles * p.n_tiles * splits));
+      if (wide) hipLaunchKernelGGL((lbm_linear_bf16_kernel<LBM_LINEAR_BIAS_RESIDUAL, 128, 0, false, false, true>), grid_s, block, 0, stream, p);
+      else hipLaunchKernelGGL((lbm_linear_bf16_kernel<LBM_LINEAR_BIAS_RESIDUAL, 64, 0, false, false, true>), grid_s, block, 0, stream, p);
+      return lbm_check_launch("lbm_linear_bf16_kernel<split K>");
+    }
+  }
+  const dim3 grid((unsigned)(p.m_tiles * p.n_tiles));
 #define LBM_LINEAR_LAUNCH(E, L)                                                                                  \
   {                                                                                                              \
     if (wide) hipLaunchKernelGGL((lbm_linear_bf16_kernel<E, 128, 0, false, L>), grid, block, 0, stream, p);      \

@@ -47,7 +47,7 @@ class RowNorm(C.Structure):
 
 
 SYMBOLS = ("lbm_abi_version", "lbm_last_error", "lbm_tables_words", "lbm_tables_step",
-           "lbm_rows_from_pages", "lbm_kv_append", "lbm_qkv_prepare", "lbm_residual_norm", "lbm_linear", "lbm_linear_norm", "lbm_linear_stats_tiles", "lbm_qkv_linear_prepare", "lbm_qkv_linear_prepare_norm", "lbm_attn_workspace_bytes", "lbm_attn_run", "lbm_attn_run_live",
+           "lbm_rows_from_pages", "lbm_kv_append", "lbm_qkv_prepare", "lbm_residual_norm", "lbm_linear", "lbm_linear_norm", "lbm_linear_stats_tiles", "lbm_linear_workspace_bytes", "lbm_qkv_linear_prepare", "lbm_qkv_linear_prepare_norm", "lbm_attn_workspace_bytes", "lbm_attn_run", "lbm_attn_run_live",
            "lbm_attn_run_static")
 
 
@@ -75,7 +75,9 @@ def _load():
     lib.lbm_linear.restype = C.c_int
     lib.lbm_linear.argtypes = [vp, vp, vp, vp, vp, vp, i32, i32, i32, i32, vp]
     lib.lbm_linear_norm.restype = C.c_int
-    lib.lbm_linear_norm.argtypes = [vp, p(RowNorm), vp, vp, vp, vp, vp, vp, i32, i32, i32, i32, vp]
+    lib.lbm_linear_norm.argtypes = [vp, p(RowNorm), vp, vp, vp, vp, vp, vp, i32, i32, i32, i32, vp, C.c_size_t, vp]
+    lib.lbm_linear_workspace_bytes.restype = C.c_size_t
+    lib.lbm_linear_workspace_bytes.argtypes = [i32, i32, i32, i32]
     lib.lbm_linear_stats_tiles.restype = i32
     lib.lbm_linear_stats_tiles.argtypes = [i32, i32]
     lib.lbm_qkv_linear_prepare_norm.restype = C.c_int

@@ -189,6 +189,21 @@ class LayerScale(nn.Module):
         return x * self.gamma
 
 
+_split_workspaces = {}
+
+
+def _split_workspace(device, nbytes: int) -> Optional[Tensor]:
+    """Zero-filled device memory for launches that split K (``lbm_linear_norm``'s workspace; the
+    launches leave its counters at zero), one per device and stream; None when nothing is needed."""
+    if nbytes <= 0:
+        return None
+    key = (device, torch.cuda.current_stream(device).cuda_stream)
+    ws = _split_workspaces.get(key)
+    if ws is None or ws.numel() < nbytes:
+        ws = _split_workspaces[key] = torch.zeros(nbytes, dtype=torch.uint8, device=device)
+    return ws
+
+
 class RowStats:
     """What a block hands the next one in place of ``norm1(x)``: per row of ``x`` and column tile of
     the launch that wrote it, the mean and the sum of squared deviations (``lbm_linear_norm``'s
@@ -278,7 +293,7 @@ class Mlp(nn.Module):
             w, colsum, bias = FoldedNorm.of(self, norm, fc1)
             row_norm = N.RowNorm(stats.stats.data_ptr(), colsum.data_ptr(), stats.tiles, float(norm.eps))
         N.check(N.lib.lbm_linear_norm(p(a), row_norm, p(w), p(bias), None, None, p(out), None, a.shape[0], fc1.out_features,
-                                      fc1.in_features, N.LINEAR_BIAS_GELU, N.stream_ptr(x.device)))
+                                      fc1.in_features, N.LINEAR_BIAS_GELU, None, 0, N.stream_ptr(x.device)))
         return out.reshape(*x.shape[:-1], fc1.out_features)
 
     def forward(self, x: Tensor) -> Tensor:
@@ -646,9 +661,11 @@ class HipPagedBlock(nn.Module):
         bias = self._f32(linear.bias) if linear.bias is not None else None
         gamma = self._f32(ls.gamma) if isinstance(ls, LayerScale) else None
         p = lambda t: None if t is None else C.c_void_p(t.data_ptr())
+        ws = _split_workspace(a.device, int(N.lib.lbm_linear_workspace_bytes(rows, n_out, a2.shape[1], N.LINEAR_BIAS_RESIDUAL)))
         N.check(N.lib.lbm_linear_norm(p(a2), None, p(w), p(bias), p(gamma), p(res), p(out),
                                       p(stats.stats) if stats is not None else None, rows, n_out, a2.shape[1],
-                                      N.LINEAR_BIAS_RESIDUAL, N.stream_ptr(a.device)))
+                                      N.LINEAR_BIAS_RESIDUAL, p(ws), ws.numel() if ws is not None else 0,
+                                      N.stream_ptr(a.device)))
         return out.reshape(residual.shape), stats
 
     def _finish_chain(self, x: Tensor, heads_out: Tensor, next_norm):

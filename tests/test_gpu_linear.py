@@ -253,7 +253,7 @@ def test_residual_epilogue_leaves_row_statistics(M, K, Nn):
     stats = torch.full((M, tiles, 2), float("nan"), dtype=torch.float32, device=dev)
     ad, wd, bd, gd, rd = a.to(dev), w.to(dev), bias.float().to(dev), gamma.float().to(dev), res.to(dev)
     N.check(N.lib.lbm_linear_norm(ptr(ad), None, ptr(wd), ptr(bd), ptr(gd), ptr(rd), ptr(out), ptr(stats), M, Nn, K,
-                                  N.LINEAR_BIAS_RESIDUAL, None))
+                                  N.LINEAR_BIAS_RESIDUAL, None, 0, None))
     torch.cuda.synchronize()
     assert torch.equal(out.cpu(), plain)
     x = out.cpu().double().reshape(M, tiles, Nn // tiles)
@@ -263,9 +263,9 @@ def test_residual_epilogue_leaves_row_statistics(M, K, Nn):
     assert (got[..., 0] - mean).abs().max().item() <= 1e-5 * max(1.0, mean.abs().max().item())
     assert ((got[..., 1] - m2).abs() <= 1e-4 * m2.clamp_min(1e-3)).all()
     # statistics only come with the residual epilogue, a folded LayerNorm never with it
-    assert N.lib.lbm_linear_norm(ptr(ad), None, ptr(wd), ptr(bd), None, None, ptr(out), ptr(stats), M, Nn, K, N.LINEAR_BIAS, None) != N.OK
+    assert N.lib.lbm_linear_norm(ptr(ad), None, ptr(wd), ptr(bd), None, None, ptr(out), ptr(stats), M, Nn, K, N.LINEAR_BIAS, None, 0, None) != N.OK
     ln = _row_norm(N, stats, gd, tiles)
-    assert N.lib.lbm_linear_norm(ptr(ad), ln, ptr(wd), ptr(bd), ptr(gd), ptr(rd), ptr(out), None, M, Nn, K, N.LINEAR_BIAS_RESIDUAL, None) != N.OK
+    assert N.lib.lbm_linear_norm(ptr(ad), ln, ptr(wd), ptr(bd), ptr(gd), ptr(rd), ptr(out), None, M, Nn, K, N.LINEAR_BIAS_RESIDUAL, None, 0, None) != N.OK
 
 
 def _stats_of(x, tiles):
@@ -303,7 +303,7 @@ def test_layernorm_folded_into_the_linear(M, K, Nn, tiles, epilogue):
     xd, wd, cd, bd = x.to(dev), wf.to(dev), colsum.to(dev), bf.to(dev)
     ln = _row_norm(N, stats, cd, tiles)
     out = torch.full((M, Nn), float("nan"), dtype=torch.bfloat16, device=dev)
-    N.check(N.lib.lbm_linear_norm(ptr(xd), ln, ptr(wd), ptr(bd), None, None, ptr(out), None, M, Nn, K, epilogue, None))
+    N.check(N.lib.lbm_linear_norm(ptr(xd), ln, ptr(wd), ptr(bd), None, None, ptr(out), None, M, Nn, K, epilogue, None, 0, None))
     torch.cuda.synchronize()
     got = out.cpu().float()
     assert torch.isfinite(got).all()
@@ -312,8 +312,8 @@ def test_layernorm_folded_into_the_linear(M, K, Nn, tiles, epilogue):
     assert err.mean().item() <= 2.0 ** -8 * pre.abs().mean().item(), (err.mean().item(), pre.abs().mean().item())
     assert (got.double() - exact).abs().mean().item() <= 1.05 * (ref.double() - exact).abs().mean().item()
     # a tile count that does not divide K, missing column sums
-    assert N.lib.lbm_linear_norm(ptr(xd), _row_norm(N, stats, cd, 7), ptr(wd), ptr(bd), None, None, ptr(out), None, M, Nn, K, epilogue, None) != N.OK
-    assert N.lib.lbm_linear_norm(ptr(xd), N.RowNorm(stats.data_ptr(), None, tiles, 1e-5), ptr(wd), ptr(bd), None, None, ptr(out), None, M, Nn, K, epilogue, None) != N.OK
+    assert N.lib.lbm_linear_norm(ptr(xd), _row_norm(N, stats, cd, 7), ptr(wd), ptr(bd), None, None, ptr(out), None, M, Nn, K, epilogue, None, 0, None) != N.OK
+    assert N.lib.lbm_linear_norm(ptr(xd), N.RowNorm(stats.data_ptr(), None, tiles, 1e-5), ptr(wd), ptr(bd), None, None, ptr(out), None, M, Nn, K, epilogue, None, 0, None) != N.OK
 
 
 def test_layernorm_folded_into_the_qkv_projection_and_producer():
@@ -354,3 +354,47 @@ def test_layernorm_folded_into_the_qkv_projection_and_producer():
         # an absolute part for the worst of three million elements (the noise of 1,024 products, 5 sigma)
         assert ((a0 - a1).abs() <= 2.0 ** -6 * a0.abs() + 2.0 ** -4).all(), (a0 - a1).abs().max().item()
         assert (a0 - a1).abs().mean().item() <= 2.0 ** -9 * a0.abs().mean().item() + 1e-3
+
+
+@pytest.mark.parametrize("M,K,Nn", [(1004, 4096, 1024), (200, 4096, 256), (130, 2048, 64)])
+def test_residual_epilogue_with_k_split_over_workgroups(M, K, Nn):
+    """With a workspace, launches with few tiles and a long K put several workgroups on a tile; the
+    one that finishes last sums the slices in a fixed order.  Against the CPU arithmetic (same bars
+    as the one-workgroup kernel), three launches in a row on one workspace (the counters go back to
+    zero by themselves) giving the same bits, statistics included."""
+    N = _native()
+    dev = torch.device("cuda:0")
+    a, w, bias, g = _inputs(M, K, Nn, seed=11 * M + Nn)
+    gamma = torch.randn(Nn, generator=g)
+    res = torch.randn(M, Nn, generator=g).to(torch.bfloat16)
+    ref = expected(a, w, bias, N.LINEAR_BIAS_RESIDUAL, gamma=gamma, residual=res)
+    need = N.lib.lbm_linear_workspace_bytes(M, Nn, K, N.LINEAR_BIAS_RESIDUAL)
+    assert need > 0 and N.lib.lbm_linear_workspace_bytes(M, Nn, K, N.LINEAR_BIAS) == 0
+    assert N.lib.lbm_linear_workspace_bytes(1004, 1024, 1024, N.LINEAR_BIAS_RESIDUAL) == 0      # proj: K too short to split
+    ws = torch.zeros(need, dtype=torch.uint8, device=dev)
+    tiles = N.lib.lbm_linear_stats_tiles(M, Nn)
+    ad, wd, bd, gd, rd = a.to(dev), w.to(dev), bias.float().to(dev), gamma.float().to(dev), res.to(dev)
+    outs = []
+    for _ in range(3):
+        out = torch.full((M, Nn), float("nan"), dtype=torch.bfloat16, device=dev)
+        stats = torch.full((M, tiles, 2), float("nan"), dtype=torch.float32, device=dev)
+        N.check(N.lib.lbm_linear_norm(ptr(ad), None, ptr(wd), ptr(bd), ptr(gd), ptr(rd), ptr(out), ptr(stats), M, Nn, K,
+                                      N.LINEAR_BIAS_RESIDUAL, ptr(ws), need, None))
+        torch.cuda.synchronize()
+        outs.append((out.cpu(), stats.cpu()))
+    n_tiles = ((M + 127) // 128) * tiles
+    assert ws[:4 * n_tiles].view(torch.int32).abs().sum().item() == 0            # counters back at zero
+    scale = torch.maximum(res.float().abs(), (ref.float() - res.float()).abs())
+    check(outs[0][0], ref, scale=scale, bar=2.0 ** -6)
+    for o, st in outs[1:]:
+        assert torch.equal(o, outs[0][0]) and torch.equal(st, outs[0][1])
+    x = outs[0][0].double().reshape(M, tiles, Nn // tiles)
+    assert (outs[0][1][..., 0].double() - x.mean(-1)).abs().max().item() <= 1e-5 * max(1.0, x.mean(-1).abs().max().item())
+    # a workspace that is too small: the launch runs unsplit; the residual aliasing the output is refused with a workspace
+    out = torch.full((M, Nn), float("nan"), dtype=torch.bfloat16, device=dev)
+    N.check(N.lib.lbm_linear_norm(ptr(ad), None, ptr(wd), ptr(bd), ptr(gd), ptr(rd), ptr(out), None, M, Nn, K,
+                                  N.LINEAR_BIAS_RESIDUAL, ptr(ws), 1024, None))
+    torch.cuda.synchronize()
+    check(out.cpu(), ref, scale=scale, bar=2.0 ** -6)
+    assert N.lib.lbm_linear_norm(ptr(ad), None, ptr(wd), ptr(bd), ptr(gd), ptr(rd), ptr(rd), None, M, Nn, K,
+                                 N.LINEAR_BIAS_RESIDUAL, ptr(ws), need, None) != N.OK
