@@ -378,8 +378,12 @@ def aggregator_step(torch, blocks: int, steps: int, warmup: int, windows=(WINDOW
     base.py:575-606), special tokens first, group outputs concatenated, all at ViT-L size (dim
     1024, 16 heads, MLP 4096, LayerNorm, LayerScale; qk-norm and rotary embeddings in the
     aggregator blocks), random init, bf16.  The global blocks run the HIP cache path, every
-    block's pre-attention producer and cache-less attention are HIP kernels too; linears,
-    LayerNorm, GELU and the patch convolution are PyTorch-ROCm library calls.  The prediction
+    block's pre-attention producer and cache-less attention are HIP kernels too.  With one
+    stream (one frame's rows per launch) a block is five launches of the package's own GEMM -
+    qkv projection with norm1 folded in and the producer as its store, proj and fc2 with
+    LayerScale + residual in theirs, fc1 with norm2 folded in and the GELU in its store - plus the
+    attention; with several streams batched the linears are PyTorch-ROCm library calls and the
+    LayerNorm / residual steps a HIP kernel.  The patch convolution is PyTorch-ROCm.  The prediction
     heads are not part of the step.  `windows` holds one sliding window per stream: more than
     one entry runs that many independent streams as one ragged batch (a step is then one frame
     of every stream).  `keyframe_interval` > 1 caches every n-th frame only (config 4)."""
@@ -435,8 +439,11 @@ def aggregator_step(torch, blocks: int, steps: int, warmup: int, windows=(WINDOW
             "hip_graph": {"value": B / dt_graph, "unit": "frames/s", "ms_per_step": dt_graph * 1e3},
             "what": f"HipAggregatorStream: patch convolution + 24 encoder blocks + {blocks} x (frame block + global block), "
                     f"dim {H * D}, {H} heads, MLP {4 * H * D}, {B} stream(s), {T} tokens/frame, steady-state cache of {kv} "
-                    f"KV tokens; PyTorch-ROCm for linears / LayerNorm / GELU / convolution, HIP kernels for q/k norm + "
-                    f"rotary + append, the cache path and every block's cache-less attention; prediction heads excluded"}
+                    f"KV tokens; " + ("the package's GEMM with fused LayerNorm / GELU / LayerScale + residual / producer for every "
+                                      "linear" if B == 1 else "PyTorch-ROCm for the linears and GELU, HIP kernels for LayerNorm + residual and "
+                                      "q/k norm + rotary + append") +
+                    ", HIP kernels for the cache path and every block's cache-less attention, PyTorch-ROCm for the patch "
+                    "convolution; prediction heads excluded"}
 
 
 def main() -> None:
@@ -506,7 +513,42 @@ def main() -> None:
                 flop = 2.0 * M * K * Nn
                 rows.append({"layer": name, "M": M, "K": K, "N": Nn, "lbm_linear_us": t_ours, "torch_us": t_theirs,
                              "lbm_linear_tflops": flop / t_ours * 1e-6, "torch_tflops": flop / t_theirs * 1e-6})
-        print(json.dumps({"mode": "linear", "rows": rows}))
+        # the chained forms at one frame's rows: row statistics out of the residual launches (fc2
+        # with K split over two workgroups per tile), LayerNorm folded into the launch that follows
+        chained = []
+        M = 1004
+        for name, K, Nn, epi, fold in (("qkv, norm1 folded in", 1024, 3072, N.LINEAR_BIAS, True),
+                                       ("proj + ls + residual + row statistics", 1024, 1024, N.LINEAR_BIAS_RESIDUAL, False),
+                                       ("fc1 + gelu, norm2 folded in", 1024, 4096, N.LINEAR_BIAS_GELU, True),
+                                       ("fc2 + ls + residual + row statistics, K split", 4096, 1024, N.LINEAR_BIAS_RESIDUAL, False)):
+            a = torch.randn(M, K, generator=g, device=dev).to(torch.bfloat16)
+            w = (torch.randn(Nn, K, generator=g, device=dev) / K ** 0.5).to(torch.bfloat16)
+            b32 = torch.randn(Nn, generator=g, device=dev)
+            g32 = torch.rand(Nn, generator=g, device=dev)
+            res = torch.randn(M, Nn, generator=g, device=dev).to(torch.bfloat16)
+            out = torch.empty(M, Nn, dtype=torch.bfloat16, device=dev)
+            stream = lambda: C.c_void_p(torch.cuda.current_stream().cuda_stream)
+            if fold:
+                tiles = 16
+                xs = a.float().reshape(M, tiles, -1)
+                mean = xs.mean(-1)
+                stats = torch.stack([mean, ((xs - mean[..., None]) ** 2).sum(-1)], -1).contiguous()
+                colsum = w.float().sum(1).contiguous()
+                ln = N.RowNorm(stats.data_ptr(), colsum.data_ptr(), tiles, 1e-5)
+                fn = lambda: N.check(N.lib.lbm_linear_norm(vp(a), ln, vp(w), vp(b32), None, None, vp(out), None, M, Nn, K, epi,
+                                                           None, 0, stream()))
+            else:
+                tiles = N.lib.lbm_linear_stats_tiles(M, Nn)
+                stats = torch.empty(M, tiles, 2, device=dev)
+                need = N.lib.lbm_linear_workspace_bytes(M, Nn, K, epi)
+                ws = torch.zeros(max(need, 256), dtype=torch.uint8, device=dev)
+                fn = lambda: N.check(N.lib.lbm_linear_norm(vp(a), None, vp(w), vp(b32), vp(g32), vp(res), vp(out), vp(stats), M, Nn, K,
+                                                           epi, vp(ws) if need else None, need, stream()))
+            for _ in range(3):
+                fn()
+            t = kernel_time_ms(fn, 50, torch) * 1e3
+            chained.append({"layer": name, "M": M, "K": K, "N": Nn, "lbm_linear_norm_us": t, "tflops": 2.0 * M * K * Nn / t * 1e-6})
+        print(json.dumps({"mode": "linear", "rows": rows, "chained": chained}))
         return
     blocks = args.blocks
     m = HipPagedKVCacheManager(blocks, ANCHOR + WINDOW + 16, T, H, D, torch.bfloat16, dev,
