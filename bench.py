@@ -455,7 +455,7 @@ def main() -> None:
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-aggregator", action="store_true",
                     help="skip the full aggregator-trunk step (frame + global blocks) timed after the hot path")
-    ap.add_argument("--mode", choices=["full", "attention", "attention_frame", "attention_f32", "attention_f32_few", "append", "prepare", "residual", "tables", "copy", "linear"], default="full",
+    ap.add_argument("--mode", choices=["full", "attention", "attention_frame", "attention_f32", "attention_f32_few", "append", "prepare", "residual", "tables", "copy", "linear", "aggregator"], default="full",
                     help="full = the benchmark line; attention/attention_frame (a frame block's 1004 x 1004 without cache)/attention_f32/attention_f32_few/append/prepare/residual/tables launch one kernel --steps "
                          "times on the steady-state cache (for rocprofv3 runs); copy = a plain 256 MiB "
                          "device copy, the known-size kernel the HBM counters are calibrated on")
@@ -477,6 +477,10 @@ def main() -> None:
         ms = event_time_ms(lambda: dst.copy_(src), args.steps, torch)
         print(json.dumps({"mode": "copy", "bytes_read": src.numel(), "bytes_written": dst.numel(),
                           "launches": args.steps, "avg_launch_us": ms * 1e3}))
+        return
+    if args.mode == "aggregator":
+        # the one-stream aggregator step alone (eager, then replayed as HIP graphs)
+        print(json.dumps({"mode": "aggregator", "aggregator_step": aggregator_step(torch, args.blocks, 12, 3)}))
         return
     if args.mode == "linear":
         # the four linears of a block at one frame (1004 rows) and at four streams (4016 rows):
