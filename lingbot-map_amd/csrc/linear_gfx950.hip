@@ -285,8 +285,8 @@ __global__ __launch_bounds__(kGThreads, 1) void lbm_linear_bf16_kernel(LinearArg
     for (int i = 0; i < kLnHeld; ++i)
       if (part + 4 * i < p.ln_tiles) sm += ln_part[i][0];
     for (int i = part + 4 * kLnHeld; i < p.ln_tiles; i += 4) sm += ln_st[2 * i];
-    sm += __shfl_xor(sm, 1);
-    sm += __shfl_xor(sm, 2);
+    sm += lbm_qkv::lane_xor1(sm);
+    sm += lbm_qkv::lane_xor2(sm);
     const float mean = sm / (float)p.ln_tiles;
     const float n_i = (float)p.K / (float)p.ln_tiles;
     float m2 = 0.f;
@@ -300,8 +300,8 @@ __global__ __launch_bounds__(kGThreads, 1) void lbm_linear_bf16_kernel(LinearArg
       const float d = ln_st[2 * i] - mean;
       m2 += ln_st[2 * i + 1] + n_i * d * d;
     }
-    m2 += __shfl_xor(m2, 1);
-    m2 += __shfl_xor(m2, 2);
+    m2 += lbm_qkv::lane_xor1(m2);
+    m2 += lbm_qkv::lane_xor2(m2);
     const float rstd = __builtin_amdgcn_rsqf(m2 / (float)p.K + p.ln_eps);
     if (part == 0) {
       ln_rows[2 * r] = rstd;
@@ -526,14 +526,14 @@ __global__ __launch_bounds__(kGThreads, 1) void lbm_linear_bf16_kernel(LinearArg
         x[2 * e + 1] = bf16_bits_to_f32(v[e] >> 16);
       }
       float sm = ((x[0] + x[1]) + (x[2] + x[3])) + ((x[4] + x[5]) + (x[6] + x[7]));
-#pragma unroll
-      for (int m = 1; m < kPieces; m <<= 1) sm += __shfl_xor(sm, m);
+      sm = lbm_qkv::sum_of_8(sm);
+      if (kPieces == 16) sm += lbm_qkv::other_half_of_16(sm);
       const float mean = sm / (float)TN;
       float m2 = 0.f;
 #pragma unroll
       for (int e = 0; e < 8; ++e) m2 += (x[e] - mean) * (x[e] - mean);
-#pragma unroll
-      for (int m = 1; m < kPieces; m <<= 1) m2 += __shfl_xor(m2, m);
+      m2 = lbm_qkv::sum_of_8(m2);
+      if (kPieces == 16) m2 += lbm_qkv::other_half_of_16(m2);
       if (row < p.M && (tid % kPieces) == 0) {
         float* so = p.stats_out + ((size_t)row * p.n_tiles + nt) * 2;
         so[0] = mean;

@@ -23,6 +23,42 @@ __device__ __forceinline__ float sub_rn(float a, float b) { return a - b; }
 // v_cvt_pk_bf16_f32 rounds the same way
 __device__ __forceinline__ float round_bf16(float f) { return (float)(__bf16)f; }
 
+// Lane exchanges inside aligned groups of 4, 8 and 16 lanes as DPP moves (vector ALU, no LDS
+// round trip as the permute instructions behind __shfl_xor make): xor 1 and xor 2 are quad
+// permutations; once a quad's lanes agree, the mirror of a half row (lane i <-> 7 - i of 8) or of a
+// row (i <-> 15 - i of 16) brings in the value of the other quad / other half, which is what xor 4 /
+// xor 8 would have fetched.
+template <int CTRL>
+__device__ __forceinline__ float dpp_move(float v) {
+  const int i = __builtin_bit_cast(int, v);
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(i, i, CTRL, 0xf, 0xf, true));
+}
+__device__ __forceinline__ float lane_xor1(float v) { return dpp_move<0xB1>(v); }          // quad_perm [1, 0, 3, 2]
+__device__ __forceinline__ float lane_xor2(float v) { return dpp_move<0x4E>(v); }          // quad_perm [2, 3, 0, 1]
+__device__ __forceinline__ float other_quad_of_8(float v) { return dpp_move<0x141>(v); }   // row_half_mirror
+__device__ __forceinline__ float other_half_of_16(float v) { return dpp_move<0x140>(v); }  // row_mirror
+// sum over an aligned group of 8 lanes, every lane ends up with it (same additions, in the same
+// order, as s += xor 1; s += xor 2; s += xor 4)
+__device__ __forceinline__ float sum_of_8(float s) {
+  s += lane_xor1(s);
+  s += lane_xor2(s);
+  s += other_quad_of_8(s);
+  return s;
+}
+
+// sum over the 64 lanes of a wavefront, every lane ends up with it: 16-lane rows by DPP, the four
+// row sums through scalar registers
+__device__ __forceinline__ float sum_of_wave(float s) {
+  s = sum_of_8(s);
+  s += other_half_of_16(s);
+  const int bits = __builtin_bit_cast(int, s);
+  const float r0 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(bits, 0));
+  const float r1 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(bits, 16));
+  const float r2 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(bits, 32));
+  const float r3 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(bits, 48));
+  return (r0 + r1) + (r2 + r3);
+}
+
 // x: this lane's elements 8 c .. 8 c + 7 of the row (c = lane % 8; the row's 8 lanes are
 // consecutive and aligned, so the shuffles below stay inside it).  SRC 0: bf16 activations
 // (roundings after the LayerNorm, of cos and sin, and after every product and sum), 1: fp32.
@@ -36,16 +72,12 @@ __device__ __forceinline__ void norm_rope(float (&x)[8], const f32x4 (&w4)[2], c
     float s = 0.f;
 #pragma unroll
     for (int i = 0; i < 8; ++i) s += x[i];
-    s += __shfl_xor(s, 1);
-    s += __shfl_xor(s, 2);
-    s += __shfl_xor(s, 4);
+    s = sum_of_8(s);
     const float mean = s * (1.0f / 64.0f);
     float v = 0.f;
 #pragma unroll
     for (int i = 0; i < 8; ++i) v += (x[i] - mean) * (x[i] - mean);
-    v += __shfl_xor(v, 1);
-    v += __shfl_xor(v, 2);
-    v += __shfl_xor(v, 4);
+    v = sum_of_8(v);
     const float rstd = __builtin_amdgcn_rsqf(v * (1.0f / 64.0f) + eps);  // torch's LayerNorm uses rsqrt too
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
@@ -86,7 +118,7 @@ __device__ __forceinline__ void norm_rope(float (&x)[8], const f32x4 (&w4)[2], c
         const int i = 2 * p + j;
         float co = q4[2 * j], si = q4[2 * j + 1];
         const float own = x[i];
-        const float other = __shfl_xor(own, 2);
+        const float other = lane_xor2(own);
         if (SRC == 0) {
           co = round_bf16(co);
           si = round_bf16(si);

@@ -13,6 +13,7 @@
 // rounded once.  For fp32 activations every step is a separately rounded fp32 operation.
 #include <hip/hip_runtime.h>
 #include "lbm_internal.h"
+#include "qkv_math.h"
 
 typedef __attribute__((ext_vector_type(4))) unsigned int u32x4;
 typedef __attribute__((ext_vector_type(4))) float f32x4;
@@ -60,8 +61,7 @@ __device__ __forceinline__ void store8(void* base, long long elem, const float (
 
 // sum over the 128 threads of the workgroup (two wavefronts)
 __device__ __forceinline__ float block_sum(float v, float* lds2) {
-#pragma unroll
-  for (int o = 32; o >= 1; o >>= 1) v += __shfl_xor(v, o);
+  v = lbm_qkv::sum_of_wave(v);
   const int wave = threadIdx.x >> 6;
   __syncthreads();  // lds2 may still be read from the previous reduction
   if ((threadIdx.x & 63) == 0) lds2[wave] = v;
@@ -199,8 +199,7 @@ __global__ __launch_bounds__(256) void lbm_residual_norm_wave_kernel(ResidualNor
     }
   }
   if (!has_norm) return;
-#pragma unroll
-  for (int o = 32; o >= 1; o >>= 1) sum += __shfl_xor(sum, o);
+  sum = lbm_qkv::sum_of_wave(sum);
   const float mean = sum / (float)a.cols;
   float sq = 0.f;
 #pragma unroll
@@ -209,8 +208,7 @@ __global__ __launch_bounds__(256) void lbm_residual_norm_wave_kernel(ResidualNor
 #pragma unroll
       for (int i = 0; i < 8; ++i) sq += (v[c][i] - mean) * (v[c][i] - mean);
     }
-#pragma unroll
-  for (int o = 32; o >= 1; o >>= 1) sq += __shfl_xor(sq, o);
+  sq = lbm_qkv::sum_of_wave(sq);
   const float rstd = __builtin_amdgcn_rsqf(sq / (float)a.cols + a.eps);
 #pragma unroll
   for (int c = 0; c < NV; ++c) {
