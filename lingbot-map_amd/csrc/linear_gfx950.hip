@@ -9,6 +9,16 @@
 // Roundings follow the sequence of separate bf16 torch ops: the linear's output is rounded to
 // bf16, then each elementwise op rounds again.
 //
+// Around that, so that a transformer block needs no LayerNorm, residual or producer launch:
+//   * the residual epilogue can leave the row statistics (mean, M2 per column tile) of what it
+//     stores (block.py:283-285 feeding the next LayerNorm);
+//   * a launch can take activations whose LayerNorm is still to be applied: the product runs on
+//     the raw rows and the store applies rstd * (acc - mean * colsum(w)) + bias, the LayerNorm's
+//     affine part folded into w and bias by the caller (block.py:194-195, 217; the normalised rows
+//     are then never rounded to bf16, the folded weights are);
+//   * the qkv projection can carry the pre-attention producer as its epilogue (kEpiQkvPrepare);
+//   * a launch with few tiles and a long K can put several workgroups on a tile (SPLITK).
+//
 // Shapes this is written for: M about 1,000 rows per stream (one frame), K, N in 1024 .. 4096.
 // At that size a launch has only a few hundred tiles and 16-64 k-steps, so what counts is a
 // tile count that matches the 256 CUs and a short prologue, not asymptotic throughput.
