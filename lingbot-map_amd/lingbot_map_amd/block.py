@@ -515,9 +515,7 @@ class HipPagedAttention(nn.Module):
 
     def forward(self, x: Tensor, pos=None, num_patches=None, num_special=None, num_frames=None,
                 enable_3d_rope=False, kv_cache=None, global_idx=0, num_frame_per_block=1,
-                num_frame_for_scale=-1, num_register_tokens=4, project: bool = True) -> Tensor:
-        """The reference's arguments (attention.py:428-441); ``project=False`` returns the heads'
-        output before ``proj`` (for a caller that fuses the projection with what follows)."""
+                num_frame_for_scale=-1, num_register_tokens=4) -> Tensor:
         B, N, _ = x.shape
         has_manager = kv_cache is not None and hasattr(kv_cache, "append_frame")
         if not has_manager:
@@ -546,7 +544,7 @@ class HipPagedAttention(nn.Module):
                 q, k, v = self.prepare_qkv(x, pos=pos, enable_3d_rope=enable_3d_rope)
                 out = self.stream_attend(kv_cache, global_idx, q, k, v, num_register_tokens)
             out = out.reshape(B, N, self.num_heads * self.head_dim).to(x.dtype)
-        return self.proj(out) if project else out
+        return self.proj(out)
 
 
 class HipPagedBlock(nn.Module):
