@@ -23,18 +23,19 @@
 // At that size a launch has only a few hundred tiles and 16-64 k-steps, so what counts is a
 // tile count that matches the 256 CUs and a short prologue, not asymptotic throughput.
 //
-// One workgroup = 8 wavefronts on a 128 x 128 tile of the output (TN = 64: 128 x 64), k-steps of
-// 128.  The product is computed transposed, C^T = W A^T with v_mfma_f32_32x32x16_bf16 (A operand
-// = 32 rows of W, B operand = 32 rows of the activations), so an accumulator register holds
-// four consecutive output columns of one row.  The eight wavefronts are two groups of four:
-// each group covers the whole tile (a wavefront owns 64 x TN / 2 of it) over its own half of
-// every k-step, which gives each SIMD two wavefronts to cover each other's LDS and barrier
-// waits without giving up the fragment reuse of the large per-wave tile; the two groups' sums
-// meet through LDS once, at the end.  Both operands are K-contiguous and travel global ->
-// registers -> LDS (rows of 128 elements padded to 272 bytes: neither the b128 fragment reads nor
-// the b128 stores put two lanes on one bank) two k-steps ahead of the multiply, the LDS stores
-// two per 16-wide slice in the shadow of the MFMAs, one workgroup barrier per k-step.  The tile
-// leaves through LDS as whole rows: 16-byte stores, and the residual is read the same way.
+// One workgroup = 8 wavefronts on a 128 x 128 tile of the output (TN = 64: 128 x 64).  The product
+// is computed transposed, C^T = W A^T with v_mfma_f32_32x32x16_bf16 (A operand = 32 rows of W, B
+// operand = 32 rows of the activations), so an accumulator register holds four consecutive output
+// columns of one row.  The eight wavefronts are two groups of four: each group covers the whole
+// tile (a wavefront owns 64 x TN / 2 of it) over its own half of every K slice, which gives each
+// SIMD two wavefronts to cover each other's LDS and barrier waits without giving up the fragment
+// reuse of the large per-wave tile; the two groups' sums meet through LDS once, at the end.
+// Both operands are K-contiguous and travel global -> LDS directly (global_load_lds_dwordx4, no
+// registers and no LDS store instructions in between) in 64-wide slices of K, four LDS stages,
+// three slices ahead of the multiply; rows are unpadded and their 16-byte chunks XOR-swizzled by
+// the choice of source address, so the b128 fragment reads are free of bank conflicts.  One
+// workgroup barrier per slice.  The tile leaves through LDS as whole rows: 16-byte stores, and
+// the residual is read the same way.
 #include <hip/hip_runtime.h>
 #include "lbm_internal.h"
 #include "qkv_math.h"
@@ -51,10 +52,11 @@ typedef __attribute__((ext_vector_type(2))) float f32x2;
 typedef __attribute__((ext_vector_type(4))) unsigned int u32x4;
 typedef __attribute__((ext_vector_type(2))) unsigned int u32x2;
 
-constexpr int kGK = 128;         // k-step of the workgroup (64 per wave group)
-constexpr int kGStride = 136;    // bf16 per LDS row of a k-step (128 elements + 16 bytes: 272 B)
+constexpr int kGK = 128;         // K granularity the launches accept
 constexpr int kGM = 128;         // activation rows per tile
 constexpr int kGThreads = 512;
+constexpr int kKS = 64;          // K elements per LDS stage
+constexpr int kStagesG = 4;      // LDS stages: three being loaded while one is multiplied
 
 struct LinearArgs {
   const unsigned short* a;       // [M, K]
@@ -151,12 +153,13 @@ template <int EPI, int TN, int ROPE = 0, bool NORM = false, bool LNA = false, bo
 __global__ __launch_bounds__(kGThreads, 1) void lbm_linear_bf16_kernel(LinearArgs p) {
   constexpr int NT = TN / 64;   // 32-column blocks of W per wavefront
   // [buffer][k half][row][64 + pad]
-  __shared__ __attribute__((aligned(16))) unsigned short lds_a[2][kGM * kGStride];
-  __shared__ __attribute__((aligned(16))) unsigned short lds_w[2][TN * kGStride];
+  // [stage][row][64]: 64-wide slices of K, kStagesG of them in flight or in use
+  __shared__ __attribute__((aligned(16))) unsigned short lds_a[kStagesG][kGM * kKS];
+  __shared__ __attribute__((aligned(16))) unsigned short lds_w[kStagesG][TN * kKS];
   __shared__ unsigned short gelu_tab[EPI == LBM_LINEAR_BIAS_GELU ? kGeluEntries : 1];
   __shared__ __attribute__((aligned(8))) float ln_rows[LNA ? kGM * 2 : 2];   // per row of the tile: rstd, -mean * rstd
 
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int n32 = lane & 31, g = lane >> 5;
   const int kh = wave >> 2, ws = wave & 3;    // k half of this wave's group, its sub-tile
   // Workgroups are dealt to the 8 XCDs round-robin: an XCD keeps its own column tiles of W (read
@@ -187,39 +190,47 @@ __global__ __launch_bounds__(kGThreads, 1) void lbm_linear_bf16_kernel(LinearArg
   const int m0 = mt * kGM, n0 = nt * TN;
   const int wm = (ws & 1) * 64, wn = (ws >> 1) * (TN / 2);
 
-  // ---- staging: thread t moves the 16-byte piece (t & 15) of rows (t >> 4) + 32 j of a k-step
-  constexpr int kPassA = kGM / 32, kPassW = TN / 32;
-  const int ld_r = tid >> 4, ld_c = (tid & 15) * 8;          // ld_c: element within the 128 of the k-step
-  // 32-bit byte offsets from uniform bases (a scalar base + a vector offset per load instead of a
-  // 64-bit vector address per row pass: 11 registers less)
+  // ---- staging.  Operands travel global -> LDS without passing through registers
+  // (global_load_lds_dwordx4: a wavefront's 64 lanes x 16 bytes land as one contiguous KB, i.e.
+  // eight whole 128-byte rows of a 64-wide K slice; wavefront w covers rows 8 w .. 8 w + 7 of every
+  // block of 64 rows).  Rows are not padded; instead the 16-byte chunk c of row r sits at chunk
+  // position c ^ ((r >> 1) & 7), which the lane arranges by asking for the chunk that belongs at
+  // ITS position - then the b128 fragment reads of 16 rows at one logical chunk hit all 64 banks.
+  constexpr int kPassA = kGM / 64, kPassW = TN / 64;
+  const int ld_r = wave * 8 + (lane >> 3);                                   // row within a block of 64
+  const unsigned sw_c = (unsigned)(((lane & 7) ^ ((ld_r >> 1) & 7)) * 8);    // logical element offset this lane fetches
   unsigned a_off[kPassA];
 #pragma unroll
-  for (int j = 0; j < kPassA; ++j) a_off[j] = ((unsigned)min(m0 + ld_r + 32 * j, p.M - 1) * (unsigned)p.K + ld_c) * 2u;   // rows past M re-read the last row
-  const unsigned w_off = ((unsigned)ld_r * (unsigned)p.K + ld_c) * 2u;
-  const int nk = SPLITK ? p.K / kGK / p.k_splits : p.K / kGK;   // k-steps of this workgroup
-  const size_t k_first = SPLITK ? (size_t)split * nk * kGK : 0;
+  for (int j = 0; j < kPassA; ++j) a_off[j] = ((unsigned)min(m0 + ld_r + 64 * j, p.M - 1) * (unsigned)p.K + sw_c) * 2u;   // rows past M re-read the last row
+  const unsigned w_off = ((unsigned)ld_r * (unsigned)p.K + sw_c) * 2u;
+  const int nk = (SPLITK ? p.K / p.k_splits : p.K) / kKS;   // 64-wide steps of this workgroup
+  const size_t k_first = SPLITK ? (size_t)split * nk * kKS : 0;
   const char* a_base = (const char*)(p.a + k_first);
   const char* w_base = (const char*)(p.w + (size_t)n0 * p.K + k_first);
-  auto load_a = [&](int j, int ks) -> u32x4 { return *(const u32x4*)(a_base + ks * (kGK * 2) + a_off[j]); };
-  auto load_w = [&](int j, int ks) -> u32x4 {
-    return *(const u32x4*)(w_base + ((size_t)(32 * j) * p.K + (size_t)ks * kGK) * 2 + w_off);
+  // The loads are written as inline assembly: the compiler would otherwise wait for every
+  // LDS-direct load in flight before any LDS read that might alias it (it cannot tell the two
+  // buffers apart), which serialises load and multiply.  M0 carries the LDS address of the
+  // wavefront's KB; nothing else in this kernel uses M0.  The waits for these loads are placed
+  // by hand (dma_wait) - the compiler's own counts only see fewer loads in flight than there
+  // are, which makes its waits stricter, never laxer.
+  auto dma_row = [&](const char* base, unsigned voff, const unsigned short* lds_dst) {
+    const unsigned m0v = (unsigned)(size_t)(__attribute__((address_space(3))) const void*)lds_dst;
+    asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1"
+                 :
+                 : "v"(voff), "s"(base), "s"(__builtin_amdgcn_readfirstlane(m0v))
+                 : "memory");
   };
-  // Two register sets: the rows of k-step s are asked for at the top of iteration s - 2 and
-  // written into the LDS buffer at the end of iteration s - 1, so a load has two multiply
-  // phases to arrive before anything waits for it.
-  u32x4 ra0[kPassA], rw0[kPassW], ra1[kPassA], rw1[kPassW];
-  auto load_step = [&](int ks, u32x4 (&ra)[kPassA], u32x4 (&rw)[kPassW]) {
+  auto dma_step = [&](int ks, int stage) {
 #pragma unroll
-    for (int j = 0; j < kPassA; ++j) ra[j] = load_a(j, ks);
+    for (int j = 0; j < kPassA; ++j)
+      dma_row(a_base + ks * (kKS * 2), a_off[j], &lds_a[stage][(64 * j + 8 * wave) * kKS]);
 #pragma unroll
-    for (int j = 0; j < kPassW; ++j) rw[j] = load_w(j, ks);
+    for (int j = 0; j < kPassW; ++j)
+      dma_row(w_base + ((size_t)(64 * j) * p.K + (size_t)ks * kKS) * 2, w_off, &lds_w[stage][(64 * j + 8 * wave) * kKS]);
   };
-  auto store_step = [&](int buf, const u32x4 (&ra)[kPassA], const u32x4 (&rw)[kPassW]) {
-#pragma unroll
-    for (int j = 0; j < kPassA; ++j) *(u32x4*)&lds_a[buf][(ld_r + 32 * j) * kGStride + ld_c] = ra[j];
-#pragma unroll
-    for (int j = 0; j < kPassW; ++j) *(u32x4*)&lds_w[buf][(ld_r + 32 * j) * kGStride + ld_c] = rw[j];
-  };
+  // loads of this wavefront still allowed in flight: N (vmcnt(N); expcnt and lgkmcnt untouched)
+  constexpr int kDmaPerStep = kPassA + kPassW;
+#define LBM_DMA_WAIT(N) __builtin_amdgcn_s_waitcnt(0x0F70 | ((N) & 15) | (((N) >> 4) << 14))
 
   f32x16 acc[NT][2];   // [column block of W][row block of A]; element i: column 8 (i / 4) + 4 g + i % 4, row n32
 #pragma unroll
@@ -229,50 +240,34 @@ __global__ __launch_bounds__(kGThreads, 1) void lbm_linear_bf16_kernel(LinearArg
 #pragma unroll
       for (int i = 0; i < 16; ++i) acc[a][b][i] = 0.f;
 
-  // One k-step: the fragments of 16-wide slice j + 1 are read while the MFMAs of slice j run,
-  // and the rows of the step after next (held in `ra`, `rw` since the previous iteration) go
-  // into the other LDS buffer two stores per slice, in the shadow of the MFMAs, followed by the
-  // loads that refill the set.  sched_barrier keeps the slices as written.
-  auto step = [&](int buf, u32x4 (&ra)[kPassA], u32x4 (&rw)[kPassW], int next_ks) {
-    const unsigned short* la = &lds_a[buf][kh * 64];
-    const unsigned short* lw = &lds_w[buf][kh * 64];
+  // One 64-wide step on stage `stage`: each wave group multiplies its 32-wide half, the fragments
+  // of the second 16-wide slice read while the MFMAs of the first run.
+  const int sw_r = (n32 >> 1) & 7;
+  auto step = [&](int stage) {
+    const unsigned short* la = &lds_a[stage][0];
+    const unsigned short* lw = &lds_w[stage][0];
     bf16x8 wf[2][NT], af[2][2];
     auto read = [&](int k16, bf16x8 (&wfr)[NT], bf16x8 (&afr)[2]) {
+      const int pos = ((kh * 4 + k16 * 2 + g) ^ sw_r) * 8;
 #pragma unroll
       for (int a = 0; a < NT; ++a)
-        wfr[a] = __builtin_bit_cast(bf16x8, *(const u32x4*)&lw[(wn + a * 32 + n32) * kGStride + k16 * 16 + g * 8]);
+        wfr[a] = __builtin_bit_cast(bf16x8, *(const u32x4*)&lw[(wn + a * 32 + n32) * kKS + pos]);
 #pragma unroll
       for (int b = 0; b < 2; ++b)
-        afr[b] = __builtin_bit_cast(bf16x8, *(const u32x4*)&la[(wm + b * 32 + n32) * kGStride + k16 * 16 + g * 8]);
+        afr[b] = __builtin_bit_cast(bf16x8, *(const u32x4*)&la[(wm + b * 32 + n32) * kKS + pos]);
     };
     read(0, wf[0], af[0]);
+    read(1, wf[1], af[1]);
 #pragma unroll
-    for (int k16 = 0; k16 < 4; ++k16) {
-      if (k16 + 1 < 4) read(k16 + 1, wf[(k16 + 1) & 1], af[(k16 + 1) & 1]);
+    for (int k16 = 0; k16 < 2; ++k16) {
 #pragma unroll
       for (int a = 0; a < NT; ++a)
 #pragma unroll
         for (int b = 0; b < 2; ++b)
-          acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wf[k16 & 1][a], af[k16 & 1][b], acc[a][b], 0, 0, 0);
-      // this slice's share of the stores: the passes j with j % 4 == k16 (after the last k-step
-      // they put a repeat of it into a buffer nobody reads any more: cheaper than a branch per slice)
-#pragma unroll
-      for (int j = 0; j < kPassA; ++j)
-        if ((j & 3) == k16) *(u32x4*)&lds_a[buf ^ 1][(ld_r + 32 * j) * kGStride + ld_c] = ra[j];
-#pragma unroll
-      for (int j = 0; j < kPassW; ++j)
-        if ((j & 3) == k16) *(u32x4*)&lds_w[buf ^ 1][(ld_r + 32 * j) * kGStride + ld_c] = rw[j];
-#pragma unroll
-      for (int j = 0; j < kPassA; ++j)
-        if ((j & 3) == k16) ra[j] = load_a(j, next_ks);
-#pragma unroll
-      for (int j = 0; j < kPassW; ++j)
-        if ((j & 3) == k16) rw[j] = load_w(j, next_ks);
-      __builtin_amdgcn_sched_barrier(0);
+          acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wf[k16][a], af[k16][b], acc[a][b], 0, 0, 0);
     }
   };
 
-  const int last = nk - 1;                       // steps past the end re-read the last one (never multiplied)
   // LNA, row statistics: row r of the tile is handled by threads 4 r .. 4 r + 3, each taking every
   // fourth (mean, M2) partial; equal-sized partials merge as mean = avg(mean_i),
   // M2 = sum(M2_i) + n_i * sum((mean_i - mean)^2) (Chan et al.), variance = M2 / K.  The partials
@@ -286,8 +281,10 @@ __global__ __launch_bounds__(kGThreads, 1) void lbm_linear_bf16_kernel(LinearArg
     for (int i = 0; i < kLnHeld; ++i)
       if ((tid & 3) + 4 * i < p.ln_tiles) ln_part[i] = *(const f32x2*)(ln_st + 2 * ((tid & 3) + 4 * i));
   }
-  load_step(0, ra0, rw0);
-  load_step(min(1, last), ra1, rw1);
+  // three steps ahead: steps 0, 1, 2 on their way before anything else happens
+#pragma unroll
+  for (int i = 0; i < kStagesG - 1; ++i)
+    if (i < nk) dma_step(i, i);
   if (LNA) {
     const int r = tid >> 2, part = tid & 3;
     float sm = 0.f;
@@ -327,18 +324,24 @@ __global__ __launch_bounds__(kGThreads, 1) void lbm_linear_bf16_kernel(LinearArg
       gelu_tab[i] = __builtin_bit_cast(unsigned short, (__bf16)gelu_erf(bf16_bits_to_f32(bits)));
     }
   }
-  store_step(0, ra0, rw0);
-  load_step(min(2, last), ra0, rw0);
-  __syncthreads();
-  // iteration ks multiplies buffer ks & 1 and moves the set holding step ks + 1 into the other
-  // buffer, then refills that set with step ks + 3
-  for (int ks = 0; ks < nk; ks += 2) {
-    step(0, ra1, rw1, min(ks + 3, last));
-    __syncthreads();
-    if (ks + 1 >= nk) break;
-    step(1, ra0, rw0, min(ks + 4, last));
-    __syncthreads();
+  // Step s: wait until its rows have landed (the loads of at most two later steps may still be in
+  // flight), barrier (everyone's rows of step s are there, and everyone is done with step s - 1,
+  // whose stage is the one step s + 3 lands in), ask for step s + 3, multiply step s.
+  for (int s0 = 0; s0 < nk; s0 += kStagesG) {
+#pragma unroll
+    for (int st = 0; st < kStagesG; ++st) {
+      const int sidx = s0 + st;
+      if (sidx < nk) {
+        if (sidx + 2 < nk) LBM_DMA_WAIT(2 * kDmaPerStep);
+        else if (sidx + 1 < nk) LBM_DMA_WAIT(kDmaPerStep);
+        else LBM_DMA_WAIT(0);
+        __syncthreads();
+        if (sidx + kStagesG - 1 < nk) dma_step(sidx + kStagesG - 1, (st + kStagesG - 1) % kStagesG);
+        step(st);
+      }
+    }
   }
+  __syncthreads();
 
   // ---- the two wave groups' sums meet: group 0 finishes row block 0 of every sub-tile, group 1
   // row block 1; each parks the other's half in LDS (the operand buffers are dead)
