@@ -552,7 +552,23 @@ def main() -> None:
                 fn()
             t = kernel_time_ms(fn, 50, torch) * 1e3
             chained.append({"layer": name, "M": M, "K": K, "N": Nn, "lbm_linear_norm_us": t, "tflops": 2.0 * M * K * Nn / t * 1e-6})
-        print(json.dumps({"mode": "linear", "rows": rows, "chained": chained}))
+        # time against K at one shape: slope = the loop per 128 of K, intercept = launch, prologue, store
+        sweep = []
+        Nn = 3072
+        for K in (256, 512, 1024, 2048, 4096):
+            a = torch.randn(M, K, generator=g, device=dev).to(torch.bfloat16)
+            w = (torch.randn(Nn, K, generator=g, device=dev) / K ** 0.5).to(torch.bfloat16)
+            b = torch.randn(Nn, generator=g, device=dev).to(torch.bfloat16)
+            b32 = b.float()
+            out = torch.empty(M, Nn, dtype=torch.bfloat16, device=dev)
+            stream = lambda: C.c_void_p(torch.cuda.current_stream().cuda_stream)
+            ours = lambda: N.check(N.lib.lbm_linear(vp(a), vp(w), vp(b32), None, None, vp(out), M, Nn, K, N.LINEAR_BIAS, stream()))
+            theirs = lambda: F.linear(a, w, b)
+            for _ in range(3):
+                ours(); theirs()
+            sweep.append({"M": M, "N": Nn, "K": K, "lbm_linear_us": kernel_time_ms(ours, 50, torch) * 1e3,
+                          "torch_us": kernel_time_ms(theirs, 50, torch) * 1e3})
+        print(json.dumps({"mode": "linear", "rows": rows, "chained": chained, "k_sweep": sweep}))
         return
     blocks = args.blocks
     m = HipPagedKVCacheManager(blocks, ANCHOR + WINDOW + 16, T, H, D, torch.bfloat16, dev,
