@@ -37,7 +37,8 @@
 // block written as 20 slices (22 with the extra k-step; one MFMA plus its share of the vector
 // work and LDS reads each) fenced with sched_barrier, and the two wavefronts of a SIMD fill
 // each other's issue gaps.  K/V tiles are shared by all eight waves through a three-stage
-// LDS ring with one workgroup barrier per tile.
+// LDS ring with one workgroup barrier per tile; the rows go from global memory straight into
+// the ring (global_load_lds_dwordx4), no staging registers and no LDS store instructions.
 #include <hip/hip_runtime.h>
 #include <climits>
 #include <mutex>
@@ -61,8 +62,9 @@ constexpr int kWaves = 8;
 constexpr int kThreads = kWaves * 64;
 constexpr int kQTile = kQPerWave * kWaves;
 constexpr int kStages = 3;              // LDS ring depth
-constexpr int kKStride = 72;            // bf16 per LDS row of K: 144 B, b128 reads hit 64 distinct banks
-constexpr int kVStride = 96;            // bf16 per LDS row of V: 192 B, 4-row transpose reads conflict-free
+constexpr int kRingRow = 64;            // bf16 per row of a K/V tile in the LDS ring: 128 B, unpadded, 16-byte chunks swizzled
+constexpr int kKStride = 72;            // bf16 per row of a padded patch (Q, short-KV K, output transpose): 144 B, b128 reads hit 64 distinct banks
+constexpr int kVStride = 96;            // bf16 per row of the short-KV kernel's V patch: 192 B, 4-row transpose reads conflict-free
 constexpr float kHeadroom = 11.0f;      // the softmax reference is set this far above the row maxima (log2 units)
 
 struct AttnCore {
@@ -114,9 +116,9 @@ __device__ __forceinline__ float swap_max(float x) {
 
 // LDS of the split-KV kernel, at namespace scope because the kernel and the out-of-line second
 // pass below both work in it.
-__shared__ __attribute__((aligned(16))) unsigned short lds_k[kStages][kKvTile * kKStride];
-__shared__ __attribute__((aligned(16))) unsigned short lds_v[kStages][kKvTile * kVStride];
-__shared__ __attribute__((aligned(16))) unsigned short lds_q[kWaves][kQPerWave * kKStride];   // per-wave patch: Q on the way in
+__shared__ __attribute__((aligned(1024))) unsigned short lds_k[kStages][kKvTile * kRingRow];
+__shared__ __attribute__((aligned(1024))) unsigned short lds_v[kStages][kKvTile * kRingRow];
+__shared__ __attribute__((aligned(16))) unsigned short lds_q[kWaves][kQPerWave * kKStride];   // per-wave patch: Q on the way in, O on the way out
 
 // The repeat pass is a function of its own, not inlined: it is entered once in a blue moon,
 // and compiled into the kernel body its registers would push the common path into scratch
@@ -132,7 +134,7 @@ __device__ __noinline__ void lbm_attn_split_safe(AttnCore a, LbmAttnStreamPlan s
 // the call.  SAFE = true is the repeat with a reference that follows the row maxima.
 template <bool SAFE>
 __device__ __forceinline__ void lbm_attn_split(const AttnCore& a, const LbmAttnStreamPlan& sp) {
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int n32 = lane & 31, g = lane >> 5;
 
   // ---- which piece of this stream's work is this workgroup
@@ -171,38 +173,50 @@ __device__ __forceinline__ void lbm_attn_split(const AttnCore& a, const LbmAttnS
   const int n = t1 - t0;
   const unsigned row_bytes = (unsigned)H * 128u;
 
-  // ---- tile staging: each thread moves one 16-byte piece of a K row and of a V row per tile.
+  // ---- tile staging: each thread moves one 16-byte piece of a K row and of a V row per tile,
+  // global -> LDS without a stop in registers (global_load_lds_dwordx4: the wavefront's 64
+  // pieces land on 1 KiB of consecutive LDS starting at M0, i.e. on eight 128-byte rows).  A
+  // tile in the ring is therefore 64 unpadded rows, and what keeps the fragment reads off each
+  // other's banks is the order of the eight 16-byte chunks within a row, which each lane
+  // chooses by the global address it reads: chunk c of K row r sits at position
+  // c ^ ((r >> 1) & 7) (the b128 fragment reads of 16 rows x one chunk hit all 64 banks), chunk
+  // c of V row r at c ^ 4 ((r >> 1) & 1) (the 8-byte transposed reads touch four rows x 64
+  // bytes; rows r+2 and r+3 move to the other half).  The compiler does not count these loads
+  // (its own waits only get stricter by that); LBM_DMA_LANDED waits for them before the
+  // barrier that publishes a tile.  Nothing else in this kernel uses M0.
   // Rows past the last token re-read the last token (finite data; the softmax masks them).
-  const int ld_r = tid >> 3, ld_c = (tid & 7) * 8;
-  const char* pool_k = (const char*)(a.pool + (size_t)head * 64 + ld_c);
-  const char* pool_v = pool_k + (size_t)a.page_size * row_bytes;
-  const char* own_k = (const char*)(a.self_k + (size_t)head * 64 + ld_c);
-  const char* own_v = (const char*)(a.self_v + (size_t)head * 64 + ld_c);
+  const int ld_r = tid >> 3;
+  const int ld_ck = ((lane & 7) ^ ((ld_r >> 1) & 7)) * 8, ld_cv = ((lane & 7) ^ (((ld_r >> 1) & 1) * 4)) * 8;
+  const char* pool_k = (const char*)(a.pool + (size_t)head * 64 + ld_ck);
+  const char* pool_v = (const char*)(a.pool + (size_t)head * 64 + ld_cv) + (size_t)a.page_size * row_bytes;
+  const char* own_k = (const char*)(a.self_k + (size_t)head * 64 + ld_ck);
+  const char* own_v = (const char*)(a.self_v + (size_t)head * 64 + ld_cv);
   const int32_t* rows = a.kv_rows + sp.kv_row_begin;
   const int last_token = max(kv_tokens - 1, 0);
   // Tiles past the end of this split re-read its last tile: the data lands in ring stages
   // nobody reads any more, and the code stays free of branches.
   auto row_entry = [&](int t) -> int { return rows[min(max(min(t, t1 - 1), 0) * kKvTile + ld_r, last_token)]; };
-  auto fetch = [&](int e, const char* pool_base, const char* own_base) -> u32x4 {
+  auto dma = [&](int e, const char* pool_base, const char* own_base, const unsigned short* lds_tile) {
     // negative entries name rows of the caller's own K/V (read-only tail of a non-keyframe)
     const char* base = e < 0 ? own_base : pool_base;
     const unsigned r = (unsigned)(e ^ (e >> 31));
-    return *(const u32x4*)(base + (unsigned long long)r * row_bytes);
+    const char* src = base + (unsigned long long)r * row_bytes;
+    const unsigned m0v = (unsigned)(size_t)(__attribute__((address_space(3))) const void*)(lds_tile + wave * (8 * kRingRow));
+    asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off"
+                 :
+                 : "v"(src), "s"(__builtin_amdgcn_readfirstlane(m0v))
+                 : "memory");
   };
-  auto put_k = [&](int stage, u32x4 v) { *(u32x4*)&lds_k[stage][ld_r * kKStride + ld_c] = v; };
-  auto put_v = [&](int stage, u32x4 v) { *(u32x4*)&lds_v[stage][ld_r * kVStride + ld_c] = v; };
+#define LBM_DMA_LANDED() __builtin_amdgcn_s_waitcnt(0x0F70)   /* vmcnt(0); expcnt and lgkmcnt untouched */
 
   // The first tiles' rows are asked for before anything else: the row table entry, then the K/V
   // row it names, is the longest chain of memory latencies in front of the first MFMA, and the
   // Q rows below travel at the same time.
-  const int e_t0 = row_entry(t0), e_t1 = row_entry(t0 + 1), e_t2 = row_entry(t0 + 2);
-  int ek = row_entry(t0 + 3), ev = e_t2;   // entries of the fetches after those
-  const u32x4 k_t0 = fetch(e_t0, pool_k, own_k);
-  const u32x4 k_t1 = fetch(e_t1, pool_k, own_k);
-  const u32x4 v_t0 = fetch(e_t0, pool_v, own_v);
-  // in flight across the first iteration: K(2), V(1)
-  u32x4 kreg = fetch(e_t2, pool_k, own_k);
-  u32x4 vreg = fetch(e_t1, pool_v, own_v);
+  const int e_t0 = row_entry(t0), e_t1 = row_entry(t0 + 1);
+  int ek = row_entry(t0 + 2), ev = e_t1;   // entries of the loads of the first iteration
+  dma(e_t0, pool_k, own_k, lds_k[0]);
+  dma(e_t1, pool_k, own_k, lds_k[1]);
+  dma(e_t0, pool_v, own_v, lds_v[0]);
 
   // ---- Q fragments (B operand of S^T = K Q^T): lane holds q row n32, d = ks*16 + g*8 .. +8.
   // Each wavefront reads its 64 query rows as whole 128-byte rows (eight lanes per row), parks
@@ -273,11 +287,11 @@ __device__ __forceinline__ void lbm_attn_split(const AttnCore& a, const LbmAttnS
   // ks*16 + {4g..4g+3, 8+4g..8+4g+3} of the V tile in stage st
   auto v_frag = [&](int st, int ks, int db) -> bf16x8 {
     const int row = ks * 16 + 4 * g + ((lane & 15) >> 2);
-    const int col = db * 32 + ((lane >> 4) & 1) * 16 + (lane & 3) * 4;
+    const int col = (db * 32 + ((lane >> 4) & 1) * 16 + (lane & 3) * 4) ^ (((lane >> 3) & 1) * 32);
     const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-        (s16x4 __attribute__((address_space(3)))*)&lds_v[st][row * kVStride + col]);
+        (s16x4 __attribute__((address_space(3)))*)&lds_v[st][row * kRingRow + col]);
     const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-        (s16x4 __attribute__((address_space(3)))*)&lds_v[st][(row + 8) * kVStride + col]);
+        (s16x4 __attribute__((address_space(3)))*)&lds_v[st][(row + 8) * kRingRow + col]);
     s16x8 both;
     both[0] = lo[0]; both[1] = lo[1]; both[2] = lo[2]; both[3] = lo[3];
     both[4] = hi[0]; both[5] = hi[1]; both[6] = hi[2]; both[7] = hi[3];
@@ -305,7 +319,7 @@ __device__ __forceinline__ void lbm_attn_split(const AttnCore& a, const LbmAttnS
 #pragma unroll
     for (int ks = 0; ks < 4; ++ks) {
       const bf16x8 ka = __builtin_bit_cast(
-          bf16x8, *(const u32x4*)&lds_k[st][(h * 32 + n32) * kKStride + ks * 16 + g * 8]);
+          bf16x8, *(const u32x4*)&lds_k[st][(h * 32 + n32) * kRingRow + ((ks * 2 + g) ^ ((n32 >> 1) & 7)) * 8]);
 #pragma unroll
       for (int qb = 0; qb < 2; ++qb)
         sd[qb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka, qf[qb][ks], sd[qb], 0, 0, 0);
@@ -431,7 +445,7 @@ __device__ __forceinline__ void lbm_attn_split(const AttnCore& a, const LbmAttnS
     if ((j) == 1) va[1] = v_frag(st_pv, ks_pv, 1);                                               \
     if ((j) == 10 || (j) == 12 || (j) == 14 || (j) == 16)                                        \
       ka[((j) - 10) >> 1] = __builtin_bit_cast(                                                  \
-          bf16x8, *(const u32x4*)&lds_k[st_qk][((h_qk) * 32 + n32) * kKStride + (((j) - 10) >> 1) * 16 + g * 8]); \
+          bf16x8, *(const u32x4*)&lds_k[st_qk][((h_qk) * 32 + n32) * kRingRow + (((((j) - 10) >> 1) * 2 + g) ^ ((n32 >> 1) & 7)) * 8]); \
     if ((j) == 17) vnext[0] = v_frag(st_vn, ks_vn, 0);                                           \
     if ((j) == 18) vnext[1] = v_frag(st_vn, ks_vn, 1);                                           \
     __builtin_amdgcn_sched_barrier(0);                                                           \
@@ -490,7 +504,7 @@ __device__ __forceinline__ void lbm_attn_split(const AttnCore& a, const LbmAttnS
     if ((j) == 1) va[1] = v_frag(st_pv, ks_pv, 1);                                               \
     if ((j) == 8 || (j) == 10 || (j) == 12 || (j) == 14)                                         \
       ka[((j) - 8) >> 1] = __builtin_bit_cast(                                                   \
-          bf16x8, *(const u32x4*)&lds_k[st_qk][((h_qk) * 32 + n32) * kKStride + (((j) - 8) >> 1) * 16 + g * 8]); \
+          bf16x8, *(const u32x4*)&lds_k[st_qk][((h_qk) * 32 + n32) * kRingRow + (((((j) - 8) >> 1) * 2 + g) ^ ((n32 >> 1) & 7)) * 8]); \
     if ((j) == 16) vnext[0] = v_frag(st_vn, ks_vn, 0);                                           \
     if ((j) == 17) vnext[1] = v_frag(st_vn, ks_vn, 1);                                           \
     __builtin_amdgcn_sched_barrier(0);                                                           \
@@ -535,18 +549,14 @@ __device__ __forceinline__ void lbm_attn_split(const AttnCore& a, const LbmAttnS
       qaug_bits[qb][0] = 0u;
     }
 
-    // ---- prologue: K(0), K(1), V(0) into the ring; the V stage the first PV reads is zeroed
-    put_k(0, k_t0);
-    put_k(1, k_t1);
-    put_v(0, v_t0);
-    {
-      const u32x4 zero = {0u, 0u, 0u, 0u};
-      put_v(2, zero);
-    }
+    // ---- prologue: K(0), K(1), V(0) are on their way into the ring; the V stage the first PV
+    // reads is zeroed
+    *(u32x4*)&lds_v[2][tid * 8] = u32x4{0u, 0u, 0u, 0u};
 #pragma unroll
     for (int qb = 0; qb < 2; ++qb)
 #pragma unroll
       for (int kk = 0; kk < 2; ++kk) pB[qb][kk] = __builtin_bit_cast(bf16x8, u32x4{0u, 0u, 0u, 0u});
+    LBM_DMA_LANDED();
     __syncthreads();
     qk_half(0, 0, kv_tokens - t0 * kKvTile, sA);
     if (safe) {
@@ -564,29 +574,25 @@ __device__ __forceinline__ void lbm_attn_split(const AttnCore& a, const LbmAttnS
     vnext[1] = v_frag(2, 2, 1);
 
     int st_k = 0, st_v = 0, st_vm1 = 2;  // stages of K(i), V(i), V(i-1)
-    // Common frame of one tile iteration.  K/V rows travel global -> registers -> LDS ring with
-    // a full iteration in the registers: the fetches of K(i+3), V(i+2) start at the top of
-    // iteration i, and the rows fetched one iteration earlier (K(i+2), V(i+1), long since
-    // arrived) are written into the ring between the two half-steps, so neither the wait for
-    // the loads nor the LDS write sits in front of the barrier that ends the iteration.  Past
-    // the last tile the data lands in stages nobody reads any more.  The row entry fetched for
-    // K now serves V in the next iteration.
+    // Common frame of one tile iteration.  The loads of K(i+2) and V(i+1) into their ring
+    // stages (free since the barrier that ended iteration i-1) start at the top of iteration
+    // i and have the whole iteration to land; the wait for them sits right before the barrier
+    // that ends it.  Past the last tile the data lands in stages nobody reads any more.  The
+    // row entry fetched for K now serves V in the next iteration.
 #define LBM_TILE_ITERATION(PRE, HALF0, HALF1)                                        \
     {                                                                                \
       const int t = t0 + i;                                                          \
       int st_k1 = st_k + 1; if (st_k1 >= kStages) st_k1 -= kStages;                  \
       int st_k2 = st_k1 + 1; if (st_k2 >= kStages) st_k2 -= kStages;                 \
       int st_v1 = st_v + 1; if (st_v1 >= kStages) st_v1 -= kStages;                  \
-      const u32x4 khold = kreg, vhold = vreg;                                        \
-      kreg = fetch(ek, pool_k, own_k);                                               \
-      vreg = fetch(ev, pool_v, own_v);                                               \
+      dma(ek, pool_k, own_k, lds_k[st_k2]);                                          \
+      dma(ev, pool_v, own_v, lds_v[st_v1]);                                          \
       ev = ek;                                                                       \
-      ek = row_entry(t + 4);                                                         \
+      ek = row_entry(t + 3);                                                         \
       PRE                                                                            \
       HALF0                                                                          \
-      put_k(st_k2, khold);                                                           \
-      put_v(st_v1, vhold);                                                           \
       HALF1                                                                          \
+      LBM_DMA_LANDED();                                                              \
       __syncthreads();                                                               \
       st_k = st_k1;                                                                  \
       st_vm1 = st_v;                                                                 \
@@ -659,10 +665,9 @@ __device__ __forceinline__ void lbm_attn_split(const AttnCore& a, const LbmAttnS
 
   // ---- epilogue.  The accumulators hold O^T (a lane owns 4-element runs of 32 different
   // rows); written straight out that is 32 scattered 8-byte stores per instruction.  Each
-  // wavefront instead transposes its rows through LDS (the ring is dead by now) and stores
-  // whole 128-byte rows, eight lanes per row.
-  __syncthreads();  // every wave has finished reading the ring
-  unsigned short* stage = &lds_v[0][0] + wave * (32 * kKStride);
+  // wavefront instead transposes its rows through its Q patch (idle since the prologue) and
+  // stores whole 128-byte rows, eight lanes per row.
+  unsigned short* stage = lds_q[wave];
   const bool direct = sp.n_splits == 1;
   unsigned short* dst = direct ? a.out : a.part_o;
   const size_t dst_row0 = direct ? (size_t)sp.q_begin : (size_t)sp.part_begin + (size_t)split * sp.q_rows;
