@@ -101,48 +101,27 @@ struct LinearArgs {
 constexpr int kEpiQkvPrepare = 3;   // internal: reached through lbm_qkv_linear_prepare only
 
 __device__ __forceinline__ float round_bf16(float f) { return (float)(__bf16)f; }
-// Exact (erf) GELU as torch evaluates it in fp32, 0.5 v (1 + erf(v / sqrt 2)).  erf comes from the
-// Chebyshev fit erfc(z) = t exp(-z^2 + P(t)), t = 1 / (1 + z / 2), z >= 0 (Numerical Recipes,
-// erfcc: fractional error below 1.2e-7 for every z) - a sixth of the library erff's
-// instructions.  In the negative tail 1 + erf cancels and torch's result carries the last bits
-// of ITS erff, so there (v < -3: a few elements per thousand behind a LayerNorm) the library
-// function is called, behind a wave-uniform branch.
-__device__ __forceinline__ float gelu_erf(float v) {
-  const float x = 0.70710678118654752440f * v;
-  const float z = __builtin_fabsf(x);
-  const float t = __builtin_amdgcn_rcpf(__builtin_fmaf(0.5f, z, 1.0f));
-  float p = 0.17087277f;
-  p = __builtin_fmaf(p, t, -0.82215223f);
-  p = __builtin_fmaf(p, t, 1.48851587f);
-  p = __builtin_fmaf(p, t, -1.13520398f);
-  p = __builtin_fmaf(p, t, 0.27886807f);
-  p = __builtin_fmaf(p, t, -0.18628806f);
-  p = __builtin_fmaf(p, t, 0.09678418f);
-  p = __builtin_fmaf(p, t, 0.37409196f);
-  p = __builtin_fmaf(p, t, 1.00002368f);
-  p = __builtin_fmaf(p, t, -1.26551223f);
-  const float e = t * __builtin_amdgcn_exp2f(1.44269504088896340736f * __builtin_fmaf(-z, z, p));   // erfc(z)
-  float erf_x = 1.0f - e;
-  erf_x = x < 0.f ? -erf_x : erf_x;
-  const bool tail = v < -3.0f;
-  if (__builtin_amdgcn_ballot_w64(tail)) {
-    const float lib = erff(x);
-    erf_x = tail ? lib : erf_x;
-  }
-  return 0.5f * v * (1.0f + erf_x);
-}
 __device__ __forceinline__ float bf16_bits_to_f32(unsigned v) { return __builtin_bit_cast(float, v << 16); }
-// The GELU of the fused fc1 epilogue acts on a value already rounded to bf16 and is rounded to
-// bf16 again: a function from 16 bits to 16 bits.  Evaluating it costs about 32 vector
-// instructions per element (more where the negative tail calls erff), 4 us of a 20 us launch;
-// the workgroup instead tabulates it in LDS for |v| in [2^-12, 2^3) - 15 binades x 128 mantissas
-// x 2 signs, 7.5 KB, filled from gelu_erf while the first operand tiles are on their way - and
-// looks the elements up.  Values outside the table (tiny, huge, inf, NaN: a handful per
-// million behind a LayerNorm) are evaluated directly behind a wave-uniform branch, so every
-// result is gelu_erf's, bit for bit.
+// The GELU of the fused fc1 epilogue (torch's exact-erf nn.GELU, lingbot_map/layers/mlp.py:24) acts
+// on a value already rounded to bf16 and is rounded to bf16 again: a function from 16 bits to
+// 16 bits.  Evaluated per element it costs about 32 vector instructions, 4 us of a 20 us launch;
+// instead it is tabulated for |v| in [2^-12, 2^3) - 15 binades x 128 mantissas x 2 signs, 7.5 KB,
+// exact values rounded once (gen_gelu_table.py) - and each workgroup pulls the table into LDS with
+// one 16-byte LDS-direct load per thread, ahead of its first operand tiles, and looks the
+// elements up, without a branch, so that the lookups of a lane's 32 elements overlap.
+// Outside the table the function has closed forms that agree with torch's fp32 evaluation
+// after the rounding to bf16: below 2^-12, 1 + erf differs from 1 by less than 2^-12 and
+// v / 2 is the nearest bf16 value (zeros and denormals included); from 8 up erff is exactly
+// +-1, so the result is v on the positive side (+inf and NaN included) and v * 0 on the
+// negative side (-0, and NaN for -inf and NaN, like 0.5 * v * (1 - 1)).  Between -8 and -3,
+// where torch's 1 + erff cancels and its result carries the last bits of its erff, the table
+// holds the exact value, within one bf16 step of torch's.
 constexpr int kGeluE0 = 127 - 12;              // biased exponent of the first tabulated binade
 constexpr int kGeluHalf = 15 * 128;            // entries per sign
 constexpr int kGeluEntries = 2 * kGeluHalf;
+static __device__ __attribute__((aligned(16))) const unsigned short g_gelu_table[kGeluEntries] = {
+#include "gelu_table.inc"
+};
 
 // TN: output columns per tile (128 or 64); a wavefront owns 64 x (TN / 2) of the tile.
 // ROPE / NORM: rotary layout (0 none, 1 interleaved, 2 half-split) and qk-LayerNorm of the
@@ -156,7 +135,7 @@ __global__ __launch_bounds__(kGThreads, 1) void lbm_linear_bf16_kernel(LinearArg
   // [stage][row][64]: 64-wide slices of K, kStagesG of them in flight or in use
   __shared__ __attribute__((aligned(16))) unsigned short lds_a[kStagesG][kGM * kKS];
   __shared__ __attribute__((aligned(16))) unsigned short lds_w[kStagesG][TN * kKS];
-  __shared__ unsigned short gelu_tab[EPI == LBM_LINEAR_BIAS_GELU ? kGeluEntries : 1];
+  __shared__ __attribute__((aligned(16))) unsigned short gelu_tab[EPI == LBM_LINEAR_BIAS_GELU ? kGeluEntries : 8];
   __shared__ __attribute__((aligned(8))) float ln_rows[LNA ? kGM * 2 : 2];   // per row of the tile: rstd, -mean * rstd
 
   const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -281,7 +260,11 @@ __global__ __launch_bounds__(kGThreads, 1) void lbm_linear_bf16_kernel(LinearArg
     for (int i = 0; i < kLnHeld; ++i)
       if ((tid & 3) + 4 * i < p.ln_tiles) ln_part[i] = *(const f32x2*)(ln_st + 2 * ((tid & 3) + 4 * i));
   }
-  // three steps ahead: steps 0, 1, 2 on their way before anything else happens
+  // The GELU table travels first (480 threads x 16 bytes; the loads return in order, so the wait
+  // for the first operand tile covers it and the barrier behind that wait publishes it) ...
+  if (EPI == LBM_LINEAR_BIAS_GELU && tid < kGeluEntries / 8)
+    dma_row((const char*)g_gelu_table, (unsigned)tid * 16u, &gelu_tab[wave * 512]);
+  // ... then three steps ahead: steps 0, 1, 2 on their way before anything else happens
 #pragma unroll
   for (int i = 0; i < kStagesG - 1; ++i)
     if (i < nk) dma_step(i, i);
@@ -315,14 +298,6 @@ __global__ __launch_bounds__(kGThreads, 1) void lbm_linear_bf16_kernel(LinearArg
       ln_rows[2 * r + 1] = -mean * rstd;
     }
     // (read in the epilogue, many barriers from here)
-  }
-  if (EPI == LBM_LINEAR_BIAS_GELU) {
-    // (under the latency of the loads above; the barrier before the first multiply publishes it)
-    for (int i = tid; i < kGeluEntries; i += kGThreads) {
-      const unsigned neg = i >= kGeluHalf ? 1u : 0u;
-      const unsigned bits = (neg << 15) | (unsigned)((kGeluE0 << 7) + (i - (int)neg * kGeluHalf));
-      gelu_tab[i] = __builtin_bit_cast(unsigned short, (__bf16)gelu_erf(bf16_bits_to_f32(bits)));
-    }
   }
   // Step s: wait until its rows have landed (the loads of at most two later steps may still be in
   // flight), barrier (everyone's rows of step s are there, and everyone is done with step s - 1,
@@ -432,15 +407,12 @@ __global__ __launch_bounds__(kGThreads, 1) void lbm_linear_bf16_kernel(LinearArg
         float v = round_bf16(lin + bias4[e]);
         if (EPI == LBM_LINEAR_BIAS_GELU) {
           const unsigned b16 = __builtin_bit_cast(unsigned, v) >> 16;
-          const unsigned rel = (b16 & 0x7fffu) - (unsigned)(kGeluE0 << 7);
-          const bool tabulated = rel < (unsigned)kGeluHalf;
-          const unsigned looked_up = gelu_tab[min(rel, (unsigned)(kGeluHalf - 1)) + (b16 >> 15) * kGeluHalf];
-          float r = bf16_bits_to_f32(looked_up);
-          if (__builtin_amdgcn_ballot_w64(!tabulated)) {
-            const float direct = gelu_erf(v);
-            r = tabulated ? r : direct;
-          }
-          v = r;
+          const unsigned mag = b16 & 0x7fffu, neg = b16 >> 15;
+          const unsigned rel = mag - (unsigned)(kGeluE0 << 7);
+          const unsigned looked_up = gelu_tab[min(rel, (unsigned)(kGeluHalf - 1)) + neg * kGeluHalf];
+          // outside the table: v / 2 below it, v or v * 0 above it (see kGeluE0)
+          const float outside = mag < (unsigned)(kGeluE0 << 7) ? 0.5f * v : (neg ? v * 0.0f : v);
+          v = rel < (unsigned)kGeluHalf ? bf16_bits_to_f32(looked_up) : outside;
         }
         if (EPI == LBM_LINEAR_BIAS_RESIDUAL && p.gamma) v = v * gamma4[e];
         y[e] = v;

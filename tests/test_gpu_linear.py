@@ -73,8 +73,8 @@ def test_gelu_epilogue_on_every_bf16_pre_activation():
     a 512 x 128 weight matrix puts every finite bf16 bit pattern through the epilogue: the
     tabulated range, the values below and above it, both zeros, the negative tail.  torch's GELU
     of the same bf16 values is the expectation: bit-equal from -3 up (zeros compare equal whatever
-    their sign), within one bf16 ulp of the pre-activation's scale below -3, where the result is
-    the last bits of an erff."""
+    their sign), within one bf16 ulp of the pre-activation's scale below -3, where torch's result
+    is the last bits of its erff (1 + erf cancels) and the table holds the exact value."""
     N = _native()
     bits = torch.arange(65536, dtype=torch.int32)
     exp_field = (bits >> 7) & 0xFF
