@@ -56,7 +56,8 @@ constexpr int kGK = 128;         // K granularity the launches accept
 constexpr int kGM = 128;         // activation rows per tile
 constexpr int kGThreads = 512;
 constexpr int kKS = 64;          // K elements per LDS stage
-constexpr int kStagesG = 4;      // LDS stages: three being loaded while one is multiplied
+constexpr int kStagesG = 4;      // LDS stages: three being loaded while one is multiplied (six stages for the 64-column tile,
+                                 // which has the room: slower, 8.4 -> 8.8 us for proj - the longer prologue costs more than the depth gains)
 
 struct LinearArgs {
   const unsigned short* a;       // [M, K]
@@ -318,6 +319,90 @@ __global__ __launch_bounds__(kGThreads, 1) void lbm_linear_bf16_kernel(LinearArg
   }
   __syncthreads();
 
+  // What the epilogue needs from global memory is asked for here, all at once, and arrives while
+  // the wave groups exchange their sums (asked for where it is used - per column group, per
+  // pass - every load would wait out a trip to L2 or HBM on its own, and behind the stores of
+  // the pass before it; asked for before the multiply, it delays the first operand tiles): the
+  // per-column vectors of this lane's accumulator columns ...
+  f32x4 bias_v[NT][4], colsum_v[NT][4], gamma_v[NT][4];
+#pragma unroll
+  for (int a = 0; a < NT; ++a)
+#pragma unroll
+    for (int c4 = 0; c4 < 4; ++c4) {
+      bias_v[a][c4] = f32x4{0.f, 0.f, 0.f, 0.f};
+      colsum_v[a][c4] = f32x4{0.f, 0.f, 0.f, 0.f};
+      gamma_v[a][c4] = f32x4{1.f, 1.f, 1.f, 1.f};
+    }
+  {
+    const int col0 = n0 + wn + g * 4;     // + a * 32 + c4 * 8: four consecutive output columns
+    if (p.bias) {
+#pragma unroll
+      for (int a = 0; a < NT; ++a)
+#pragma unroll
+        for (int c4 = 0; c4 < 4; ++c4) bias_v[a][c4] = *(const f32x4*)(p.bias + col0 + a * 32 + c4 * 8);
+    }
+    if (LNA) {
+#pragma unroll
+      for (int a = 0; a < NT; ++a)
+#pragma unroll
+        for (int c4 = 0; c4 < 4; ++c4) colsum_v[a][c4] = *(const f32x4*)(p.ln_colsum + col0 + a * 32 + c4 * 8);
+    }
+    if (EPI == LBM_LINEAR_BIAS_RESIDUAL && p.gamma) {
+#pragma unroll
+      for (int a = 0; a < NT; ++a)
+#pragma unroll
+        for (int c4 = 0; c4 < 4; ++c4) gamma_v[a][c4] = *(const f32x4*)(p.gamma + col0 + a * 32 + c4 * 8);
+    }
+  }
+  // ... and the residual rows of the store passes (a workgroup that shares its tile under SPLITK
+  // asks only once it knows that it is the one to store).
+  constexpr int kPieces = TN / 8;                 // 16-byte pieces per row of the tile
+  constexpr int kRowsPerPass = kGThreads / kPieces;
+  constexpr int kPasses = kGM / kRowsPerPass;
+  u32x4 res_v[kPasses] = {};
+  auto load_residual = [&]() {
+#pragma unroll
+    for (int j = 0; j < kPasses; ++j) {
+      const int row = min(m0 + j * kRowsPerPass + tid / kPieces, p.M - 1);   // rows past M: read, never stored
+      res_v[j] = *(const u32x4*)(p.res + (size_t)row * p.N + n0 + (tid % kPieces) * 8);
+    }
+  };
+  if (EPI == LBM_LINEAR_BIAS_RESIDUAL && !SPLITK) load_residual();
+  // The producer's own inputs - q/k norm weights, every pass's rotary table entries and pool rows -
+  // are asked for now as well.
+  const int H = p.num_heads;
+  struct {
+    int c, which, h, c8;
+    lbm_qkv::f32x4 w4[2], b4[2], cs4[kPasses][4];
+    int pool_row[kPasses];
+  } pq = {};
+  if (EPI == kEpiQkvPrepare) {
+    typedef lbm_qkv::f32x4 qf4;
+    pq.c = (tid % kPieces) * 8;
+    const int col = n0 + pq.c;                    // column of the projection: [q|k|v][head][64]
+    pq.which = col / (H * 64);                    // uniform over the workgroup (H * 64 is a multiple of TN)
+    pq.h = (col - pq.which * H * 64) >> 6;
+    pq.c8 = (col & 63) >> 3;                      // = tid % 8: the lane's place in its row of 64
+    if (NORM && pq.which < 2) {
+      const qf4* wp = (const qf4*)((pq.which == 0 ? p.q_norm_w : p.k_norm_w) + pq.c8 * 8);
+      const qf4* bp = (const qf4*)((pq.which == 0 ? p.q_norm_b : p.k_norm_b) + pq.c8 * 8);
+      pq.w4[0] = wp[0]; pq.w4[1] = wp[1];
+      pq.b4[0] = bp[0]; pq.b4[1] = bp[1];
+    }
+#pragma unroll
+    for (int j = 0; j < kPasses; ++j) {
+      const int t = min(m0 + j * kRowsPerPass + tid / kPieces, p.M - 1);
+      if (ROPE == 1 && pq.which < 2) {
+        const qf4* cs = (const qf4*)(p.rope_cs + ((long long)t * 32 + pq.c8 * 4) * 2);
+        pq.cs4[j][0] = cs[0]; pq.cs4[j][1] = cs[1];
+      } else if (ROPE == 2 && pq.which < 2) {
+        const qf4* cs = (const qf4*)(p.rope_cs + ((long long)t * 64 + pq.c8 * 8) * 2);
+        pq.cs4[j][0] = cs[0]; pq.cs4[j][1] = cs[1]; pq.cs4[j][2] = cs[2]; pq.cs4[j][3] = cs[3];
+      }
+      pq.pool_row[j] = -1;
+      if (pq.which > 0 && p.append_rows) pq.pool_row[j] = p.append_rows[t];
+    }
+  }
   // ---- the two wave groups' sums meet: group 0 finishes row block 0 of every sub-tile, group 1
   // row block 1; each parks the other's half in LDS (the operand buffers are dead)
   float* xch = (float*)&lds_a[0][0];            // [wave][NT][16][64 lanes] floats
@@ -364,6 +449,7 @@ __global__ __launch_bounds__(kGThreads, 1) void lbm_linear_bf16_kernel(LinearArg
     if (ticket_lds != (unsigned)(p.k_splits - 1)) return;          // (uniform over the workgroup)
     if (tid == 0) __hip_atomic_store(&p.split_counters[tile], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // as the next launch expects it
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+    if (EPI == LBM_LINEAR_BIAS_RESIDUAL) load_residual();
     // two slices: this workgroup's own sum is still in its registers and a + b = b + a; more
     // slices: all of them from memory, in slice order, so the sum does not depend on who is last
     const bool pair = p.k_splits == 2;
@@ -395,10 +481,7 @@ __global__ __launch_bounds__(kGThreads, 1) void lbm_linear_bf16_kernel(LinearArg
 #pragma unroll
     for (int c4 = 0; c4 < 4; ++c4) {
       const int col = wn + a * 32 + c4 * 8 + g * 4;     // four consecutive output columns
-      f32x4 bias4 = {0.f, 0.f, 0.f, 0.f}, gamma4 = {1.f, 1.f, 1.f, 1.f}, colsum4 = {0.f, 0.f, 0.f, 0.f};
-      if (p.bias) bias4 = *(const f32x4*)(p.bias + n0 + col);
-      if (LNA) colsum4 = *(const f32x4*)(p.ln_colsum + n0 + col);
-      if (EPI == LBM_LINEAR_BIAS_RESIDUAL && p.gamma) gamma4 = *(const f32x4*)(p.gamma + n0 + col);
+      const f32x4 bias4 = bias_v[a][c4], gamma4 = gamma_v[a][c4], colsum4 = colsum_v[a][c4];
       f32x4 y;
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
@@ -420,59 +503,32 @@ __global__ __launch_bounds__(kGThreads, 1) void lbm_linear_bf16_kernel(LinearArg
       *(bf16x4*)&stage[(wm + b * 32 + n32) * kCStride + col] = __builtin_convertvector(y, bf16x4);
     }
   __syncthreads();
-  constexpr int kPieces = TN / 8;                 // 16-byte pieces per row
-  constexpr int kRowsPerPass = kGThreads / kPieces;
   if (EPI == kEpiQkvPrepare) {
     // The staged tile holds the projection's output rounded to bf16, 8 consecutive columns per
     // thread: exactly the producer's layout (8 lanes per (token, q|k|v, head) row of 64), so its
     // LayerNorm, rotary embedding and scatter run here instead of in a pass of their own
     // (lingbot_map/layers/attention.py:402-426, rope.py:438-461, flashinfer_cache.py:215-218).
-    const int H = p.num_heads;
-    const int c = (tid % kPieces) * 8;
-    const int col = n0 + c;                       // column of the projection: [q|k|v][head][64]
-    const int which = col / (H * 64);             // uniform over the workgroup (H * 64 is a multiple of TN)
-    const int h = (col - which * H * 64) >> 6;
-    const int c8 = (col & 63) >> 3;               // = tid % 8: the lane's place in its row of 64
-    typedef lbm_qkv::f32x4 qf4;
-    qf4 w4[2] = {}, b4[2] = {};
-    if (NORM && which < 2) {
-      const qf4* wp = (const qf4*)((which == 0 ? p.q_norm_w : p.k_norm_w) + c8 * 8);
-      const qf4* bp = (const qf4*)((which == 0 ? p.q_norm_b : p.k_norm_b) + c8 * 8);
-      w4[0] = wp[0]; w4[1] = wp[1];
-      b4[0] = bp[0]; b4[1] = bp[1];
-    }
-    unsigned short* dst_plain = which == 0 ? p.out : (which == 1 ? p.k_out : p.v_out);
+    unsigned short* dst_plain = pq.which == 0 ? p.out : (pq.which == 1 ? p.k_out : p.v_out);
 #pragma unroll
-    for (int r0 = 0; r0 < kGM; r0 += kRowsPerPass) {
-      const int r = r0 + tid / kPieces;
-      const int t = min(m0 + r, p.M - 1);         // rows past M compute on (and never store) the last token's entries
-      const bool valid = m0 + r < p.M;
-      qf4 cs4[4] = {};
-      if (ROPE == 1 && which < 2) {
-        const qf4* cs = (const qf4*)(p.rope_cs + ((long long)t * 32 + c8 * 4) * 2);
-        cs4[0] = cs[0]; cs4[1] = cs[1];
-      } else if (ROPE == 2 && which < 2) {
-        const qf4* cs = (const qf4*)(p.rope_cs + ((long long)t * 64 + c8 * 8) * 2);
-        cs4[0] = cs[0]; cs4[1] = cs[1]; cs4[2] = cs[2]; cs4[3] = cs[3];
-      }
-      int pool_row = -1;
-      if (which > 0 && p.append_rows) pool_row = p.append_rows[t];
-      const u32x2 lo = *(const u32x2*)&stage[r * kCStride + c], hi = *(const u32x2*)&stage[r * kCStride + c + 4];
+    for (int j = 0; j < kPasses; ++j) {
+      const int r = j * kRowsPerPass + tid / kPieces;
+      const bool valid = m0 + r < p.M;            // rows past M computed on the last token's entries, never stored
+      const u32x2 lo = *(const u32x2*)&stage[r * kCStride + pq.c], hi = *(const u32x2*)&stage[r * kCStride + pq.c + 4];
       const u32x4 raw = {lo[0], lo[1], hi[0], hi[1]};
       float x[8];
 #pragma unroll
       for (int i = 0; i < 8; ++i) x[i] = __builtin_bit_cast(float, (i & 1) ? (raw[i >> 1] & 0xffff0000u) : (raw[i >> 1] << 16));
-      if (which < 2) lbm_qkv::norm_rope<0, ROPE, NORM>(x, w4, b4, cs4, c8, p.eps);
+      if (pq.which < 2) lbm_qkv::norm_rope<0, ROPE, NORM>(x, pq.w4, pq.b4, pq.cs4[j], pq.c8, p.eps);
       bf16x8 o8;
 #pragma unroll
       for (int i = 0; i < 8; ++i) o8[i] = (__bf16)x[i];
       if (valid) {
-        const long long nhd = ((long long)(m0 + r) * H + h) * 64 + c8 * 8;
+        const long long nhd = ((long long)(m0 + r) * H + pq.h) * 64 + pq.c8 * 8;
         if (dst_plain) *(bf16x8*)(dst_plain + nhd) = o8;
-        if (which > 0 && pool_row >= 0) {
+        if (pq.which > 0 && pq.pool_row[j] >= 0) {
           const long long row_elems = (long long)H * 64;
-          const long long d = (long long)pool_row * row_elems + (which == 2 ? (long long)p.page_size * row_elems : 0) +
-                              h * 64 + c8 * 8;
+          const long long d = (long long)pq.pool_row[j] * row_elems + (pq.which == 2 ? (long long)p.page_size * row_elems : 0) +
+                              pq.h * 64 + pq.c8 * 8;
           *(bf16x8*)(p.pool + d) = o8;
         }
       }
@@ -480,8 +536,8 @@ __global__ __launch_bounds__(kGThreads, 1) void lbm_linear_bf16_kernel(LinearArg
     return;
   }
 #pragma unroll
-  for (int r0 = 0; r0 < kGM; r0 += kRowsPerPass) {
-    const int r = r0 + tid / kPieces, c = (tid % kPieces) * 8;
+  for (int j = 0; j < kPasses; ++j) {
+    const int r = j * kRowsPerPass + tid / kPieces, c = (tid % kPieces) * 8;
     const int row = m0 + r;
     // (an 8-byte aligned read of the padded row: two halves)
     const u32x2 lo = *(const u32x2*)&stage[r * kCStride + c], hi = *(const u32x2*)&stage[r * kCStride + c + 4];
@@ -489,7 +545,7 @@ __global__ __launch_bounds__(kGThreads, 1) void lbm_linear_bf16_kernel(LinearArg
     if (row < p.M) {
       unsigned short* dst = p.out + (size_t)row * p.N + n0 + c;
       if (EPI == LBM_LINEAR_BIAS_RESIDUAL) {
-        const u32x4 x = *(const u32x4*)(p.res + (size_t)row * p.N + n0 + c);
+        const u32x4 x = res_v[j];
         u32x4 o;
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
