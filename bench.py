@@ -190,7 +190,7 @@ def hbm_kernels_4_streams(torch) -> dict:
     fns = {
         "append": (lambda: m._scatter(0, m._append_rows[0], k, v), 2 * 2 * B * T * H * D * 2),
         "qkv_prepare": (lambda: N.check(N.lib.lbm_qkv_prepare(
-            vp(qkv), N.DTYPE_BF16, vp(ln[0]), vp(ln[1]), vp(ln[2]), vp(ln[3]), 1e-5, vp(cs), N.ROPE_INTERLEAVED, vp(q_out),
+            vp(qkv), N.DTYPE_BF16, vp(ln[0]), vp(ln[1]), vp(ln[2]), vp(ln[3]), 1e-5, 1.0, vp(cs), N.ROPE_INTERLEAVED, vp(q_out),
             None, None, N.DTYPE_BF16, vp(m.kv_caches[0]), vp(m._append_rows[0]), B * T, H, D, PAGE, stream())),
             6 * B * T * H * D * 2 + cs.numel() * 4),
         "residual_norm": (lambda: N.check(N.lib.lbm_residual_norm(
@@ -590,7 +590,7 @@ def main() -> None:
         from lingbot_map_amd import _native as N
         import ctypes as C
         vp = lambda t: C.c_void_p(t.data_ptr())
-        N.check(N.lib.lbm_qkv_prepare(vp(qkv_in), N.DTYPE_BF16, vp(ln[0]), vp(ln[1]), vp(ln[2]), vp(ln[3]), 1e-5,
+        N.check(N.lib.lbm_qkv_prepare(vp(qkv_in), N.DTYPE_BF16, vp(ln[0]), vp(ln[1]), vp(ln[2]), vp(ln[3]), 1e-5, 1.0,
                                       vp(rope_cs), N.ROPE_INTERLEAVED, vp(q_tmp), None, None, N.DTYPE_BF16, vp(m.kv_caches[block]),
                                       vp(m._append_rows[0]), T, H, D, PAGE, m._stream_handle()))
 

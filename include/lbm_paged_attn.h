@@ -24,7 +24,7 @@
 extern "C" {
 #endif
 
-#define LBM_ABI_VERSION 6
+#define LBM_ABI_VERSION 7
 
 #define LBM_OK 0
 #define LBM_ERR_INVALID 1     /* bad argument (null pointer, negative size, bad enum)      */
@@ -38,12 +38,12 @@ extern "C" {
 #define LBM_LAYOUT_TWO_STREAM 0  /* reference: patch pages + packed special stream         */
 #define LBM_LAYOUT_FRAME_PAGES 1 /* whole frame in pages; eviction compacts index-only     */
 
-/* pairing of the rotary embedding in lbm_qkv_prepare */
 /* epilogue of lbm_linear */
 #define LBM_LINEAR_BIAS 0
 #define LBM_LINEAR_BIAS_GELU 1
 #define LBM_LINEAR_BIAS_RESIDUAL 2
 
+/* pairing of the rotary embedding in lbm_qkv_prepare */
 #define LBM_ROPE_INTERLEAVED 0
 #define LBM_ROPE_HALF_SPLIT 1
 
@@ -191,7 +191,8 @@ int lbm_residual_norm(const void* x, const void* y, int32_t dtype, const float* 
  *   a         [M][K] bf16          w      [N][K] bf16 (nn.Linear's weight)
  *   bias      [N] float32 or NULL  gamma  [N] float32 or NULL (RESIDUAL only)
  *   residual  [M][N] bf16 (RESIDUAL only; may alias out)       out  [M][N] bf16
- * K: a multiple of 128, N: a multiple of 64.  Roundings follow the sequence of separate bf16 torch ops (the
+ * K: a multiple of 128, N: a multiple of 64, M * K and N * K below 2^31 elements (LBM_ERR_UNSUPPORTED
+ * otherwise).  Roundings follow the sequence of separate bf16 torch ops (the
  * linear's output rounded to bf16, then each elementwise op). */
 int lbm_linear(const void* a, const void* w, const float* bias, const float* gamma,
                const void* residual, void* out, int32_t M, int32_t N, int32_t K, int32_t epilogue,
@@ -206,7 +207,7 @@ int lbm_linear(const void* a, const void* w, const float* bias, const float* gam
  *   head_dim is 64, K a multiple of 128. */
 int lbm_qkv_linear_prepare(const void* a, const void* w, const float* bias, int32_t M, int32_t K,
                            const float* q_norm_w, const float* q_norm_b, const float* k_norm_w,
-                           const float* k_norm_b, float norm_eps, const float* rope_cs,
+                           const float* k_norm_b, float norm_eps, float q_scale, const float* rope_cs,
                            int32_t rope_layout, void* q_out, void* k_out, void* v_out, void* pool,
                            const int32_t* append_rows, int32_t num_heads, int32_t head_dim,
                            int32_t page_size, void* stream);
@@ -260,7 +261,7 @@ size_t lbm_linear_workspace_bytes(int32_t M, int32_t N, int32_t K, int32_t epilo
 int lbm_qkv_linear_prepare_norm(const void* a, const lbm_row_norm* a_norm, const void* w,
                                 const float* bias, int32_t M, int32_t K, const float* q_norm_w,
                                 const float* q_norm_b, const float* k_norm_w, const float* k_norm_b,
-                                float norm_eps, const float* rope_cs, int32_t rope_layout,
+                                float norm_eps, float q_scale, const float* rope_cs, int32_t rope_layout,
                                 void* q_out, void* k_out, void* v_out, void* pool,
                                 const int32_t* append_rows, int32_t num_heads, int32_t head_dim,
                                 int32_t page_size, void* stream);
@@ -288,6 +289,12 @@ int lbm_attn_run_live(const void* q, const void* pool, void* out, const void* se
  * product and each sum rounded to bf16) and plain fp32 arithmetic when it is fp32.
  *   qkv          [n_tokens][3][num_heads][head_dim], dtype src_dtype
  *   q_norm_w/_b, k_norm_w/_b   [head_dim] float32 LayerNorm affine; all four NULL = no qk-norm
+ *   q_scale      > 0; every q row is multiplied by it in float32 BEFORE the rounding that ends the
+ *                row's last operation (rotary sum, else LayerNorm, else the copy).  1 gives the
+ *                reference's q.  sm_scale * log2(e) gives a q that lbm_attn_run takes with
+ *                sm_scale = 0: the scale then costs q no second rounding to bf16 (the reference
+ *                applies it inside its attention kernel, flashinfer_cache.py:418-421).  k and v
+ *                are never scaled.
  *   rope_cs      NULL = no rotary embedding; otherwise float32 (cos, sin) pairs:
  *                LBM_ROPE_INTERLEAVED  [n_tokens][head_dim / 2][2], element pairs (2i, 2i+1),
  *                  i.e. torch.view_as_real of the complex freqs of apply_rotary_emb (rope.py:438-461)
@@ -300,7 +307,7 @@ int lbm_attn_run_live(const void* q, const void* pool, void* out, const void* se
  * head_dim must be 64. */
 int lbm_qkv_prepare(const void* qkv, int32_t src_dtype, const float* q_norm_w,
                     const float* q_norm_b, const float* k_norm_w, const float* k_norm_b,
-                    float norm_eps, const float* rope_cs, int32_t rope_layout, void* q_out,
+                    float norm_eps, float q_scale, const float* rope_cs, int32_t rope_layout, void* q_out,
                     void* k_out, void* v_out, int32_t dst_dtype, void* pool,
                     const int32_t* append_rows, int32_t n_tokens, int32_t num_heads,
                     int32_t head_dim, int32_t page_size, void* stream);
@@ -323,6 +330,10 @@ size_t lbm_attn_workspace_bytes(const lbm_attn_stream* streams, int32_t n_stream
  *                  the pool or of this array, so a table that is too short or names rows outside
  *                  the pool makes the kernel read out of bounds.  Tables written by
  *                  lbm_tables_step / lbm_rows_from_pages satisfy this by construction.
+ *   sm_scale       > 0: the softmax scale (the reference's 1 / sqrt(head_dim)).  The bf16 kernels
+ *                  fold sm_scale * log2(e) into q, which rounds q to bf16 a second time.
+ *                  0: q already carries sm_scale * log2(e) (a producer run with that q_scale)
+ *                  and is used as it is.
  *   A stream with kv_tokens == 0 gets zeros; a stream with q_rows == 0 launches nothing. */
 int lbm_attn_run(const void* q, const void* pool, void* out, const void* self_k,
                  const void* self_v, const int32_t* kv_rows, const lbm_attn_stream* streams,

@@ -100,7 +100,7 @@ int lbm_kv_append(const void* k, const void* v, int32_t src_dtype, void* pool, i
 }
 
 int lbm_qkv_prepare(const void* qkv, int32_t src_dtype, const float* q_norm_w, const float* q_norm_b,
-                    const float* k_norm_w, const float* k_norm_b, float norm_eps, const float* rope_cs,
+                    const float* k_norm_w, const float* k_norm_b, float norm_eps, float q_scale, const float* rope_cs,
                     int32_t rope_layout, void* q_out, void* k_out, void* v_out, int32_t dst_dtype, void* pool,
                     const int32_t* append_rows, int32_t n_tokens, int32_t num_heads, int32_t head_dim,
                     int32_t page_size, void* stream) {
@@ -117,7 +117,8 @@ int lbm_qkv_prepare(const void* qkv, int32_t src_dtype, const float* q_norm_w, c
   if (append_rows && !pool) return lbm_fail(LBM_ERR_INVALID, "lbm_qkv_prepare: append_rows without a pool");
   if (rope_cs && rope_layout != LBM_ROPE_INTERLEAVED && rope_layout != LBM_ROPE_HALF_SPLIT)
     return lbm_fail(LBM_ERR_INVALID, "lbm_qkv_prepare: unknown rope_layout %d", rope_layout);
-  return lbm_launch_qkv_prepare(qkv, src_dtype, q_norm_w, q_norm_b, k_norm_w, k_norm_b, norm_eps, rope_cs, rope_layout, q_out,
+  if (!(q_scale > 0.f)) return lbm_fail(LBM_ERR_INVALID, "lbm_qkv_prepare: q_scale must be positive (1 = plain q), got %g", (double)q_scale);
+  return lbm_launch_qkv_prepare(qkv, src_dtype, q_norm_w, q_norm_b, k_norm_w, k_norm_b, norm_eps, q_scale, rope_cs, rope_layout, q_out,
                                 k_out, v_out, dst_dtype, pool, append_rows, n_tokens, num_heads, page_size,
                                 (hipStream_t)stream);
 }
@@ -152,19 +153,20 @@ int32_t lbm_linear_stats_tiles(int32_t M, int32_t N) {
 
 int lbm_qkv_linear_prepare(const void* a, const void* w, const float* bias, int32_t M, int32_t K,
                            const float* q_norm_w, const float* q_norm_b, const float* k_norm_w,
-                           const float* k_norm_b, float norm_eps, const float* rope_cs, int32_t rope_layout,
+                           const float* k_norm_b, float norm_eps, float q_scale, const float* rope_cs, int32_t rope_layout,
                            void* q_out, void* k_out, void* v_out, void* pool, const int32_t* append_rows,
                            int32_t num_heads, int32_t head_dim, int32_t page_size, void* stream) {
-  return lbm_qkv_linear_prepare_norm(a, nullptr, w, bias, M, K, q_norm_w, q_norm_b, k_norm_w, k_norm_b, norm_eps, rope_cs,
+  return lbm_qkv_linear_prepare_norm(a, nullptr, w, bias, M, K, q_norm_w, q_norm_b, k_norm_w, k_norm_b, norm_eps, q_scale, rope_cs,
                                      rope_layout, q_out, k_out, v_out, pool, append_rows, num_heads, head_dim, page_size,
                                      stream);
 }
 
 int lbm_qkv_linear_prepare_norm(const void* a, const lbm_row_norm* a_norm, const void* w, const float* bias, int32_t M,
                                 int32_t K, const float* q_norm_w, const float* q_norm_b, const float* k_norm_w,
-                                const float* k_norm_b, float norm_eps, const float* rope_cs, int32_t rope_layout,
+                                const float* k_norm_b, float norm_eps, float q_scale, const float* rope_cs, int32_t rope_layout,
                                 void* q_out, void* k_out, void* v_out, void* pool, const int32_t* append_rows,
                                 int32_t num_heads, int32_t head_dim, int32_t page_size, void* stream) {
+  if (!(q_scale > 0.f)) return lbm_fail(LBM_ERR_INVALID, "lbm_qkv_linear_prepare: q_scale must be positive (1 = plain q), got %g", (double)q_scale);
   if (!a || !w || !q_out) return lbm_fail(LBM_ERR_INVALID, "lbm_qkv_linear_prepare: null a, w or q_out");
   if (M < 0 || K <= 0 || num_heads <= 0) return lbm_fail(LBM_ERR_INVALID, "lbm_qkv_linear_prepare: bad shape");
   if (head_dim != 64) return lbm_fail(LBM_ERR_UNSUPPORTED, "lbm_qkv_linear_prepare: head_dim must be 64 (got %d)", head_dim);
@@ -174,7 +176,7 @@ int lbm_qkv_linear_prepare_norm(const void* a, const lbm_row_norm* a_norm, const
     return lbm_fail(LBM_ERR_INVALID, "lbm_qkv_linear_prepare: unknown rope_layout %d", rope_layout);
   if (append_rows && !pool) return lbm_fail(LBM_ERR_INVALID, "lbm_qkv_linear_prepare: append_rows without a pool");
   if (append_rows && page_size <= 0) return lbm_fail(LBM_ERR_INVALID, "lbm_qkv_linear_prepare: bad page_size");
-  return lbm_launch_qkv_linear_prepare(a, a_norm, w, bias, M, K, q_norm_w, q_norm_b, k_norm_w, k_norm_b, norm_eps, rope_cs,
+  return lbm_launch_qkv_linear_prepare(a, a_norm, w, bias, M, K, q_norm_w, q_norm_b, k_norm_w, k_norm_b, norm_eps, q_scale, rope_cs,
                                        rope_layout, q_out, k_out, v_out, pool, append_rows, num_heads, page_size,
                                        (hipStream_t)stream);
 }
@@ -217,6 +219,7 @@ static int lbm_attn_run_impl(const char* who, const void* q, const void* pool, v
   if (rc != LBM_OK) return rc;
   if (!q || !pool || !out || !kv_rows) return lbm_fail(LBM_ERR_INVALID, "%s: null q, pool, out or kv_rows", who);
   if (num_heads <= 0 || head_dim <= 0 || page_size <= 0) return lbm_fail(LBM_ERR_INVALID, "%s: non-positive size", who);
+  if (!(sm_scale >= 0.f)) return lbm_fail(LBM_ERR_INVALID, "%s: sm_scale must be positive, or 0 for a q that already carries it (got %g)", who, (double)sm_scale);
   if ((self_k == nullptr) != (self_v == nullptr)) return lbm_fail(LBM_ERR_INVALID, "%s: self_k and self_v go together", who);
   if (live_kv_tokens)
     for (int i = 0; i < n_streams; ++i)

@@ -24,7 +24,7 @@ int lbm_launch_append(const void* k, const void* v, int src_dtype, void* pool, i
                       int page_size, hipStream_t stream);
 
 int lbm_launch_qkv_prepare(const void* qkv, int src_dtype, const float* q_norm_w, const float* q_norm_b,
-                           const float* k_norm_w, const float* k_norm_b, float norm_eps,
+                           const float* k_norm_w, const float* k_norm_b, float norm_eps, float q_scale,
                            const float* rope_cs, int rope_layout, void* q_out, void* k_out, void* v_out,
                            int dst_dtype, void* pool, const int32_t* append_rows, int n_tokens,
                            int num_heads, int page_size, hipStream_t stream);
@@ -41,7 +41,7 @@ size_t lbm_linear_workspace_for(int M, int N, int K, int epilogue);
 
 int lbm_launch_qkv_linear_prepare(const void* a, const lbm_row_norm* a_norm, const void* w, const float* bias, int M, int K,
                                   const float* q_norm_w, const float* q_norm_b, const float* k_norm_w,
-                                  const float* k_norm_b, float norm_eps, const float* rope_cs, int rope_layout,
+                                  const float* k_norm_b, float norm_eps, float q_scale, const float* rope_cs, int rope_layout,
                                   void* q_out, void* k_out, void* v_out, void* pool, const int32_t* append_rows,
                                   int num_heads, int page_size, hipStream_t stream);
 

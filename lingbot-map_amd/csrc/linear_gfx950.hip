@@ -79,6 +79,7 @@ struct LinearArgs {
   unsigned short* pool;
   const int32_t* append_rows;    // null: nothing is appended
   float eps;
+  float q_scale;                 // q rows are multiplied by this in fp32 before their last rounding (1 = plain q)
   int num_heads, page_size;
   // LNA kernels: the rows of the activations are standardised, (x - mean) * rstd, without ever
   // being rewritten: the product runs on the raw rows and the store applies
@@ -190,7 +191,8 @@ __global__ __launch_bounds__(kGThreads, 1) void lbm_linear_bf16_kernel(LinearArg
   // The loads are written as inline assembly: the compiler would otherwise wait for every
   // LDS-direct load in flight before any LDS read that might alias it (it cannot tell the two
   // buffers apart), which serialises load and multiply.  M0 carries the LDS address of the
-  // wavefront's KB; nothing else in this kernel uses M0.  The waits for these loads are placed
+  // wavefront's KB (declared as clobbered, so the compiler keeps nothing of its own in M0 across
+  // the load).  The waits for these loads are placed
   // by hand (dma_wait) - the compiler's own counts only see fewer loads in flight than there
   // are, which makes its waits stricter, never laxer.
   auto dma_row = [&](const char* base, unsigned voff, const unsigned short* lds_dst) {
@@ -198,7 +200,7 @@ __global__ __launch_bounds__(kGThreads, 1) void lbm_linear_bf16_kernel(LinearArg
     asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1"
                  :
                  : "v"(voff), "s"(base), "s"(__builtin_amdgcn_readfirstlane(m0v))
-                 : "memory");
+                 : "memory", "m0");
   };
   auto dma_step = [&](int ks, int stage) {
 #pragma unroll
@@ -429,9 +431,10 @@ __global__ __launch_bounds__(kGThreads, 1) void lbm_linear_bf16_kernel(LinearArg
     // Partials and counters travel as scope-qualified relaxed atomics, which go past the caches
     // that are not coherent between workgroups (the CU's and, between XCDs, the L2) - a
     // device-wide fence would write back and invalidate the whole L2 instead, once per
-    // workgroup (measured: 60 us on a 25 us launch).  Order: a thread's stores are complete
-    // (the workgroup-scope fence waits for their acknowledgements), the barrier collects all
-    // threads, thread 0 draws the ticket.
+    // workgroup (measured: 60 us on a 25 us launch).  Order: every thread waits until its own
+    // stores are acknowledged (an explicit s_waitcnt vmcnt(0): the stores are write-through, so an
+    // acknowledged store is visible device-wide, and a workgroup-scope fence alone does not wait
+    // for it), the barrier collects all threads, only then thread 0 draws the ticket.
     __shared__ unsigned ticket_lds;
     const int tile = mt * p.n_tiles + nt;
     constexpr int kPartFloats = 8 * NT * 16 * 64;                 // one workgroup's partial tile
@@ -443,6 +446,7 @@ __global__ __launch_bounds__(kGThreads, 1) void lbm_linear_bf16_kernel(LinearArg
       for (int i = 0; i < 16; ++i)
         __hip_atomic_store(&mine[(a * 16 + i) * 64 + lane], fin[a][i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    LBM_DMA_WAIT(0);
     __syncthreads();
     if (tid == 0) ticket_lds = __hip_atomic_fetch_add(&p.split_counters[tile], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     __syncthreads();
@@ -518,7 +522,7 @@ __global__ __launch_bounds__(kGThreads, 1) void lbm_linear_bf16_kernel(LinearArg
       float x[8];
 #pragma unroll
       for (int i = 0; i < 8; ++i) x[i] = __builtin_bit_cast(float, (i & 1) ? (raw[i >> 1] & 0xffff0000u) : (raw[i >> 1] << 16));
-      if (pq.which < 2) lbm_qkv::norm_rope<0, ROPE, NORM>(x, pq.w4, pq.b4, pq.cs4[j], pq.c8, p.eps);
+      if (pq.which < 2) lbm_qkv::norm_rope<0, ROPE, NORM>(x, pq.w4, pq.b4, pq.cs4[j], pq.c8, p.eps, pq.which == 0 ? p.q_scale : 1.0f);
       bf16x8 o8;
 #pragma unroll
       for (int i = 0; i < 8; ++i) o8[i] = (__bf16)x[i];
@@ -600,6 +604,13 @@ int lbm_linear_tiles(LinearArgs& p) {
 }  // namespace
 
 namespace {
+// the kernel addresses a row of either operand with a 32-bit byte offset from a 64-bit base
+bool lbm_offsets_fit(int M, int N, int K) {
+  return (long long)M * K * 2 < (1LL << 32) && (long long)N * K * 2 < (1LL << 32);
+}
+}  // namespace
+
+namespace {
 // the folded LayerNorm of the activations, checked and copied into the kernel arguments
 int lbm_set_row_norm(LinearArgs& p, const lbm_row_norm* ln, const char* who) {
   if (!ln) return LBM_OK;
@@ -649,6 +660,8 @@ int lbm_launch_linear(const void* a, const lbm_row_norm* a_norm, const void* w, 
   if (M == 0) return LBM_OK;
   if (K % kGK != 0 || N % 64 != 0)
     return lbm_fail(LBM_ERR_UNSUPPORTED, "lbm_linear: K must be a multiple of 128 and N of 64 (got K %d, N %d)", K, N);
+  if (!lbm_offsets_fit(M, N, K))
+    return lbm_fail(LBM_ERR_UNSUPPORTED, "lbm_linear: M * K and N * K must stay below 2^31 elements (32-bit byte offsets), got %d x %d x %d", M, N, K);
   if (a_norm && epilogue == LBM_LINEAR_BIAS_RESIDUAL)
     return lbm_fail(LBM_ERR_UNSUPPORTED, "lbm_linear: no row standardisation with the residual epilogue");
   if (out_stats && epilogue != LBM_LINEAR_BIAS_RESIDUAL)
@@ -698,12 +711,14 @@ int lbm_launch_linear(const void* a, const lbm_row_norm* a_norm, const void* w, 
 
 int lbm_launch_qkv_linear_prepare(const void* a, const lbm_row_norm* a_norm, const void* w, const float* bias, int M, int K,
                                   const float* q_norm_w, const float* q_norm_b, const float* k_norm_w,
-                                  const float* k_norm_b, float norm_eps, const float* rope_cs, int rope_layout,
+                                  const float* k_norm_b, float norm_eps, float q_scale, const float* rope_cs, int rope_layout,
                                   void* q_out, void* k_out, void* v_out, void* pool, const int32_t* append_rows,
                                   int num_heads, int page_size, hipStream_t stream) {
   if (M == 0) return LBM_OK;
   const int N = 3 * num_heads * 64;
   if (K % kGK != 0) return lbm_fail(LBM_ERR_UNSUPPORTED, "lbm_qkv_linear_prepare: K must be a multiple of 128 (got %d)", K);
+  if (!lbm_offsets_fit(M, N, K))
+    return lbm_fail(LBM_ERR_UNSUPPORTED, "lbm_qkv_linear_prepare: M * K and N * K must stay below 2^31 elements (32-bit byte offsets), got %d x %d x %d", M, N, K);
   LinearArgs p = {};
   p.a = (const unsigned short*)a;
   p.w = (const unsigned short*)w;
@@ -716,6 +731,7 @@ int lbm_launch_qkv_linear_prepare(const void* a, const lbm_row_norm* a_norm, con
   p.pool = (unsigned short*)pool;
   p.append_rows = append_rows;
   p.eps = norm_eps;
+  p.q_scale = q_scale;
   p.num_heads = num_heads; p.page_size = page_size;
   if (int rc = lbm_set_row_norm(p, a_norm, "lbm_qkv_linear_prepare_norm")) return rc;
   const bool lna = a_norm != nullptr;

@@ -222,8 +222,9 @@ __device__ __forceinline__ void lbm_attn_split(const AttnCore& a, const LbmAttnS
   // Each wavefront reads its 64 query rows as whole 128-byte rows (eight lanes per row), parks
   // them in its own LDS patch and picks the fragments up from there; read directly in the
   // fragment layout every load instruction would touch 64 different rows with 16 bytes each.
-  // The softmax scale and log2(e) are folded into Q here (one extra bf16 rounding of q), so
-  // the MFMA result is already the exponent of 2.
+  // The softmax scale and log2(e) are folded into Q here (one extra bf16 rounding of q; none
+  // when the producer already multiplied q by them before its own rounding and the caller
+  // passed sm_scale = 0), so the MFMA result is already the exponent of 2.
   bf16x8 qf[2][4];
   const int q_row0 = qt * kQTile + wave * kQPerWave;
   {
@@ -249,6 +250,7 @@ __device__ __forceinline__ void lbm_attn_split(const AttnCore& a, const LbmAttnS
         f32x8 f = __builtin_convertvector(rawf, f32x8);
 #pragma unroll
         for (int j = 0; j < 8; ++j) f[j] *= a.scale_log2;
+        // (a q that already carries the scale - scale_log2 == 1 - comes back bit for bit: x * 1 is exact)
         qf[qb][ks] = __builtin_convertvector(f, bf16x8);
       }
   }
@@ -1752,7 +1754,7 @@ int lbm_launch_attention(const void* q, const void* pool, void* out, const void*
     f.live_kv_tokens = live_kv_tokens;
     f.num_heads = num_heads;
     f.page_size = page_size;
-    f.scale_log2 = sm_scale * 1.4426950408889634f;
+    f.scale_log2 = sm_scale == 0.f ? 1.0f : sm_scale * 1.4426950408889634f;   // 0: q already carries scale * log2(e)
     f.n_streams = sch.n_streams;
     int wg = 0;
     for (int i = 0; i < LBM_MAX_STREAMS; ++i) {
@@ -1809,7 +1811,7 @@ int lbm_launch_attention(const void* q, const void* pool, void* out, const void*
   a.part_lse = (float*)(a.part_o + (size_t)sch.part_rows * num_heads * head_dim);
   a.num_heads = num_heads;
   a.page_size = page_size;
-  a.scale_log2 = sm_scale * 1.4426950408889634f;
+  a.scale_log2 = sm_scale == 0.f ? 1.0f : sm_scale * 1.4426950408889634f;   // 0: q already carries scale * log2(e)
   a.sch = sch;
   if (sch.total_wgs == 0) return LBM_OK;
   if (sch.small) {

@@ -65,9 +65,17 @@ __device__ __forceinline__ float sum_of_wave(float s) {
 // ROPE 0 none, 1 interleaved pairs (cs4[0..1] = (cos, sin) of this lane's four pairs), 2
 // half-split pairs (cs4[0..3] = (cos, sin) of its eight elements).  w4 / b4: LayerNorm weight
 // and bias of the lane's eight elements.
+// post: a factor the row is multiplied by in fp32 BEFORE the rounding that ends its last
+// operation (the rotary sum, else the LayerNorm, else the plain copy), so that a scaled q row
+// is rounded once; 1.0f leaves every result as it was (x * 1.0f is exact).
 template <int SRC, int ROPE, bool NORM>
 __device__ __forceinline__ void norm_rope(float (&x)[8], const f32x4 (&w4)[2], const f32x4 (&b4)[2],
-                                          const f32x4 (&cs4)[4], int c, float eps) {
+                                          const f32x4 (&cs4)[4], int c, float eps, float post = 1.0f) {
+  const float post_norm = ROPE == 0 ? post : 1.0f;
+  if (!NORM && ROPE == 0) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) x[i] = SRC == 0 ? round_bf16(mul_rn(x[i], post)) : mul_rn(x[i], post);
+  }
   if (NORM) {
     float s = 0.f;
 #pragma unroll
@@ -81,7 +89,7 @@ __device__ __forceinline__ void norm_rope(float (&x)[8], const f32x4 (&w4)[2], c
     const float rstd = __builtin_amdgcn_rsqf(v * (1.0f / 64.0f) + eps);  // torch's LayerNorm uses rsqrt too
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
-      const float y = add_rn(mul_rn(mul_rn(x[i] - mean, rstd), w4[i >> 2][i & 3]), b4[i >> 2][i & 3]);
+      const float y = mul_rn(add_rn(mul_rn(mul_rn(x[i] - mean, rstd), w4[i >> 2][i & 3]), b4[i >> 2][i & 3]), post_norm);
       x[i] = SRC == 0 ? round_bf16(y) : y;
     }
   }
@@ -97,11 +105,11 @@ __device__ __forceinline__ void norm_rope(float (&x)[8], const f32x4 (&w4)[2], c
         if (SRC == 0) {
           co = round_bf16(co);
           si = round_bf16(si);
-          x[i] = round_bf16(sub_rn(round_bf16(mul_rn(x1, co)), round_bf16(mul_rn(x2, si))));
-          x[i + 1] = round_bf16(add_rn(round_bf16(mul_rn(x1, si)), round_bf16(mul_rn(x2, co))));
+          x[i] = round_bf16(mul_rn(sub_rn(round_bf16(mul_rn(x1, co)), round_bf16(mul_rn(x2, si))), post));
+          x[i + 1] = round_bf16(mul_rn(add_rn(round_bf16(mul_rn(x1, si)), round_bf16(mul_rn(x2, co))), post));
         } else {
-          x[i] = sub_rn(mul_rn(x1, co), mul_rn(x2, si));
-          x[i + 1] = add_rn(mul_rn(x1, si), mul_rn(x2, co));
+          x[i] = mul_rn(sub_rn(mul_rn(x1, co), mul_rn(x2, si)), post);
+          x[i + 1] = mul_rn(add_rn(mul_rn(x1, si), mul_rn(x2, co)), post);
         }
       }
     }
@@ -123,10 +131,10 @@ __device__ __forceinline__ void norm_rope(float (&x)[8], const f32x4 (&w4)[2], c
           co = round_bf16(co);
           si = round_bf16(si);
           const float a0 = round_bf16(mul_rn(own, co)), b0 = round_bf16(mul_rn(other, si));
-          x[i] = round_bf16(first ? sub_rn(a0, b0) : add_rn(a0, b0));
+          x[i] = round_bf16(mul_rn(first ? sub_rn(a0, b0) : add_rn(a0, b0), post));
         } else {
           const float a0 = mul_rn(own, co), b0 = mul_rn(other, si);
-          x[i] = first ? sub_rn(a0, b0) : add_rn(a0, b0);
+          x[i] = mul_rn(first ? sub_rn(a0, b0) : add_rn(a0, b0), post);
         }
       }
     }

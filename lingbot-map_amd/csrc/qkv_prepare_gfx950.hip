@@ -80,6 +80,7 @@ struct PrepareArgs {
   void* pool;
   const int32_t* append_rows;
   float eps;
+  float q_scale;           // q is multiplied by this in fp32 before its last rounding (1 = plain q)
   int n_tokens, num_heads, page_size;
 };
 
@@ -159,7 +160,7 @@ __global__ __launch_bounds__(256) void lbm_qkv_prepare_d64_kernel(PrepareArgs a)
 
   // q and k rows: LayerNorm and rotary embedding
 #pragma unroll
-  for (int w = 0; w < 2; ++w) lbm_qkv::norm_rope<SRC, ROPE, NORM>(x[w], w4[w], b4[w], cs4, c, a.eps);
+  for (int w = 0; w < 2; ++w) lbm_qkv::norm_rope<SRC, ROPE, NORM>(x[w], w4[w], b4[w], cs4, c, a.eps, w == 0 ? a.q_scale : 1.0f);
 
   const long long nhd = ((long long)t * H + h) * 64 + c * 8;
   store8<DST>(a.q_out, nhd, x[0]);
@@ -176,7 +177,7 @@ __global__ __launch_bounds__(256) void lbm_qkv_prepare_d64_kernel(PrepareArgs a)
 }  // namespace
 
 int lbm_launch_qkv_prepare(const void* qkv, int src_dtype, const float* q_norm_w, const float* q_norm_b,
-                           const float* k_norm_w, const float* k_norm_b, float norm_eps,
+                           const float* k_norm_w, const float* k_norm_b, float norm_eps, float q_scale,
                            const float* rope_cs, int rope_layout, void* q_out, void* k_out, void* v_out,
                            int dst_dtype, void* pool, const int32_t* append_rows, int n_tokens,
                            int num_heads, int page_size, hipStream_t stream) {
@@ -190,6 +191,7 @@ int lbm_launch_qkv_prepare(const void* qkv, int src_dtype, const float* q_norm_w
   a.pool = pool;
   a.append_rows = append_rows;
   a.eps = norm_eps;
+  a.q_scale = q_scale;
   a.n_tokens = n_tokens; a.num_heads = num_heads; a.page_size = page_size;
   const long long rows = (long long)n_tokens * 3 * num_heads;
   if (rows == 0) return LBM_OK;

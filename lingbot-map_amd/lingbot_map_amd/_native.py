@@ -22,7 +22,7 @@ HDR = {"frame_count": 0, "n_anchor": 1, "win_head": 2, "win_count": 3, "n_free_p
        "n_free_special": 5, "n_special_pages": 6, "special_tokens": 7, "n_memory": 8,
        "n_memory_pages": 9, "error": 10, "plan_kv_tokens": 11, "plan_n_pages": 12}
 HDR_WORDS = 16
-ABI_VERSION = 6
+ABI_VERSION = 7
 
 
 class CacheGeom(C.Structure):
@@ -69,7 +69,7 @@ def _load():
     lib.lbm_kv_append.restype = C.c_int
     lib.lbm_kv_append.argtypes = [vp, vp, i32, vp, i32, vp, i32, i32, i32, i32, vp]
     lib.lbm_qkv_prepare.restype = C.c_int
-    lib.lbm_qkv_prepare.argtypes = [vp, i32, vp, vp, vp, vp, C.c_float, vp, i32, vp, vp, vp, i32, vp, vp, i32, i32, i32, i32, vp]
+    lib.lbm_qkv_prepare.argtypes = [vp, i32, vp, vp, vp, vp, C.c_float, C.c_float, vp, i32, vp, vp, vp, i32, vp, vp, i32, i32, i32, i32, vp]
     lib.lbm_residual_norm.restype = C.c_int
     lib.lbm_residual_norm.argtypes = [vp, vp, i32, vp, vp, vp, C.c_float, vp, vp, i32, i32, vp]
     lib.lbm_linear.restype = C.c_int
@@ -81,9 +81,9 @@ def _load():
     lib.lbm_linear_stats_tiles.restype = i32
     lib.lbm_linear_stats_tiles.argtypes = [i32, i32]
     lib.lbm_qkv_linear_prepare_norm.restype = C.c_int
-    lib.lbm_qkv_linear_prepare_norm.argtypes = [vp, p(RowNorm), vp, vp, i32, i32, vp, vp, vp, vp, C.c_float, vp, i32, vp, vp, vp, vp, vp, i32, i32, i32, vp]
+    lib.lbm_qkv_linear_prepare_norm.argtypes = [vp, p(RowNorm), vp, vp, i32, i32, vp, vp, vp, vp, C.c_float, C.c_float, vp, i32, vp, vp, vp, vp, vp, i32, i32, i32, vp]
     lib.lbm_qkv_linear_prepare.restype = C.c_int
-    lib.lbm_qkv_linear_prepare.argtypes = [vp, vp, vp, i32, i32, vp, vp, vp, vp, C.c_float, vp, i32, vp, vp, vp, vp, vp, i32, i32, i32, vp]
+    lib.lbm_qkv_linear_prepare.argtypes = [vp, vp, vp, i32, i32, vp, vp, vp, vp, C.c_float, C.c_float, vp, i32, vp, vp, vp, vp, vp, i32, i32, i32, vp]
     lib.lbm_attn_workspace_bytes.restype = C.c_size_t
     lib.lbm_attn_workspace_bytes.argtypes = [p(AttnStream), i32, i32, i32]
     lib.lbm_attn_run.restype = C.c_int
@@ -112,6 +112,13 @@ def check(rc: int) -> None:
         if rc == ERR_INVALID:
             raise ValueError(msg)
         raise LbmError(f"lbm error {rc}: {msg}")
+
+
+def q_scale_log2(sm_scale: float) -> float:
+    """The ``q_scale`` to hand the producers so that ``lbm_attn_run`` can be called with
+    ``sm_scale = 0``: the softmax scale times log2(e), as a float32 value."""
+    import struct
+    return struct.unpack("f", struct.pack("f", sm_scale * 1.4426950408889634))[0]
 
 
 def stream_ptr(device) -> C.c_void_p:

@@ -22,6 +22,7 @@ reference's method-by-method sequence is used.
 """
 from __future__ import annotations
 
+import math
 from typing import Callable, Optional
 
 import torch
@@ -194,13 +195,18 @@ _split_workspaces = {}
 
 def _split_workspace(device, nbytes: int) -> Optional[Tensor]:
     """Zero-filled device memory for launches that split K (``lbm_linear_norm``'s workspace; the
-    launches leave its counters at zero), one per device and stream; None when nothing is needed."""
+    launches leave its counters at zero), one per device; None when nothing is needed.  The
+    blocks' launches on one device are serialised (one manager, one stream at a time), so they
+    share it.  It is never allocated or filled under stream capture: a graph would own the
+    memory and replay the fill."""
     if nbytes <= 0:
         return None
-    key = (device, torch.cuda.current_stream(device).cuda_stream)
-    ws = _split_workspaces.get(key)
+    ws = _split_workspaces.get(device)
     if ws is None or ws.numel() < nbytes:
-        ws = _split_workspaces[key] = torch.zeros(nbytes, dtype=torch.uint8, device=device)
+        if torch.cuda.is_current_stream_capturing():
+            raise RuntimeError("the K-split workspace must exist before a frame is captured: run the frame once "
+                               "eagerly first (GraphedFrame does)")
+        ws = _split_workspaces[device] = torch.zeros(nbytes, dtype=torch.uint8, device=device)
     return ws
 
 
@@ -502,16 +508,18 @@ class HipPagedAttention(nn.Module):
         dt = N.DTYPE_BF16 if x.dtype == torch.bfloat16 else N.DTYPE_F32
         eps = float(self.q_norm.eps) if has_norm else 1e-5
         stream = N.stream_ptr(x.device)
+        # q comes out multiplied by the softmax scale and log2(e) (rounded once), see dense_attention
+        q_scale = N.q_scale_log2(1.0 / math.sqrt(D))
         if proj is not None:
             N.check(N.lib.lbm_qkv_linear_prepare_norm(
                 p(proj[0]), proj[3] if len(proj) > 3 else None, p(proj[1]), p(proj[2]), B * n, proj[0].shape[1],
                 p(qk_norm[0]), p(qk_norm[1]), p(qk_norm[2]), p(qk_norm[3]),
-                eps, p(table), layout, p(q), p(k), p(v), None, None, H, D, 16, stream))
+                eps, q_scale, p(table), layout, p(q), p(k), p(v), None, None, H, D, 16, stream))
         else:
             N.check(N.lib.lbm_qkv_prepare(
-                p(qkv), dt, p(qk_norm[0]), p(qk_norm[1]), p(qk_norm[2]), p(qk_norm[3]), eps, p(table), layout, p(q), p(k), p(v), dt,
+                p(qkv), dt, p(qk_norm[0]), p(qk_norm[1]), p(qk_norm[2]), p(qk_norm[3]), eps, q_scale, p(table), layout, p(q), p(k), p(v), dt,
                 None, None, B * n, H, D, 16, stream))
-        return dense_attention(q, k, v, num_streams=B).reshape(B, n, H * D)
+        return dense_attention(q, k, v, num_streams=B, q_prescaled=True).reshape(B, n, H * D)
 
     def forward(self, x: Tensor, pos=None, num_patches=None, num_special=None, num_frames=None,
                 enable_3d_rope=False, kv_cache=None, global_idx=0, num_frame_per_block=1,

@@ -20,12 +20,13 @@ _plans: Dict[tuple, tuple] = {}          # (rows, streams, H, D, device) -> (row
 _workspace: Dict[object, Tensor] = {}
 
 
-def dense_attention(q: Tensor, k: Tensor, v: Tensor, num_streams: int = 1) -> Tensor:
+def dense_attention(q: Tensor, k: Tensor, v: Tensor, num_streams: int = 1, q_prescaled: bool = False) -> Tensor:
     """softmax(q k^T / sqrt(D)) v for ``num_streams`` independent token groups.
 
     ``q``, ``k``, ``v``: ``[num_streams * n, H, D]`` contiguous, bf16 or fp32, on the GPU; group
     ``s`` is rows ``s * n .. (s + 1) * n - 1`` and attends to itself only.  Returns the same
-    shape and dtype.  Raises on anything the HIP kernels do not cover (there is no fallback)."""
+    shape and dtype.  ``q_prescaled``: q already carries 1 / sqrt(D) and log2(e) (a producer run
+    with ``q_scale = q_scale_log2(1 / sqrt(D))``).  Raises on anything the HIP kernels do not cover (there is no fallback)."""
     assert q.is_cuda and q.dim() == 3 and q.shape == k.shape == v.shape, "q, k, v: [tokens, H, D] on the GPU"
     assert q.dtype == k.dtype == v.dtype and q.dtype in (torch.bfloat16, torch.float32), "bf16 or fp32"
     rows, H, D = q.shape
@@ -49,6 +50,6 @@ def dense_attention(q: Tensor, k: Tensor, v: Tensor, num_streams: int = 1) -> Te
     p = lambda t: C.c_void_p(t.data_ptr())
     N.check(N.lib.lbm_attn_run(
         p(q), p(k), p(out), p(k), p(v), p(kv_rows), streams, num_streams, H, D, 16,
-        N.DTYPE_BF16 if q.dtype == torch.bfloat16 else N.DTYPE_F32, 1.0 / math.sqrt(D),
+        N.DTYPE_BF16 if q.dtype == torch.bfloat16 else N.DTYPE_F32, 0.0 if q_prescaled else 1.0 / math.sqrt(D),
         p(ws), ws.numel(), N.stream_ptr(q.device)))
     return out

@@ -504,20 +504,24 @@ class HipPagedKVCacheManager:
         vp = lambda t: None if t is None else C.c_void_p(t.data_ptr())
         rope_ptr = vp(rope_cs)
         append_ptr = vp(self._append_rows[ts]) if any(keyframe) else None
+        # q leaves the producer multiplied by the softmax scale and log2(e) - one rounding for the
+        # row instead of the producer's and then the attention kernel's - and the attention call
+        # below is told so (sm_scale = 0)
+        q_scale = N.q_scale_log2(1.0 / math.sqrt(D))
         if proj is None:
             N.check(N.lib.lbm_qkv_prepare(
-                vp(qkv), dt(qkv.dtype), norm_ptr[0], norm_ptr[1], norm_ptr[2], norm_ptr[3], float(norm_eps),
+                vp(qkv), dt(qkv.dtype), norm_ptr[0], norm_ptr[1], norm_ptr[2], norm_ptr[3], float(norm_eps), q_scale,
                 rope_ptr, N.ROPE_INTERLEAVED, vp(q), vp(k), vp(v), dt(self.dtype),
                 vp(self.kv_caches[block_idx]), append_ptr, rows, H, D, self.page_size, self._stream_handle()))
         else:
             N.check(N.lib.lbm_qkv_linear_prepare_norm(
                 vp(px), row_norm, vp(pw), vp(pb), rows, px.shape[1], norm_ptr[0], norm_ptr[1], norm_ptr[2], norm_ptr[3],
-                float(norm_eps), rope_ptr, N.ROPE_INTERLEAVED, vp(q), vp(k), vp(v),
+                float(norm_eps), q_scale, rope_ptr, N.ROPE_INTERLEAVED, vp(q), vp(k), vp(v),
                 vp(self.kv_caches[block_idx]), append_ptr, H, D, self.page_size, self._stream_handle()))
         if any(keyframe):
             self.frame_count[block_idx] += 1
             self._n_appends[block_idx] += 1
-        return self._attend_planned(block_idx, q, k, v)
+        return self._attend_planned(block_idx, q, k, v, q_prescaled=True)
 
     def _as_f32(self, t: Tensor, n: int) -> Tensor:
         assert t.numel() == n, f"expected {n} LayerNorm parameters, got {tuple(t.shape)}"
@@ -621,7 +625,9 @@ class HipPagedKVCacheManager:
                                f"{self._n_appends[0]}: with shared page tables every block takes the frame block 0 took")
         return ts, keyframe, tail
 
-    def _attend_planned(self, block_idx: int, q: Tensor, self_k: Optional[Tensor], self_v: Optional[Tensor]) -> Tensor:
+    def _attend_planned(self, block_idx: int, q: Tensor, self_k: Optional[Tensor], self_v: Optional[Tensor],
+                        q_prescaled: bool = False) -> Tensor:
+        """``q_prescaled``: q already carries 1 / sqrt(D) and log2(e) (``step_qkv``'s producer)."""
         ts = self._set(block_idx)
         rows = self.num_streams * self.tokens_per_frame
         assert q.dim() == 3 and tuple(q.shape) == (rows, self.num_heads, self.head_dim), (
@@ -647,7 +653,8 @@ class HipPagedKVCacheManager:
         if need > self.workspace_buffer.numel():
             self.workspace_buffer = torch.empty(int(need * 1.25) + 256, dtype=torch.uint8, device=self.device)
         common = (streams, n, self.num_heads, self.head_dim, self.page_size,
-                  N.DTYPE_BF16 if self.dtype == torch.bfloat16 else N.DTYPE_F32, 1.0 / math.sqrt(self.head_dim),
+                  N.DTYPE_BF16 if self.dtype == torch.bfloat16 else N.DTYPE_F32,
+                  0.0 if q_prescaled else 1.0 / math.sqrt(self.head_dim),
                   C.c_void_p(self.workspace_buffer.data_ptr()), self.workspace_buffer.numel(), self._stream_handle())
         tensors = (C.c_void_p(qc.data_ptr()), C.c_void_p(self.kv_caches[block_idx].data_ptr()), C.c_void_p(out.data_ptr()),
                    C.c_void_p(self_k.data_ptr()) if has_tail else None, C.c_void_p(self_v.data_ptr()) if has_tail else None,

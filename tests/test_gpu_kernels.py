@@ -359,15 +359,72 @@ def test_attention_random_shapes(seed):
         assert err_max <= BF16_MAX_ABS and err_mean <= BF16_MEAN_ABS, (what, err_max, err_mean)
 
 
-@pytest.mark.xfail(strict=False, reason=(
-    "keys three times as long as any benchmark configuration draws them (N(0, 9) against N(0, 1)): the softmax "
-    "is then dominated by a handful of tokens and the one rounding the kernel adds to the reference's arithmetic - "
-    "q * scale * log2(e) is rounded to bf16 before the QK^T product - shows up undamped; the worst element of "
-    "some draws lands between 2e-2 and 4e-2.  The mean-abs bar holds; see test_attention_peaked_scores_mean_bar."))
 @pytest.mark.parametrize("seed", range(3))
 def test_attention_peaked_scores_max_bar(seed):
+    """Keys three times as long as any benchmark configuration draws them (N(0, 9) against N(0, 1)):
+    the softmax is then dominated by a handful of tokens and the one rounding the bare entry point
+    adds to the reference's arithmetic - q * scale * log2(e) is rounded to bf16 before the QK^T
+    product - shows up undamped.  The bar holds on these draws with little room."""
     for what, err_max, _ in _random_shape_cases(seed, [3.0], n_cases=4):
         assert err_max <= BF16_MAX_ABS, (what, err_max)
+
+
+@pytest.mark.parametrize("n_tok", [1500, 4500])
+@pytest.mark.parametrize("seed", range(3))
+def test_attention_peaked_scores_through_the_producer(seed, n_tok):
+    """The same peaked keys on the path the blocks take: the producer multiplies q by
+    scale * log2(e) before its own rounding (q_scale) and the attention call is told so
+    (sm_scale = 0), so the q row is rounded to bf16 once, as the reference's q is - but it is a
+    different rounding of the same fp32 row than the reference's (scaled before instead of after).
+    What that buys is measured against float64 attention on the UNROUNDED q (k, v as cached): the
+    fused path must be as close to it as the reference's own path (oracle producer with the
+    reference's bf16 rounding sequence, then its SDPA) is, and closer than the bare entry point
+    fed with the reference's rounded q (which rounds q a second time).  Against the reference
+    itself the two roundings add up: the mean-abs bar holds, the worst element may be two bf16
+    steps of an O(1) output away (4e-2).  1,500 tokens run on the short-KV kernel, 4,500 on the
+    split-KV kernel."""
+    from oracle.prepare_qkv import prepare_qkv
+    from oracle.sdpa_cache import sdpa_nhd
+    N = _native()
+    dev = torch.device("cuda:0")
+    H, D = 2, 64
+    g = torch.Generator().manual_seed(100 + seed)
+    qkv = torch.randn(n_tok, 3, H, D, generator=g)
+    qkv[:, 1] *= 3.0
+    qkv = qkv.reshape(n_tok, 3 * H * D).to(torch.bfloat16)
+    ang = torch.rand(1, 1, n_tok, D // 2, generator=g) * 2 * math.pi
+    freqs = torch.polar(torch.ones_like(ang), ang)
+    rq, rk, rv = prepare_qkv(qkv, H, D, None, None, freqs)
+    ref = sdpa_nhd(rq, rk, rv).float()
+    q_unrounded = prepare_qkv(qkv.float(), H, D, None, None, freqs)[0]
+    exact = sdpa_nhd(q_unrounded.double(), rk.double(), rv.double(), compute_dtype=torch.float64).float()
+    cs = torch.view_as_real(freqs).reshape(n_tok, D // 2, 2).float().contiguous().to(dev)
+    x = qkv.to(dev)
+    rows = (-1 - torch.arange(n_tok, dtype=torch.int32)).to(dev)
+    arr = (N.AttnStream * 1)(N.AttnStream(0, n_tok, 0, n_tok))
+    ws = torch.empty(max(int(N.lib.lbm_attn_workspace_bytes(arr, 1, H, D)), 16), dtype=torch.uint8, device=dev)
+
+    def run(q_scale, sm_scale):
+        q, k, v = (torch.empty(n_tok, H, D, dtype=torch.bfloat16, device=dev) for _ in range(3))
+        N.check(N.lib.lbm_qkv_prepare(ptr(x), N.DTYPE_BF16, None, None, None, None, 1e-5, q_scale, ptr(cs), N.ROPE_INTERLEAVED,
+                                      ptr(q), ptr(k), ptr(v), N.DTYPE_BF16, None, None, n_tok, H, D, 16, None))
+        out = torch.full_like(q, float("nan"))
+        N.check(N.lib.lbm_attn_run(ptr(q), ptr(k), ptr(out), ptr(k), ptr(v), ptr(rows), arr, 1, H, D, 16, N.DTYPE_BF16,
+                                   sm_scale, ptr(ws), ws.numel(), None))
+        torch.cuda.synchronize()
+        assert torch.equal(k.cpu(), rk) and torch.equal(v.cpu(), rv)
+        return out.float().cpu()
+
+    fused = run(N.q_scale_log2(1.0 / math.sqrt(D)), 0.0)
+    bare = run(1.0, 1.0 / math.sqrt(D))
+    mean = lambda a, b: (a - b).abs().mean().item()
+    print(f"peaked, seed {seed}, {n_tok} tokens: mean-abs from float64 on the unrounded q: reference {mean(ref, exact):.5f} "
+          f"fused {mean(fused, exact):.5f} bare {mean(bare, exact):.5f}; from the reference: fused {mean(fused, ref):.5f} "
+          f"(max {(fused - ref).abs().max().item():.4f}) bare {mean(bare, ref):.5f} (max {(bare - ref).abs().max().item():.4f})")
+    assert mean(fused, exact) <= 1.05 * mean(ref, exact)
+    assert mean(fused, exact) < mean(bare, exact)
+    assert mean(fused, ref) <= BF16_MEAN_ABS and (fused - ref).abs().max().item() <= 2 * BF16_MAX_ABS
+    assert mean(bare, ref) <= BF16_MEAN_ABS and (bare - ref).abs().max().item() <= BF16_MAX_ABS
 
 
 @pytest.mark.parametrize("seed", range(3))

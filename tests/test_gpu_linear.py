@@ -138,7 +138,7 @@ def test_linear_rows_past_m_are_not_written_and_arguments_are_checked():
     # no rows: accepted, nothing written
     o.fill_(3.0)
     N.check(N.lib.lbm_linear(ptr(ad), ptr(wd), None, None, None, ptr(o), 0, 128, 128, N.LINEAR_BIAS, None))
-    N.check(N.lib.lbm_qkv_linear_prepare(ptr(ad), ptr(wd), None, 0, 128, None, None, None, None, 1e-5, None, 0, ptr(o), None, None,
+    N.check(N.lib.lbm_qkv_linear_prepare(ptr(ad), ptr(wd), None, 0, 128, None, None, None, None, 1e-5, 1.0, None, 0, ptr(o), None, None,
                                          None, None, 2, 64, 16, None))
     torch.cuda.synchronize()
     assert bool((o == 3.0).all())
@@ -206,10 +206,10 @@ def test_qkv_projection_with_the_producer_as_its_epilogue(M, H, K, norm, rope):
         q0, k0, v0, pool0 = outputs()
         qkv = torch.empty(M, 3 * H * D, dtype=torch.bfloat16, device=dev)
         N.check(N.lib.lbm_linear(ptr(a), ptr(w), ptr(bias), None, None, ptr(qkv), M, 3 * H * D, K, N.LINEAR_BIAS, None))
-        N.check(N.lib.lbm_qkv_prepare(ptr(qkv), N.DTYPE_BF16, *[ptr(t) for t in ln], 1e-5, ptr(cs), layout, ptr(q0), ptr(k0), ptr(v0),
+        N.check(N.lib.lbm_qkv_prepare(ptr(qkv), N.DTYPE_BF16, *[ptr(t) for t in ln], 1e-5, 1.0, ptr(cs), layout, ptr(q0), ptr(k0), ptr(v0),
                                       N.DTYPE_BF16, ptr(pool0), ptr(rows) if with_pool else None, M, H, D, S, None))
         q1, k1, v1, pool1 = outputs()
-        N.check(N.lib.lbm_qkv_linear_prepare(ptr(a), ptr(w), ptr(bias), M, K, *[ptr(t) for t in ln], 1e-5, ptr(cs), layout,
+        N.check(N.lib.lbm_qkv_linear_prepare(ptr(a), ptr(w), ptr(bias), M, K, *[ptr(t) for t in ln], 1e-5, 1.0, ptr(cs), layout,
                                              ptr(q1), ptr(k1), ptr(v1), ptr(pool1), ptr(rows) if with_pool else None, H, D, S, None))
         torch.cuda.synchronize()
         assert torch.isfinite(q1.float()).all() and torch.equal(q0, q1)
@@ -220,9 +220,9 @@ def test_qkv_projection_with_the_producer_as_its_epilogue(M, H, K, norm, rope):
     # argument checks
     bad = lambda *args: N.lib.lbm_qkv_linear_prepare(*args) != N.OK
     q1 = torch.empty(M, H, D, dtype=torch.bfloat16, device=dev)
-    assert bad(ptr(a), ptr(w), None, M, K, None, None, None, None, 1e-5, None, 0, ptr(q1), None, None, None, None, H, 128, S, None)   # head_dim
-    assert bad(ptr(a), ptr(w), None, M, K, ptr(bias), None, None, None, 1e-5, None, 0, ptr(q1), None, None, None, None, H, D, S, None)  # one norm parameter
-    assert bad(ptr(a), ptr(w), None, M, K, None, None, None, None, 1e-5, None, 0, ptr(q1), None, None, None, ptr(rows), H, D, S, None)  # rows without pool
+    assert bad(ptr(a), ptr(w), None, M, K, None, None, None, None, 1e-5, 1.0, None, 0, ptr(q1), None, None, None, None, H, 128, S, None)   # head_dim
+    assert bad(ptr(a), ptr(w), None, M, K, ptr(bias), None, None, None, 1e-5, 1.0, None, 0, ptr(q1), None, None, None, None, H, D, S, None)  # one norm parameter
+    assert bad(ptr(a), ptr(w), None, M, K, None, None, None, None, 1e-5, 1.0, None, 0, ptr(q1), None, None, None, ptr(rows), H, D, S, None)  # rows without pool
 
 
 def _row_norm(N, stats, colsum, tiles, eps=1e-5):
@@ -340,11 +340,11 @@ def test_layernorm_folded_into_the_qkv_projection_and_producer():
         if fold:
             xd, wd, cd, bd, stats = x.to(dev), wf.to(dev), colsum.to(dev), bf.to(dev), _stats_of(x, tiles).to(dev)
             ln = _row_norm(N, stats, cd, tiles)
-            N.check(N.lib.lbm_qkv_linear_prepare_norm(ptr(xd), ln, ptr(wd), ptr(bd), M, K, *[ptr(t) for t in qk], 1e-5, ptr(cs),
+            N.check(N.lib.lbm_qkv_linear_prepare_norm(ptr(xd), ln, ptr(wd), ptr(bd), M, K, *[ptr(t) for t in qk], 1e-5, 1.0, ptr(cs),
                                                       N.ROPE_INTERLEAVED, ptr(q), ptr(k), ptr(v), None, None, H, D, S, None))
         else:
             wd, bd = w.to(dev), bias.to(dev)
-            N.check(N.lib.lbm_qkv_linear_prepare(ptr(normed), ptr(wd), ptr(bd), M, K, *[ptr(t) for t in qk], 1e-5, ptr(cs),
+            N.check(N.lib.lbm_qkv_linear_prepare(ptr(normed), ptr(wd), ptr(bd), M, K, *[ptr(t) for t in qk], 1e-5, 1.0, ptr(cs),
                                                  N.ROPE_INTERLEAVED, ptr(q), ptr(k), ptr(v), None, None, H, D, S, None))
         torch.cuda.synchronize()
         outs.append([t.float().cpu() for t in (q, k, v)])

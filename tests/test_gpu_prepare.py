@@ -35,7 +35,7 @@ def _inputs(n, H, D, dtype, seed):
 
 
 def run_prepare(qkv, H, D, qn, kn, freqs, dst_dtype, pool=None, rows=None, page_size=16, want_kv=True, eps=1e-5,
-                table=None):
+                table=None, q_scale=1.0):
     """freqs: complex table of the interleaved embedding; table: [n, D, 2] (cos, sin) of the half-split one."""
     N = _native()
     dev = torch.device("cuda:0")
@@ -51,7 +51,7 @@ def run_prepare(qkv, H, D, qn, kn, freqs, dst_dtype, pool=None, rows=None, page_
     k = torch.full_like(q, float("nan")) if want_kv else None
     v = torch.full_like(q, float("nan")) if want_kv else None
     x = qkv.to(dev)
-    N.check(N.lib.lbm_qkv_prepare(ptr(x), dt(qkv.dtype), *( [ptr(t) for t in keep] if keep else [None] * 4), eps, ptr(cs), layout,
+    N.check(N.lib.lbm_qkv_prepare(ptr(x), dt(qkv.dtype), *( [ptr(t) for t in keep] if keep else [None] * 4), eps, q_scale, ptr(cs), layout,
                                   ptr(q), ptr(k), ptr(v), dt(dst_dtype), ptr(pool), ptr(rows), n, H, D, page_size, None))
     torch.cuda.synchronize()
     return q, k, v
@@ -94,6 +94,48 @@ def test_prepare_without_norm_is_bit_exact_in_bf16():
     assert torch.equal(q.cpu(), rq) and torch.equal(k.cpu(), rk) and torch.equal(v.cpu(), rv)
 
 
+def test_prepare_q_scale_rounds_the_scaled_row_once():
+    """``q_scale``: q is multiplied in fp32 before its last rounding, k and v are left alone.  A power
+    of two commutes with the rounding (bit-equal to the plain q times it); for sm_scale * log2(e)
+    the bf16 q must be the nearest bf16 to the scaled fp32 row, which the fp32 oracle provides up
+    to the rounding of the operations before the last one (one ulp)."""
+    from oracle.prepare_qkv import prepare_qkv
+    N = _native()
+    n, H, D = 257, 4, 64
+    for qn_on, rope_on in ((True, True), (False, True), (True, False), (False, False)):
+        qkv, qn, kn, freqs = _inputs(n, H, D, torch.bfloat16, seed=21)
+        qn, kn, freqs = (qn if qn_on else None), (kn if qn_on else None), (freqs if rope_on else None)
+        q1, k1, v1 = run_prepare(qkv, H, D, qn, kn, freqs, torch.bfloat16)
+        qh, kh, vh = run_prepare(qkv, H, D, qn, kn, freqs, torch.bfloat16, q_scale=0.25)
+        assert torch.equal(qh.float(), q1.float() * 0.25) and torch.equal(kh, k1) and torch.equal(vh, v1)
+        c = N.q_scale_log2(1.0 / math.sqrt(D))
+        qc, kc, vc = run_prepare(qkv, H, D, qn, kn, freqs, torch.bfloat16, q_scale=c)
+        assert torch.equal(kc, k1) and torch.equal(vc, v1)
+        # against the reference's rounded q times c: half a bf16 step of either value apart at most
+        ref = q1.float().cpu() * c
+        got = qc.float().cpu()
+        step = lambda t: torch.exp2(torch.floor(torch.log2(t.abs().clamp_min(1e-30))) - 7)
+        assert ((got - ref).abs() <= 0.505 * (step(got) + c * step(q1.float().cpu()))).all()
+        # and nearer to the unrounded row (fp32 oracle) than the twice-rounded c * q is, on average
+        f32 = lambda t: None if t is None else tuple(x.float() for x in t)
+        exact = prepare_qkv(qkv.float(), H, D, f32(qn), f32(kn), freqs)[0] * c
+        twice = (q1.float().cpu() * c).to(torch.bfloat16).float()
+        if qn_on or rope_on:
+            assert (got - exact).abs().mean() < (twice - exact).abs().mean()
+    # fp32 activations and cache: a plain multiply
+    qkv, qn, kn, freqs = _inputs(33, 2, D, torch.float32, seed=22)
+    q1, _, _ = run_prepare(qkv, 2, D, qn, kn, freqs, torch.float32)
+    qc, _, _ = run_prepare(qkv, 2, D, qn, kn, freqs, torch.float32, q_scale=c)
+    assert torch.allclose(qc, q1 * c, rtol=2e-7, atol=0)
+    # refused: zero or negative
+    dev = torch.device("cuda:0")
+    x = torch.zeros(4, 3 * 2 * 64, dtype=torch.bfloat16, device=dev)
+    q = torch.zeros(4, 2, 64, dtype=torch.bfloat16, device=dev)
+    for bad in (0.0, -1.0, float("nan")):
+        assert N.lib.lbm_qkv_prepare(ptr(x), 0, None, None, None, None, 1e-5, bad, None, 0, ptr(q), None, None, 0, None, None,
+                                     4, 2, 64, 16, None) == N.ERR_INVALID
+
+
 def test_prepare_writes_the_pool_rows_and_respects_the_gate():
     from oracle.prepare_qkv import prepare_qkv
     dev = torch.device("cuda:0")
@@ -126,12 +168,12 @@ def test_prepare_argument_checks():
     dev = torch.device("cuda:0")
     x = torch.zeros(4, 3 * 2 * 64, dtype=torch.bfloat16, device=dev)
     q = torch.zeros(4, 2, 64, dtype=torch.bfloat16, device=dev)
-    call = lambda **kw: N.lib.lbm_qkv_prepare(ptr(x), 0, None, None, None, None, 1e-5, None, 0, ptr(q), None, None, 0, None, None,
+    call = lambda **kw: N.lib.lbm_qkv_prepare(ptr(x), 0, None, None, None, None, 1e-5, 1.0, None, 0, ptr(q), None, None, 0, None, None,
                                               4, 2, kw.get("D", 64), 16, None)
     assert call() == N.OK
     assert call(D=128) != N.OK and b"head_dim 64" in N.lib.lbm_last_error()
     w = torch.ones(64, device=dev)
-    rc = N.lib.lbm_qkv_prepare(ptr(x), 0, ptr(w), None, None, None, 1e-5, None, 0, ptr(q), None, None, 0, None, None, 4, 2, 64, 16, None)
+    rc = N.lib.lbm_qkv_prepare(ptr(x), 0, ptr(w), None, None, None, 1e-5, 1.0, None, 0, ptr(q), None, None, 0, None, None, 4, 2, 64, 16, None)
     assert rc != N.OK
     torch.cuda.synchronize()
 
