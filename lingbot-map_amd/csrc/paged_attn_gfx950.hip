@@ -183,7 +183,8 @@ __device__ __forceinline__ void lbm_attn_split(const AttnCore& a, const LbmAttnS
   // c of V row r at c ^ 4 ((r >> 1) & 1) (the 8-byte transposed reads touch four rows x 64
   // bytes; rows r+2 and r+3 move to the other half).  The compiler does not count these loads
   // (its own waits only get stricter by that); LBM_DMA_LANDED waits for them before the
-  // barrier that publishes a tile.  Nothing else in this kernel uses M0.
+  // barrier that publishes a tile.  M0 is declared clobbered, so the compiler keeps nothing of
+  // its own in it across a load.
   // Rows past the last token re-read the last token (finite data; the softmax masks them).
   const int ld_r = tid >> 3;
   const int ld_ck = ((lane & 7) ^ ((ld_r >> 1) & 7)) * 8, ld_cv = ((lane & 7) ^ (((ld_r >> 1) & 1) * 4)) * 8;
@@ -205,7 +206,7 @@ __device__ __forceinline__ void lbm_attn_split(const AttnCore& a, const LbmAttnS
     asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off"
                  :
                  : "v"(src), "s"(__builtin_amdgcn_readfirstlane(m0v))
-                 : "memory");
+                 : "memory", "m0");
   };
 #define LBM_DMA_LANDED() __builtin_amdgcn_s_waitcnt(0x0F70)   /* vmcnt(0); expcnt and lgkmcnt untouched */
 
@@ -408,7 +409,7 @@ __device__ __forceinline__ void lbm_attn_split(const AttnCore& a, const LbmAttnS
 //             k-step 1 = k-step ks_pv of the V tile in stage st_pv
 //   next      scores of the next half: K tile in stage st_qk, half h_qk, nv_qk valid tokens left
 //   st_vn, ks_vn   V tile / k-step whose V^T goes to vnext for the following half-step
-#define LBM_SLICE(j, cur, pd, prev, next, st_pv, ks_pv, st_qk, h_qk, st_vn, ks_vn)                 \
+#define LBM_SLICE(j, cur, pd, prev, next, st_pv, ks_pv, st_qk, h_qk, st_vn, ks_vn, hook)           \
   {                                                                                              \
     /* ---- the MFMA of this slice */                                                            \
     if ((j) < 4)                                                                                 \
@@ -450,11 +451,12 @@ __device__ __forceinline__ void lbm_attn_split(const AttnCore& a, const LbmAttnS
           bf16x8, *(const u32x4*)&lds_k[st_qk][((h_qk) * 32 + n32) * kRingRow + (((((j) - 10) >> 1) * 2 + g) ^ ((n32 >> 1) & 7)) * 8]); \
     if ((j) == 17) vnext[0] = v_frag(st_vn, ks_vn, 0);                                           \
     if ((j) == 18) vnext[1] = v_frag(st_vn, ks_vn, 1);                                           \
+    hook(j)                                                                                      \
     __builtin_amdgcn_sched_barrier(0);                                                           \
   }
 #define LBM_S4(j, ...) LBM_SLICE(j, __VA_ARGS__) LBM_SLICE(j + 1, __VA_ARGS__) LBM_SLICE(j + 2, __VA_ARGS__) LBM_SLICE(j + 3, __VA_ARGS__)
 // `hot` tells whether a numerator of `cur` reached 2 (bf16 exponent field >= 128)
-#define LBM_HALF_STEP(cur, pd, prev, next, st_pv, ks_pv, st_qk, h_qk, nv_qk, st_vn, ks_vn, hot)   \
+#define LBM_HALF_STEP(cur, pd, prev, next, st_pv, ks_pv, st_qk, h_qk, nv_qk, st_vn, ks_vn, hot, hook) \
   {                                                                                              \
     u32x4 kb = kaug_bits;                                                                        \
     kb[1] = (g == 0 && (h_qk) * 32 + n32 >= (nv_qk)) ? 0xBF80u : 0u;                             \
@@ -463,13 +465,13 @@ __device__ __forceinline__ void lbm_attn_split(const AttnCore& a, const LbmAttnS
     float e[32];                                                                                 \
     unsigned chk;                                                                                \
     __builtin_amdgcn_sched_barrier(0);                                                           \
-    LBM_S4(0, cur, pd, prev, next, st_pv, ks_pv, st_qk, h_qk, st_vn, ks_vn)                       \
-    LBM_S4(4, cur, pd, prev, next, st_pv, ks_pv, st_qk, h_qk, st_vn, ks_vn)                       \
-    LBM_S4(8, cur, pd, prev, next, st_pv, ks_pv, st_qk, h_qk, st_vn, ks_vn)                       \
-    LBM_S4(12, cur, pd, prev, next, st_pv, ks_pv, st_qk, h_qk, st_vn, ks_vn)                      \
-    LBM_S4(16, cur, pd, prev, next, st_pv, ks_pv, st_qk, h_qk, st_vn, ks_vn)                      \
-    LBM_SLICE(20, cur, pd, prev, next, st_pv, ks_pv, st_qk, h_qk, st_vn, ks_vn)                   \
-    LBM_SLICE(21, cur, pd, prev, next, st_pv, ks_pv, st_qk, h_qk, st_vn, ks_vn)                   \
+    LBM_S4(0, cur, pd, prev, next, st_pv, ks_pv, st_qk, h_qk, st_vn, ks_vn, hook)                       \
+    LBM_S4(4, cur, pd, prev, next, st_pv, ks_pv, st_qk, h_qk, st_vn, ks_vn, hook)                       \
+    LBM_S4(8, cur, pd, prev, next, st_pv, ks_pv, st_qk, h_qk, st_vn, ks_vn, hook)                       \
+    LBM_S4(12, cur, pd, prev, next, st_pv, ks_pv, st_qk, h_qk, st_vn, ks_vn, hook)                      \
+    LBM_S4(16, cur, pd, prev, next, st_pv, ks_pv, st_qk, h_qk, st_vn, ks_vn, hook)                      \
+    LBM_SLICE(20, cur, pd, prev, next, st_pv, ks_pv, st_qk, h_qk, st_vn, ks_vn, hook)                   \
+    LBM_SLICE(21, cur, pd, prev, next, st_pv, ks_pv, st_qk, h_qk, st_vn, ks_vn, hook)                   \
     /* the numerators exist before the test that follows, not only on its common branch */       \
     asm volatile("" : "+v"(pd[0][0]), "+v"(pd[0][1]), "+v"(pd[1][0]), "+v"(pd[1][1]));             \
     hot = (chk & 0x40004000u) != 0u;                                                             \
@@ -477,7 +479,7 @@ __device__ __forceinline__ void lbm_attn_split(const AttnCore& a, const LbmAttnS
 // The same half-step without a softmax reference (scores go to exp2 as they come out of the
 // QK^T product) and without the test: 20 slices, QK^T in slices 12-19 with its first k-step
 // starting from zero.  Only for half-steps whose 32 KV rows are all valid tokens.
-#define LBM_FSLICE(j, cur, pd, prev, next, st_pv, ks_pv, st_qk, h_qk, st_vn, ks_vn)                \
+#define LBM_FSLICE(j, cur, pd, prev, next, st_pv, ks_pv, st_qk, h_qk, st_vn, ks_vn, hook)          \
   {                                                                                              \
     if ((j) < 4)                                                                                 \
       o[(j) & 1][(j) >> 1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(                            \
@@ -509,19 +511,20 @@ __device__ __forceinline__ void lbm_attn_split(const AttnCore& a, const LbmAttnS
           bf16x8, *(const u32x4*)&lds_k[st_qk][((h_qk) * 32 + n32) * kRingRow + (((((j) - 8) >> 1) * 2 + g) ^ ((n32 >> 1) & 7)) * 8]); \
     if ((j) == 16) vnext[0] = v_frag(st_vn, ks_vn, 0);                                           \
     if ((j) == 17) vnext[1] = v_frag(st_vn, ks_vn, 1);                                           \
+    hook(j)                                                                                      \
     __builtin_amdgcn_sched_barrier(0);                                                           \
   }
 #define LBM_F4(j, ...) LBM_FSLICE(j, __VA_ARGS__) LBM_FSLICE(j + 1, __VA_ARGS__) LBM_FSLICE(j + 2, __VA_ARGS__) LBM_FSLICE(j + 3, __VA_ARGS__)
-#define LBM_FAST_HALF_STEP(cur, pd, prev, next, st_pv, ks_pv, st_qk, h_qk, st_vn, ks_vn)           \
+#define LBM_FAST_HALF_STEP(cur, pd, prev, next, st_pv, ks_pv, st_qk, h_qk, st_vn, ks_vn, hook)     \
   {                                                                                              \
     bf16x8 va[2], ka[4];                                                                         \
     float e[32];                                                                                 \
     __builtin_amdgcn_sched_barrier(0);                                                           \
-    LBM_F4(0, cur, pd, prev, next, st_pv, ks_pv, st_qk, h_qk, st_vn, ks_vn)                       \
-    LBM_F4(4, cur, pd, prev, next, st_pv, ks_pv, st_qk, h_qk, st_vn, ks_vn)                       \
-    LBM_F4(8, cur, pd, prev, next, st_pv, ks_pv, st_qk, h_qk, st_vn, ks_vn)                       \
-    LBM_F4(12, cur, pd, prev, next, st_pv, ks_pv, st_qk, h_qk, st_vn, ks_vn)                      \
-    LBM_F4(16, cur, pd, prev, next, st_pv, ks_pv, st_qk, h_qk, st_vn, ks_vn)                      \
+    LBM_F4(0, cur, pd, prev, next, st_pv, ks_pv, st_qk, h_qk, st_vn, ks_vn, hook)                       \
+    LBM_F4(4, cur, pd, prev, next, st_pv, ks_pv, st_qk, h_qk, st_vn, ks_vn, hook)                       \
+    LBM_F4(8, cur, pd, prev, next, st_pv, ks_pv, st_qk, h_qk, st_vn, ks_vn, hook)                       \
+    LBM_F4(12, cur, pd, prev, next, st_pv, ks_pv, st_qk, h_qk, st_vn, ks_vn, hook)                      \
+    LBM_F4(16, cur, pd, prev, next, st_pv, ks_pv, st_qk, h_qk, st_vn, ks_vn, hook)                      \
   }
   f32x16 zero16;
 #pragma unroll
@@ -577,20 +580,28 @@ __device__ __forceinline__ void lbm_attn_split(const AttnCore& a, const LbmAttnS
 
     int st_k = 0, st_v = 0, st_vm1 = 2;  // stages of K(i), V(i), V(i-1)
     // Common frame of one tile iteration.  The loads of K(i+2) and V(i+1) into their ring
-    // stages (free since the barrier that ended iteration i-1) start at the top of iteration
-    // i and have the whole iteration to land; the wait for them sits right before the barrier
-    // that ends it.  Past the last tile the data lands in stages nobody reads any more.  The
-    // row entry fetched for K now serves V in the next iteration.
+    // stages (free since the barrier that ended iteration i-1) and the fetch of the next row
+    // entry are issued from inside the first half-step's slices (LBM_STAGING_HOOK), not in front
+    // of it: after the barrier every wavefront goes straight to matrix instructions whose
+    // operands it already holds, and the address arithmetic of the staging shares slices with
+    // them instead of leaving the matrix pipe idle on all four SIMDs at once.  The loads have
+    // the rest of the iteration to land; the wait for them sits right before the barrier that
+    // ends it.  Past the last tile the data lands in stages nobody reads any more.  The row
+    // entry fetched for K now serves V in the next iteration.
+#define LBM_NO_HOOK(j)
+#define LBM_STAGING_HOOK(j)                                                          \
+    if ((j) == 1) dma(ek, pool_k, own_k, lds_k[st_k2]);                              \
+    if ((j) == 2) dma(ev, pool_v, own_v, lds_v[st_v1]);                              \
+    if ((j) == 3) {                                                                  \
+      ev = ek;                                                                       \
+      ek = row_entry(t + 3);                                                         \
+    }
 #define LBM_TILE_ITERATION(PRE, HALF0, HALF1)                                        \
     {                                                                                \
       const int t = t0 + i;                                                          \
       int st_k1 = st_k + 1; if (st_k1 >= kStages) st_k1 -= kStages;                  \
       int st_k2 = st_k1 + 1; if (st_k2 >= kStages) st_k2 -= kStages;                 \
       int st_v1 = st_v + 1; if (st_v1 >= kStages) st_v1 -= kStages;                  \
-      dma(ek, pool_k, own_k, lds_k[st_k2]);                                          \
-      dma(ev, pool_v, own_v, lds_v[st_v1]);                                          \
-      ev = ek;                                                                       \
-      ek = row_entry(t + 3);                                                         \
       PRE                                                                            \
       HALF0                                                                          \
       HALF1                                                                          \
@@ -606,20 +617,22 @@ __device__ __forceinline__ void lbm_attn_split(const AttnCore& a, const LbmAttnS
     for (const int n_f = safe ? 0 : n_fast; i < n_f; ++i)
       LBM_TILE_ITERATION(
         ,
-        LBM_FAST_HALF_STEP(sA, pA, pB, sB, st_vm1, 3, st_k, 1, st_v, 0);,
-        LBM_FAST_HALF_STEP(sB, pB, pA, sA, st_v, 1, st_k1, 0, st_v, 2);
+        LBM_FAST_HALF_STEP(sA, pA, pB, sB, st_vm1, 3, st_k, 1, st_v, 0, LBM_STAGING_HOOK);,
+        LBM_FAST_HALF_STEP(sB, pB, pA, sA, st_v, 1, st_k1, 0, st_v, 2, LBM_NO_HOOK);
       )
     for (; i < n; ++i)
       LBM_TILE_ITERATION(
         const int n_valid = kv_tokens - t * kKvTile;
         bool hot;,
-        LBM_HALF_STEP(sA, pA, pB, sB, st_vm1, 3, st_k, 1, n_valid, st_v, 0, hot);
+        LBM_HALF_STEP(sA, pA, pB, sB, st_vm1, 3, st_k, 1, n_valid, st_v, 0, hot, LBM_STAGING_HOOK);
         if (safe && __builtin_amdgcn_ballot_w64(hot)) raise_reference(sA, pA, sB);,
         /* after the last tile this QK reads a stale stage; its result is unused */
-        LBM_HALF_STEP(sB, pB, pA, sA, st_v, 1, st_k1, 0, n_valid - kKvTile, st_v, 2, hot);
+        LBM_HALF_STEP(sB, pB, pA, sA, st_v, 1, st_k1, 0, n_valid - kKvTile, st_v, 2, hot, LBM_NO_HOOK);
         if (safe && __builtin_amdgcn_ballot_w64(hot)) raise_reference(sB, pB, sA);
       )
 #undef LBM_TILE_ITERATION
+#undef LBM_STAGING_HOOK
+#undef LBM_NO_HOOK
     // PV and row sums of the last half: pB with half 1 of V(n-1), first k-step already in vnext
     {
       pv_step(vnext, pB, 0);
