@@ -479,10 +479,13 @@ class HipPagedAttention(nn.Module):
             return torch.is_tensor(pos) and pos.is_complex()
         return isinstance(self.rope, RotaryPositionEmbedding2D) and torch.is_tensor(pos) and pos.shape[0] in (1, x.shape[0])
 
-    def dense_attend_fused(self, x: Tensor, pos=None, enable_3d_rope: bool = False, norm=None, stats=None) -> Tensor:
+    def dense_attend_fused(self, x: Tensor, pos=None, enable_3d_rope: bool = False, norm=None, stats=None,
+                           return_kv: bool = False):
         """Attention of every frame of the batch over its own tokens (attention.py:446-465):
         qkv projection, one producer kernel, the paged kernel over a trivial row table.
-        ``norm``, ``stats``: ``x`` is the block's input and ``norm`` is folded into the projection."""
+        ``norm``, ``stats``: ``x`` is the block's input and ``norm`` is folded into the projection.
+        ``return_kv``: also return k and v as ``[B * n, H, D]`` (after q/k norm and rotary
+        embedding), which the anchor pass appends to the cache."""
         import ctypes as C
         from . import _native as N
         from .dense import dense_attention
@@ -519,7 +522,8 @@ class HipPagedAttention(nn.Module):
             N.check(N.lib.lbm_qkv_prepare(
                 p(qkv), dt, p(qk_norm[0]), p(qk_norm[1]), p(qk_norm[2]), p(qk_norm[3]), eps, q_scale, p(table), layout, p(q), p(k), p(v), dt,
                 None, None, B * n, H, D, 16, stream))
-        return dense_attention(q, k, v, num_streams=B, q_prescaled=True).reshape(B, n, H * D)
+        out = dense_attention(q, k, v, num_streams=B, q_prescaled=True).reshape(B, n, H * D)
+        return (out, k, v) if return_kv else out
 
     def forward(self, x: Tensor, pos=None, num_patches=None, num_special=None, num_frames=None,
                 enable_3d_rope=False, kv_cache=None, global_idx=0, num_frame_per_block=1,
@@ -535,15 +539,24 @@ class HipPagedAttention(nn.Module):
                 out = F.scaled_dot_product_attention(q, k, v).transpose(1, 2).reshape(B, N, -1)
         elif num_frames is not None and num_frames > 1:
             # anchor pass over several frames: dense attention among them, then one append
-            # and eviction per frame (attention.py:475-511)
-            assert B == 1, "the multi-frame anchor pass handles one stream"
-            q, k, v = self._qkv(x, pos, enable_3d_rope)
-            out = F.scaled_dot_product_attention(q, k, v).transpose(1, 2).reshape(B, N, -1)
+            # and eviction per frame (attention.py:475-511).  Every stream of the batch attends
+            # among its own frames; the cache takes the streams' frames side by side.
             tpf = kv_cache.tokens_per_frame
-            k_all, v_all = k.squeeze(0).permute(1, 0, 2), v.squeeze(0).permute(1, 0, 2)
+            assert N == num_frames * tpf, f"{N} tokens per stream are not {num_frames} frames of {tpf}"
+            H, D = self.num_heads, self.head_dim
+            if self.can_fuse_dense(x, pos, enable_3d_rope):
+                # producer + the paged kernel over the streams' own rows (8 x 1005 rows per stream
+                # at the reference's defaults: the split-KV kernel), no SDPA, no permutes
+                out, k_all, v_all = self.dense_attend_fused(x, pos, enable_3d_rope, return_kv=True)
+                k_all, v_all = k_all.view(B, num_frames, tpf, H, D), v_all.view(B, num_frames, tpf, H, D)
+            else:
+                q, k, v = self._qkv(x, pos, enable_3d_rope)
+                out = F.scaled_dot_product_attention(q, k, v).transpose(1, 2).reshape(B, N, -1)
+                k_all = k.permute(0, 2, 1, 3).reshape(B, num_frames, tpf, H, D)
+                v_all = v.permute(0, 2, 1, 3).reshape(B, num_frames, tpf, H, D)
             for f in range(num_frames):
-                s = f * tpf
-                kv_cache.append_frame(global_idx, k_all[s:s + tpf].contiguous(), v_all[s:s + tpf].contiguous())
+                kv_cache.append_frame(global_idx, k_all[:, f].reshape(B * tpf, H, D).contiguous(),
+                                      v_all[:, f].reshape(B * tpf, H, D).contiguous())
                 kv_cache.evict_frames(block_idx=global_idx, **self._evict_kwargs(num_register_tokens))
         else:
             if self.can_fuse(kv_cache, pos, enable_3d_rope):
