@@ -192,3 +192,43 @@ def test_config5_full_depth_four_ragged_streams():
         assert mgr.get_cache_stats(23, stream=b) == pols[b].get_cache_stats()
     assert mgr.frame_count == [20] * 24 and model.total_frames_processed == 20
     mgr.check_device_errors()
+
+
+def test_full_width_single_stream_against_fp32_torch():
+    """The width the model ships at - dim 1024, 16 heads, MLP 4096, 1004 tokens per 378 x 518
+    frame - at depth 2, one stream: the path on which every linear is the package's GEMM with the
+    LayerNorms folded in, GELU, LayerScale + residual and the producer in its stores.  Three
+    streamed frames (two keyframes and a read-only one) against the same weights in fp32 torch on
+    the CPU with dict caches; relative bars as above."""
+    from lingbot_map_amd import HipAggregatorStream, set_skip_append
+    dev = torch.device("cuda:0")
+    torch.manual_seed(9)
+    windows, anchor = [16], 1
+    model = HipAggregatorStream(img_size=518, patch_size=14, embed_dim=1024, depth=2, num_heads=16, init_values=1.0,
+                                patch_embed="conv", enable_3d_rope=True, max_frame_num=64,
+                                kv_cache_sliding_window=windows, kv_cache_scale_frames=anchor, use_scale_token=False,
+                                page_size=16, layout="frame_pages", num_streams=1)
+    with torch.no_grad():
+        for tok in (model.camera_token, model.register_token):
+            tok.normal_(std=1.0)
+        for blk in list(model.frame_blocks) + list(model.global_blocks):
+            for norm in (blk.norm1, blk.norm2, blk.attn.q_norm, blk.attn.k_norm):
+                norm.weight.uniform_(0.5, 1.5)
+                norm.bias.uniform_(-0.2, 0.2)
+    model = model.to(dev).eval()
+    ref = TorchReference(model, windows, anchor)
+    model = model.to(torch.bfloat16)
+    g = torch.Generator().manual_seed(10)
+    with torch.no_grad():
+        for f, keyframe in enumerate([True, True, False]):
+            images = torch.rand(1, 1, 3, 378, 518, generator=g)
+            want = ref.step(images, keyframe)
+            set_skip_append(model._get_manager(dev, torch.bfloat16, 1004), not keyframe)
+            got, start = model(images.to(dev, torch.bfloat16))
+            assert start == 5 and len(got) == 2
+            for a, b in zip(got, want):
+                assert a.shape == b.shape == (1, 1, 1004, 2048)
+                err = (a.float().cpu() - b).abs()
+                assert err.max().item() <= 0.02 * b.abs().max().item(), (f, keyframe, err.max().item(), b.abs().max().item())
+                assert err.mean().item() <= 0.01 * b.abs().mean().item(), (f, keyframe, err.mean().item(), b.abs().mean().item())
+    model.kv_cache_manager.check_device_errors()

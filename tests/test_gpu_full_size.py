@@ -161,3 +161,46 @@ def test_config3_end_of_ten_thousand_frame_stream_full_size():
     torch.cuda.synchronize()
     check(out, ref, "shuffled order")
     m.check_device_errors()
+
+
+def test_config5_four_ragged_streams_in_one_launch():
+    """Configuration 5's attention launch by itself, at full size: four streams of 1004 query rows
+    with 5,020 / 9,036 / 17,068 / 17,068 visible tokens (windows 4 / 8 / 16 / 16 plus the anchor
+    frame) in ONE ``lbm_attn_run``, pages in shuffled order, seed 4; every stream against the
+    oracle's SDPA on its own tokens, with the relative bar as well."""
+    from lingbot_map_amd import _native as N
+    from oracle.sdpa_cache import gather_paged, sdpa_nhd
+    dev = torch.device("cuda:0")
+    g = torch.Generator().manual_seed(4)
+    kv_tokens = [(1 + w) * T for w in (4, 8, 16, 16)]
+    assert kv_tokens == [5020, 9036, 17068, 17068]
+    pages_per_frame = (T + S - 1) // S                       # 63: 62 full pages and one of 12 tokens
+    n_pages = sum(n // T for n in kv_tokens) * pages_per_frame
+    pool = torch.randn(n_pages, 2, S, H, D, generator=g).to(torch.bfloat16)
+    q = torch.randn(4 * T, H, D, generator=g).to(torch.bfloat16)
+    order = torch.randperm(n_pages, generator=g).tolist()
+    ids, lens, indptr, at = [], [], [0], 0
+    for n in kv_tokens:
+        for _ in range(n // T):
+            ids += order[at:at + pages_per_frame]
+            lens += [S] * (pages_per_frame - 1) + [T - S * (pages_per_frame - 1)]
+            at += pages_per_frame
+        indptr.append(len(ids))
+    i32 = C.c_int32
+    row_begin = [sum(kv_tokens[:b]) for b in range(4)]
+    ids_d, lens_d = torch.tensor(ids, dtype=torch.int32, device=dev), torch.tensor(lens, dtype=torch.int32, device=dev)
+    rows = torch.empty(sum(kv_tokens), dtype=torch.int32, device=dev)
+    ptr = lambda t: C.c_void_p(t.data_ptr())
+    N.check(N.lib.lbm_rows_from_pages(ptr(ids_d), ptr(lens_d), (i32 * 5)(*indptr), (i32 * 4)(*kv_tokens), (i32 * 4)(*row_begin),
+                                      4, S, ptr(rows), None))
+    streams = (N.AttnStream * 4)(*[N.AttnStream(b * T, T, row_begin[b], kv_tokens[b]) for b in range(4)])
+    ws = torch.empty(max(int(N.lib.lbm_attn_workspace_bytes(streams, 4, H, D)), 16), dtype=torch.uint8, device=dev)
+    qd, pd = q.to(dev), pool.to(dev)
+    out = torch.full_like(qd, float("nan"))
+    N.check(N.lib.lbm_attn_run(ptr(qd), ptr(pd), ptr(out), None, None, ptr(rows), streams, 4, H, D, S, N.DTYPE_BF16,
+                               1.0 / math.sqrt(D), ptr(ws), ws.numel(), None))
+    torch.cuda.synchronize()
+    for b in range(4):
+        kk, vv = gather_paged(pool, ids[indptr[b]:indptr[b + 1]], lens[indptr[b]:indptr[b + 1]])
+        assert kk.shape[0] == kv_tokens[b]
+        check(out[b * T:(b + 1) * T], sdpa_nhd(q[b * T:(b + 1) * T], kk, vv), f"stream {b}: {kv_tokens[b]} tokens")
