@@ -382,8 +382,8 @@ def aggregator_step(torch, blocks: int, steps: int, warmup: int, windows=(WINDOW
     stream (one frame's rows per launch) a block is five launches of the package's own GEMM -
     qkv projection with norm1 folded in and the producer as its store, proj and fc2 with
     LayerScale + residual in theirs, fc1 with norm2 folded in and the GELU in its store - plus the
-    attention; with several streams batched the linears are PyTorch-ROCm library calls and the
-    LayerNorm / residual steps a HIP kernel.  The patch convolution is PyTorch-ROCm.  The prediction
+    attention; several streams batched take the same chain on their concatenated rows (the qkv
+    projection and fc1 then on 256 x 256 tiles).  The patch convolution is PyTorch-ROCm.  The prediction
     heads are not part of the step.  `windows` holds one sliding window per stream: more than
     one entry runs that many independent streams as one ragged batch (a step is then one frame
     of every stream).  `keyframe_interval` > 1 caches every n-th frame only (config 4)."""
@@ -452,6 +452,7 @@ def main() -> None:
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--blocks", type=int, default=24)
+    ap.add_argument("--streams", type=int, default=1, help="--mode aggregator: independent streams batched per step")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-aggregator", action="store_true",
                     help="skip the full aggregator-trunk step (frame + global blocks) timed after the hot path")
@@ -479,11 +480,14 @@ def main() -> None:
                           "launches": args.steps, "avg_launch_us": ms * 1e3}))
         return
     if args.mode == "aggregator":
-        # the one-stream aggregator step alone (eager, then replayed as HIP graphs)
-        print(json.dumps({"mode": "aggregator", "aggregator_step": aggregator_step(torch, args.blocks, 12, 3)}))
+        # the aggregator step alone (eager, then replayed as HIP graphs): one stream, or with
+        # --streams 4 configuration 5's four ragged streams
+        windows = (WINDOW,) if args.streams == 1 else (4, 8, 16, 16)[:args.streams] if args.streams <= 4 else (WINDOW,) * args.streams
+        print(json.dumps({"mode": "aggregator", "streams": args.streams,
+                          "aggregator_step": aggregator_step(torch, args.blocks, 12, 3, windows=windows)}))
         return
     if args.mode == "linear":
-        # the four linears of a block at one frame (1004 rows) and at four streams (4016 rows):
+        # the four linears of a block at one frame (1004 rows), two and four streams (2008, 4016 rows):
         # lbm_linear with its fused epilogue against the PyTorch-ROCm calls it replaces
         from lingbot_map_amd import _native as N
         import ctypes as C
@@ -491,7 +495,7 @@ def main() -> None:
         vp = lambda t: None if t is None else C.c_void_p(t.data_ptr())
         g = torch.Generator(device=dev).manual_seed(5)
         rows = []
-        for M in (1004, 4016):
+        for M in (1004, 2008, 4016):
             for name, K, Nn, epi in (("qkv", 1024, 3072, N.LINEAR_BIAS), ("proj + ls + residual", 1024, 1024, N.LINEAR_BIAS_RESIDUAL),
                                      ("fc1 + gelu", 1024, 4096, N.LINEAR_BIAS_GELU), ("fc2 + ls + residual", 4096, 1024, N.LINEAR_BIAS_RESIDUAL)):
                 a = torch.randn(M, K, generator=g, device=dev).to(torch.bfloat16)

@@ -124,6 +124,16 @@ constexpr int kGeluEntries = 2 * kGeluHalf;
 static __device__ __attribute__((aligned(16))) const unsigned short g_gelu_table[kGeluEntries] = {
 #include "gelu_table.inc"
 };
+// GELU of a value that is already a bf16 (v), rounded to bf16, from the table copy in LDS
+__device__ __forceinline__ float gelu_of_bf16(float v, const unsigned short* tab) {
+  const unsigned b16 = __builtin_bit_cast(unsigned, v) >> 16;
+  const unsigned mag = b16 & 0x7fffu, neg = b16 >> 15;
+  const unsigned rel = mag - (unsigned)(kGeluE0 << 7);
+  const unsigned looked_up = tab[min(rel, (unsigned)(kGeluHalf - 1)) + neg * kGeluHalf];
+  // outside the table: v / 2 below it, v or v * 0 above it (see kGeluE0)
+  const float outside = mag < (unsigned)(kGeluE0 << 7) ? 0.5f * v : (neg ? v * 0.0f : v);
+  return rel < (unsigned)kGeluHalf ? bf16_bits_to_f32(looked_up) : outside;
+}
 
 // TN: output columns per tile (128 or 64); a wavefront owns 64 x (TN / 2) of the tile.
 // ROPE / NORM: rotary layout (0 none, 1 interleaved, 2 half-split) and qk-LayerNorm of the
@@ -492,15 +502,7 @@ __global__ __launch_bounds__(kGThreads, 1) void lbm_linear_bf16_kernel(LinearArg
         float lin = fin[a][c4 * 4 + e];
         if (LNA) lin = __builtin_fmaf(lin, row_f[0], row_f[1] * colsum4[e]);   // rstd * acc - mean * rstd * colsum
         float v = round_bf16(lin + bias4[e]);
-        if (EPI == LBM_LINEAR_BIAS_GELU) {
-          const unsigned b16 = __builtin_bit_cast(unsigned, v) >> 16;
-          const unsigned mag = b16 & 0x7fffu, neg = b16 >> 15;
-          const unsigned rel = mag - (unsigned)(kGeluE0 << 7);
-          const unsigned looked_up = gelu_tab[min(rel, (unsigned)(kGeluHalf - 1)) + neg * kGeluHalf];
-          // outside the table: v / 2 below it, v or v * 0 above it (see kGeluE0)
-          const float outside = mag < (unsigned)(kGeluE0 << 7) ? 0.5f * v : (neg ? v * 0.0f : v);
-          v = rel < (unsigned)kGeluHalf ? bf16_bits_to_f32(looked_up) : outside;
-        }
+        if (EPI == LBM_LINEAR_BIAS_GELU) v = gelu_of_bf16(v, gelu_tab);
         if (EPI == LBM_LINEAR_BIAS_RESIDUAL && p.gamma) v = v * gamma4[e];
         y[e] = v;
       }
@@ -588,6 +590,289 @@ __global__ __launch_bounds__(kGThreads, 1) void lbm_linear_bf16_kernel(LinearArg
   }
 }
 
+
+// ---------------------------------------------------------------------------- several streams' rows
+// The same product on 256 x 256 (or 192 x 256) tiles, for launches with enough rows to give most
+// of the 256 CUs such a tile (four streams' 4,016 rows x the qkv projection's 3,072 or fc1's
+// 4,096 columns): a 256 x 256 tile moves 64 KB of operands per 64 of K for 8.4 MFLOP - 128 FLOP
+// per byte on the way from L2 into LDS, which is what bounds the 128 x 128 tiles above at 64.
+// Eight wavefronts, each on 64 rows x 128 columns of the tile (96 x 64 of a 192-row tile) over
+// the whole K slice, no K split inside the workgroup and so no exchange at the end.  Two LDS
+// stages: a 64-wide step is 24-32 MFMAs per wavefront, longer than a trip to memory, so one step
+// of prefetch is enough; the loads of the next step are issued in between the MFMAs of the
+// current one's first three quarters rather than in one burst (they share the LDS with the
+// fragment reads).  Same operand path (global -> LDS directly, swizzled 16-byte chunks), same
+// epilogue arithmetic and rounding sequence.  Epilogues: bias, bias + GELU, and the
+// pre-attention producer; the folded LayerNorm of the activations; not the residual forms (their
+// 1,024 columns make too few such tiles).  The per-column vectors wait in LDS instead of
+// registers (the accumulators take half the register file).  192-row tiles are for shapes whose
+// 256-row tiles would leave a quarter of the CUs idle (4,016 x 3,072: 192 against 252 tiles).
+constexpr int kBN = 256;
+constexpr int kBCStride = kBN + 4;                          // bf16 per staged output row
+constexpr int lbm_big_lds_bytes(int bm) {
+  return bm * kBCStride * 2 > 2 * (bm + kBN) * kKS * 2 ? bm * kBCStride * 2 : 2 * (bm + kBN) * kKS * 2;
+}
+static_assert(lbm_big_lds_bytes(256) + kGeluEntries * 2 + 2 * kBN * 4 + 256 * 8 <= 160 * 1024, "LDS budget of the 256 x 256 tile");
+
+template <int BM, int EPI, int ROPE = 0, bool NORM = false, bool LNA = false>
+__global__ __launch_bounds__(kGThreads, 1) void lbm_linear_bf16_big_kernel(LinearArgs p) {
+  constexpr int kRowGroups = BM == 256 ? 4 : 2;             // wavefronts along the rows of the tile
+  constexpr int kColGroups = 8 / kRowGroups;
+  constexpr int RB = BM / 32 / kRowGroups, CB = kBN / 32 / kColGroups;   // 32 x 32 blocks per wavefront: 2 x 4 or 3 x 2
+  constexpr int kStageBytes = (BM + kBN) * kKS * 2;
+  __shared__ __attribute__((aligned(1024))) unsigned char lds_raw[lbm_big_lds_bytes(BM)];   // two operand stages, then the staged output tile
+  __shared__ __attribute__((aligned(16))) float colvec[2][kBN];                             // bias, column sums of w (LNA)
+  __shared__ __attribute__((aligned(16))) unsigned short gelu_tab[EPI == LBM_LINEAR_BIAS_GELU ? kGeluEntries : 8];
+  __shared__ __attribute__((aligned(8))) float ln_rows[LNA ? BM * 2 : 2];                   // per row: rstd, -mean * rstd
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int n32 = lane & 31, g = lane >> 5;
+  const int rg = wave % kRowGroups, cg = wave / kRowGroups;
+  const int wm = rg * (RB * 32), wn = cg * (CB * 32);       // this wavefront's corner of the tile
+  int mt, nt;
+  if ((p.n_tiles & 7) == 0) {   // an XCD keeps its own column tiles of w and walks the row tiles with them
+    const int x = blockIdx.x & 7, i = blockIdx.x >> 3;
+    mt = i % p.m_tiles;
+    nt = (i / p.m_tiles) * 8 + x;
+  } else {
+    mt = (int)blockIdx.x % p.m_tiles;
+    nt = (int)blockIdx.x / p.m_tiles;
+  }
+  const int m0 = mt * BM, n0 = nt * kBN;
+
+  // ---- staging (as in the kernel above: eight 128-byte rows per wavefront and load)
+  constexpr int kPassA = BM / 64, kPassW = kBN / 64;
+  const int ld_r = wave * 8 + (lane >> 3);
+  const unsigned sw_c = (unsigned)(((lane & 7) ^ ((ld_r >> 1) & 7)) * 8);
+  unsigned a_off[kPassA];
+#pragma unroll
+  for (int j = 0; j < kPassA; ++j) a_off[j] = ((unsigned)min(m0 + ld_r + 64 * j, p.M - 1) * (unsigned)p.K + sw_c) * 2u;
+  const unsigned w_off = ((unsigned)ld_r * (unsigned)p.K + sw_c) * 2u;
+  const int nk = p.K / kKS;
+  const char* a_base = (const char*)p.a;
+  const char* w_base = (const char*)(p.w + (size_t)n0 * p.K);
+  auto dma_row = [&](const char* base, unsigned voff, const unsigned char* lds_dst) {
+    const unsigned m0v = (unsigned)(size_t)(__attribute__((address_space(3))) const void*)lds_dst;
+    asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1"
+                 :
+                 : "v"(voff), "s"(base), "s"(__builtin_amdgcn_readfirstlane(m0v))
+                 : "memory", "m0");
+  };
+  // load j of step ks: the activations' passes first, then the weights'
+  auto dma_one = [&](int ks, int stage, int j) {
+    unsigned char* st = lds_raw + stage * kStageBytes;
+    if (j < kPassA) dma_row(a_base + ks * (kKS * 2), a_off[j], st + (64 * j + 8 * wave) * (kKS * 2));
+    else dma_row(w_base + ((size_t)(64 * (j - kPassA)) * p.K + (size_t)ks * kKS) * 2, w_off,
+                 st + BM * kKS * 2 + (64 * (j - kPassA) + 8 * wave) * (kKS * 2));
+  };
+  constexpr int kDma = kPassA + kPassW;
+
+  // the folded LayerNorm's row statistics: two threads per row, each every second partial
+  constexpr int kLnHeld = 8;
+  f32x2 ln_part[kLnHeld] = {};
+  if (LNA) {
+    const float* ln_st = p.ln_stats + (size_t)min(m0 + (tid >> 1), p.M - 1) * p.ln_tiles * 2;
+#pragma unroll
+    for (int i = 0; i < kLnHeld; ++i)
+      if ((tid & 1) + 2 * i < p.ln_tiles) ln_part[i] = *(const f32x2*)(ln_st + 2 * ((tid & 1) + 2 * i));
+  }
+  // per-column vectors of the tile into LDS (read in the epilogue, many barriers from here)
+  float cv_bias = 0.f, cv_sum = 0.f;
+  if (tid < kBN) {
+    if (p.bias) cv_bias = p.bias[n0 + tid];
+    if (LNA) cv_sum = p.ln_colsum[n0 + tid];
+  }
+  if (EPI == LBM_LINEAR_BIAS_GELU && tid < kGeluEntries / 8)
+    dma_row((const char*)g_gelu_table, (unsigned)tid * 16u, (const unsigned char*)&gelu_tab[wave * 512]);
+#pragma unroll
+  for (int j = 0; j < kDma; ++j) dma_one(0, 0, j);
+  if (tid < kBN) {
+    colvec[0][tid] = cv_bias;
+    colvec[1][tid] = cv_sum;
+  }
+  if (LNA && (tid >> 1) < BM) {
+    const int r = tid >> 1, part = tid & 1;
+    const float* ln_st = p.ln_stats + (size_t)min(m0 + r, p.M - 1) * p.ln_tiles * 2;
+    float sm = 0.f;
+#pragma unroll
+    for (int i = 0; i < kLnHeld; ++i)
+      if (part + 2 * i < p.ln_tiles) sm += ln_part[i][0];
+    for (int i = part + 2 * kLnHeld; i < p.ln_tiles; i += 2) sm += ln_st[2 * i];
+    sm += lbm_qkv::lane_xor1(sm);
+    const float mean = sm / (float)p.ln_tiles;
+    const float n_i = (float)p.K / (float)p.ln_tiles;
+    float m2 = 0.f;
+#pragma unroll
+    for (int i = 0; i < kLnHeld; ++i)
+      if (part + 2 * i < p.ln_tiles) {
+        const float d = ln_part[i][0] - mean;
+        m2 += ln_part[i][1] + n_i * d * d;
+      }
+    for (int i = part + 2 * kLnHeld; i < p.ln_tiles; i += 2) {
+      const float d = ln_st[2 * i] - mean;
+      m2 += ln_st[2 * i + 1] + n_i * d * d;
+    }
+    m2 += lbm_qkv::lane_xor1(m2);
+    const float rstd = __builtin_amdgcn_rsqf(m2 / (float)p.K + p.ln_eps);
+    if (part == 0) {
+      ln_rows[2 * r] = rstd;
+      ln_rows[2 * r + 1] = -mean * rstd;
+    }
+  }
+
+  f32x16 acc[CB][RB];   // [column block of w][row block of a]; element i: column 8 (i / 4) + 4 g + i % 4, row n32
+#pragma unroll
+  for (int a = 0; a < CB; ++a)
+#pragma unroll
+    for (int b = 0; b < RB; ++b)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) acc[a][b][i] = 0.f;
+
+  const int sw_r = (n32 >> 1) & 7;
+  for (int s = 0; s < nk; ++s) {
+    LBM_DMA_WAIT(0);
+    __syncthreads();   // step s has landed everywhere, and everyone is done with step s - 1, whose stage step s + 1 lands in
+    const unsigned short* la = (const unsigned short*)(lds_raw + (s & 1) * kStageBytes);
+    const unsigned short* lw = la + BM * kKS;
+    bf16x8 wf[2][CB], af[2][RB];
+    auto read = [&](int kq, bf16x8 (&wfr)[CB], bf16x8 (&afr)[RB]) {
+      const int pos = ((kq * 2 + g) ^ sw_r) * 8;
+#pragma unroll
+      for (int a = 0; a < CB; ++a)
+        wfr[a] = __builtin_bit_cast(bf16x8, *(const u32x4*)&lw[(wn + a * 32 + n32) * kKS + pos]);
+#pragma unroll
+      for (int b = 0; b < RB; ++b)
+        afr[b] = __builtin_bit_cast(bf16x8, *(const u32x4*)&la[(wm + b * 32 + n32) * kKS + pos]);
+    };
+    read(0, wf[0], af[0]);
+#pragma unroll
+    for (int kq = 0; kq < 4; ++kq) {
+      if (kq < 3) read(kq + 1, wf[(kq + 1) & 1], af[(kq + 1) & 1]);
+      if (s + 1 < nk) {
+#pragma unroll
+        for (int j = 0; j < kDma; ++j)
+          if (j * 3 / kDma == kq) dma_one(s + 1, (s + 1) & 1, j);   // a third of the next step's loads per quarter step
+      }
+#pragma unroll
+      for (int a = 0; a < CB; ++a)
+#pragma unroll
+        for (int b = 0; b < RB; ++b)
+          acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wf[kq & 1][a], af[kq & 1][b], acc[a][b], 0, 0, 0);
+    }
+  }
+
+  // ---- epilogue.  What the producer's first passes need from global memory is asked for now and
+  // arrives while the tile is staged.
+  constexpr int kPieces = kBN / 8;                    // 16-byte pieces per row of the tile: 32
+  constexpr int kRowsPerPass = kGThreads / kPieces;   // 16
+  constexpr int kPasses = BM / kRowsPerPass;          // 16 or 12
+  constexpr int kGroup = 4;                           // passes whose rotary entries and pool rows travel together
+  const int pr = tid / kPieces, pc = (tid % kPieces) * 8;
+  typedef lbm_qkv::f32x4 qf4;
+  const int H = p.num_heads;
+  const int pq_col = n0 + pc;
+  const int which = EPI == kEpiQkvPrepare ? pq_col / (H * 64) : 0;   // uniform over the workgroup (H * 64 is a multiple of 256)
+  const int ph = (pq_col - which * H * 64) >> 6, c8 = (pq_col & 63) >> 3;
+  qf4 w4[2] = {}, b4[2] = {};
+  qf4 cs4[2][kGroup][4] = {};
+  int pool_row[2][kGroup];
+  auto ask = [&](int grp, qf4 (&cs)[kGroup][4], int (&rows)[kGroup]) {
+#pragma unroll
+    for (int j = 0; j < kGroup; ++j) {
+      const int t = min(m0 + (grp * kGroup + j) * kRowsPerPass + pr, p.M - 1);
+      if (ROPE == 1 && which < 2) {
+        const qf4* src = (const qf4*)(p.rope_cs + ((long long)t * 32 + c8 * 4) * 2);
+        cs[j][0] = src[0]; cs[j][1] = src[1];
+      } else if (ROPE == 2 && which < 2) {
+        const qf4* src = (const qf4*)(p.rope_cs + ((long long)t * 64 + c8 * 8) * 2);
+        cs[j][0] = src[0]; cs[j][1] = src[1]; cs[j][2] = src[2]; cs[j][3] = src[3];
+      }
+      rows[j] = -1;
+      if (which > 0 && p.append_rows) rows[j] = p.append_rows[t];
+    }
+  };
+  if (EPI == kEpiQkvPrepare) {
+    if (NORM && which < 2) {
+      const qf4* wp = (const qf4*)((which == 0 ? p.q_norm_w : p.k_norm_w) + c8 * 8);
+      const qf4* bp = (const qf4*)((which == 0 ? p.q_norm_b : p.k_norm_b) + c8 * 8);
+      w4[0] = wp[0]; w4[1] = wp[1];
+      b4[0] = bp[0]; b4[1] = bp[1];
+    }
+    ask(0, cs4[0], pool_row[0]);
+  }
+  __syncthreads();   // the operand stages are dead: the output tile is staged over them
+  // In registers: the folded LayerNorm's scale and correction, + bias, round (the linear's
+  // output), GELU, round; then the tile goes through LDS and leaves as whole rows.
+  unsigned short* stage = (unsigned short*)lds_raw;
+#pragma unroll
+  for (int b = 0; b < RB; ++b) {
+    const int row = wm + b * 32 + n32;
+    f32x2 row_f = {1.f, 0.f};
+    if (LNA) row_f = *(const f32x2*)&ln_rows[2 * row];
+#pragma unroll
+    for (int a = 0; a < CB; ++a)
+#pragma unroll
+      for (int c4 = 0; c4 < 4; ++c4) {
+        const int col = wn + a * 32 + c4 * 8 + g * 4;
+        const f32x4 bias4 = *(const f32x4*)&colvec[0][col], colsum4 = *(const f32x4*)&colvec[1][col];
+        f32x4 y;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          float lin = acc[a][b][c4 * 4 + e];
+          if (LNA) lin = __builtin_fmaf(lin, row_f[0], row_f[1] * colsum4[e]);
+          float v = round_bf16(lin + bias4[e]);
+          if (EPI == LBM_LINEAR_BIAS_GELU) v = gelu_of_bf16(v, gelu_tab);
+          y[e] = v;
+        }
+        *(bf16x4*)&stage[row * kBCStride + col] = __builtin_convertvector(y, bf16x4);
+      }
+  }
+  __syncthreads();
+  if (EPI == kEpiQkvPrepare) {
+    // the producer on the staged tile, as in the kernel above; the rotary entries and pool rows of
+    // four passes are asked for while the four before them are worked on
+    unsigned short* dst_plain = which == 0 ? p.out : (which == 1 ? p.k_out : p.v_out);
+    const float post = which == 0 ? p.q_scale : 1.0f;
+    auto work = [&](int grp, const qf4 (&cs)[kGroup][4], const int (&rows)[kGroup]) {
+#pragma unroll
+      for (int j = 0; j < kGroup; ++j) {
+        const int r = (grp * kGroup + j) * kRowsPerPass + pr;
+        const bool valid = m0 + r < p.M;
+        const u32x2 lo = *(const u32x2*)&stage[r * kBCStride + pc], hi = *(const u32x2*)&stage[r * kBCStride + pc + 4];
+        const u32x4 raw = {lo[0], lo[1], hi[0], hi[1]};
+        float x[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) x[i] = __builtin_bit_cast(float, (i & 1) ? (raw[i >> 1] & 0xffff0000u) : (raw[i >> 1] << 16));
+        if (which < 2) lbm_qkv::norm_rope<0, ROPE, NORM>(x, w4, b4, cs[j], c8, p.eps, post);
+        bf16x8 o8;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) o8[i] = (__bf16)x[i];
+        if (valid) {
+          const long long nhd = ((long long)(m0 + r) * H + ph) * 64 + c8 * 8;
+          if (dst_plain) *(bf16x8*)(dst_plain + nhd) = o8;
+          if (which > 0 && rows[j] >= 0) {
+            const long long row_elems = (long long)H * 64;
+            const long long d = (long long)rows[j] * row_elems + (which == 2 ? (long long)p.page_size * row_elems : 0) + ph * 64 + c8 * 8;
+            *(bf16x8*)(p.pool + d) = o8;
+          }
+        }
+      }
+    };
+#pragma unroll
+    for (int grp = 0; grp < kPasses / kGroup; ++grp) {
+      if (grp + 1 < kPasses / kGroup) ask(grp + 1, cs4[(grp + 1) & 1], pool_row[(grp + 1) & 1]);
+      work(grp, cs4[grp & 1], pool_row[grp & 1]);
+    }
+    return;
+  }
+#pragma unroll
+  for (int j = 0; j < kPasses; ++j) {
+    const int r = j * kRowsPerPass + pr, row = m0 + r;
+    const u32x2 lo = *(const u32x2*)&stage[r * kBCStride + pc], hi = *(const u32x2*)&stage[r * kBCStride + pc + 4];
+    if (row < p.M) *(u32x4*)(p.out + (size_t)row * p.N + n0 + pc) = u32x4{lo[0], lo[1], hi[0], hi[1]};
+  }
+}
+
 }  // namespace
 
 namespace {
@@ -600,6 +885,29 @@ int lbm_linear_tiles(LinearArgs& p) {
   const int tn = wide ? 128 : 64;
   p.n_tiles = p.N / tn;
   return tn;
+}
+}  // namespace
+
+namespace {
+// 256- or 192-row tiles of 256 columns when they give at least half of the 256 CUs a workgroup
+// (several streams' rows into the 3,072 or 4,096 columns of the qkv projection or fc1): the row
+// count of the tile (the one that needs fewer rounds of the CUs times rows), or 0; sets the tile
+// counts
+int lbm_linear_big_tiles(LinearArgs& p) {
+  if (p.N % kBN != 0) return 0;
+  const int nt = p.N / kBN;
+  int best = 0;
+  long long best_cost = 0;
+  for (int bm : {256, 192}) {
+    const long long tiles = (long long)((p.M + bm - 1) / bm) * nt;
+    if (tiles < 128) continue;
+    const long long cost = ((tiles + 255) / 256) * bm;      // rounds of the 256 CUs x rows per tile
+    if (!best || cost < best_cost) best = bm, best_cost = cost;
+  }
+  if (!best) return 0;
+  p.m_tiles = (p.M + best - 1) / best;
+  p.n_tiles = nt;
+  return best;
 }
 }  // namespace
 
@@ -676,9 +984,25 @@ int lbm_launch_linear(const void* a, const lbm_row_norm* a_norm, const void* w, 
   p.out = (unsigned short*)out;
   p.M = M; p.N = N; p.K = K;
   if (int rc = lbm_set_row_norm(p, a_norm, "lbm_linear_norm")) return rc;
-  const bool wide = lbm_linear_tiles(p) == 128;
   const bool lna = a_norm != nullptr;
   const dim3 block(kGThreads);
+  if (epilogue == LBM_LINEAR_BIAS || epilogue == LBM_LINEAR_BIAS_GELU) {
+    if (const int bm = lbm_linear_big_tiles(p)) {
+      const dim3 grid_b((unsigned)(p.m_tiles * p.n_tiles));
+#define LBM_BIG_LAUNCH(E, L)                                                                                         \
+      {                                                                                                              \
+        if (bm == 256) hipLaunchKernelGGL((lbm_linear_bf16_big_kernel<256, E, 0, false, L>), grid_b, block, 0, stream, p); \
+        else hipLaunchKernelGGL((lbm_linear_bf16_big_kernel<192, E, 0, false, L>), grid_b, block, 0, stream, p);           \
+      }
+      if (epilogue == LBM_LINEAR_BIAS && lna) LBM_BIG_LAUNCH(LBM_LINEAR_BIAS, true)
+      else if (epilogue == LBM_LINEAR_BIAS) LBM_BIG_LAUNCH(LBM_LINEAR_BIAS, false)
+      else if (lna) LBM_BIG_LAUNCH(LBM_LINEAR_BIAS_GELU, true)
+      else LBM_BIG_LAUNCH(LBM_LINEAR_BIAS_GELU, false)
+#undef LBM_BIG_LAUNCH
+      return lbm_check_launch("lbm_linear_bf16_big_kernel");
+    }
+  }
+  const bool wide = lbm_linear_tiles(p) == 128;
   if (workspace) {
     const int splits = lbm_linear_splits(p, epilogue);
     if (splits > 1 && workspace_bytes >= lbm_linear_workspace_for(M, N, K, epilogue)) {
@@ -735,6 +1059,30 @@ int lbm_launch_qkv_linear_prepare(const void* a, const lbm_row_norm* a_norm, con
   p.num_heads = num_heads; p.page_size = page_size;
   if (int rc = lbm_set_row_norm(p, a_norm, "lbm_qkv_linear_prepare_norm")) return rc;
   const bool lna = a_norm != nullptr;
+  const int rope = !rope_cs ? 0 : (rope_layout == LBM_ROPE_INTERLEAVED ? 1 : 2);
+  const bool norm = q_norm_w != nullptr;
+  // 256-wide tiles: four whole heads each, so that a tile does not straddle q | k | v
+  if (const int bm = (num_heads & 3) == 0 ? lbm_linear_big_tiles(p) : 0) {
+    const dim3 grid_b((unsigned)(p.m_tiles * p.n_tiles)), block_b(kGThreads);
+#define LBM_QKV_BIG_M(BM, R, NRM)                                                                                               \
+    {                                                                                                                           \
+      if (lna) hipLaunchKernelGGL((lbm_linear_bf16_big_kernel<BM, kEpiQkvPrepare, R, NRM, true>), grid_b, block_b, 0, stream, p);  \
+      else hipLaunchKernelGGL((lbm_linear_bf16_big_kernel<BM, kEpiQkvPrepare, R, NRM, false>), grid_b, block_b, 0, stream, p);     \
+    }
+#define LBM_QKV_BIG(R, NRM)                                                  \
+    {                                                                        \
+      if (bm == 256) LBM_QKV_BIG_M(256, R, NRM) else LBM_QKV_BIG_M(192, R, NRM) \
+    }
+    if (rope == 0 && !norm) LBM_QKV_BIG(0, false)
+    else if (rope == 0) LBM_QKV_BIG(0, true)
+    else if (rope == 1 && !norm) LBM_QKV_BIG(1, false)
+    else if (rope == 1) LBM_QKV_BIG(1, true)
+    else if (!norm) LBM_QKV_BIG(2, false)
+    else LBM_QKV_BIG(2, true)
+#undef LBM_QKV_BIG
+#undef LBM_QKV_BIG_M
+    return lbm_check_launch("lbm_linear_bf16_big_kernel<qkv prepare>");
+  }
   // a tile must not straddle q | k | v: 128-wide tiles need an even number of heads
   bool wide = lbm_linear_tiles(p) == 128;
   if (wide && (num_heads & 1)) {
@@ -742,8 +1090,6 @@ int lbm_launch_qkv_linear_prepare(const void* a, const lbm_row_norm* a_norm, con
     p.n_tiles = N / 64;
   }
   const dim3 grid((unsigned)(p.m_tiles * p.n_tiles)), block(kGThreads);
-  const int rope = !rope_cs ? 0 : (rope_layout == LBM_ROPE_INTERLEAVED ? 1 : 2);
-  const bool norm = q_norm_w != nullptr;
 #define LBM_QKV_LAUNCH_L(R, NRM, L)                                                                                   \
   {                                                                                                                   \
     if (wide) hipLaunchKernelGGL((lbm_linear_bf16_kernel<kEpiQkvPrepare, 128, R, NRM, L>), grid, block, 0, stream, p); \

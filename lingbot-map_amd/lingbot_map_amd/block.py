@@ -261,9 +261,9 @@ class Mlp(nn.Module):
         self.act = act_layer()
         self.fc2 = nn.Linear(hidden_features, in_features, bias=bias)
 
-    #: rows up to which the fused fc1 + GELU kernel beats the library GEMM followed by a GELU kernel
-    #: (one frame per call; at several streams' rows the library's larger tiles win)
-    FUSED_MAX_ROWS = 1280
+    #: rows up to which the fused launches are used: one frame's rows run on 128 x 128 tiles, several
+    #: streams' rows on 256 x 256 tiles where the launch has the columns for them (qkv, fc1)
+    FUSED_MAX_ROWS = 1 << 16
 
     def _can_fuse_fc1(self, x: Tensor) -> bool:
         fc1 = self.fc1
@@ -420,9 +420,8 @@ class HipPagedAttention(nn.Module):
                                 cross_frame_special=self.kv_cache_cross_frame_special,
                                 camera_only=self.kv_cache_camera_only, proj=proj)
 
-    #: rows up to which the projection with the producer as its epilogue is used (one frame per
-    #: call; at several streams' rows the library GEMM's larger tiles win)
-    FUSED_PROJ_MAX_ROWS = 1280
+    #: rows up to which the projection with the producer as its epilogue is used (see Mlp.FUSED_MAX_ROWS)
+    FUSED_PROJ_MAX_ROWS = 1 << 16
 
     def _fused_projection(self, x: Tensor, cache_dtype, norm: Optional[nn.LayerNorm] = None,
                           stats: Optional[RowStats] = None) -> Optional[tuple]:

@@ -60,7 +60,9 @@ def _inputs(M, K, Nn, seed, with_bias=True):
     return a, w, bias, g
 
 
-@pytest.mark.parametrize("M,K,Nn", [(1004, 1024, 3072), (1004, 1024, 1024), (70, 128, 64), (4016, 1024, 1024), (129, 128, 192), (1, 128, 128)])
+# (the 4016- and 2100-row launches into 3072 / 4096 columns run on the 256 x 256 tiles)
+@pytest.mark.parametrize("M,K,Nn", [(1004, 1024, 3072), (1004, 1024, 1024), (70, 128, 64), (4016, 1024, 1024), (129, 128, 192), (1, 128, 128),
+                                    (4016, 1024, 3072), (2100, 1024, 4096), (4016, 128, 4096)])
 def test_linear_bias(M, K, Nn):
     N = _native()
     a, w, bias, _ = _inputs(M, K, Nn, seed=M + Nn)
@@ -90,7 +92,7 @@ def test_gelu_epilogue_on_every_bf16_pre_activation():
     assert ((got.float() - ref.float()).abs()[tail] <= 2.0 ** -8 * 2.0 ** -7 * pre.float().abs()[tail] + 1e-30).all()
 
 
-@pytest.mark.parametrize("M,K,Nn", [(1004, 1024, 4096), (257, 256, 320)])
+@pytest.mark.parametrize("M,K,Nn", [(1004, 1024, 4096), (257, 256, 320), (4016, 1024, 4096)])
 def test_linear_bias_gelu(M, K, Nn):
     N = _native()
     a, w, bias, _ = _inputs(M, K, Nn, seed=7)
@@ -145,9 +147,9 @@ def test_linear_rows_past_m_are_not_written_and_arguments_are_checked():
 
 
 def test_mlp_with_fused_fc1_gelu_equals_the_unfused_module():
-    """The block's Mlp takes the fused kernel for one frame's rows in bf16 and the plain torch ops
-    otherwise (fp32, tanh GELU, many rows); both give the same numbers up to one bf16 ulp of the
-    hidden activations."""
+    """The block's Mlp takes the fused kernel for bf16 rows (one frame's or several streams') and the
+    plain torch ops otherwise (fp32, tanh GELU); both give the same numbers up to one bf16 ulp of
+    the hidden activations."""
     from lingbot_map_amd.block import Mlp
     torch.manual_seed(0)
     dev = torch.device("cuda:0")
@@ -161,15 +163,17 @@ def test_mlp_with_fused_fc1_gelu_equals_the_unfused_module():
         check(hidden.cpu(), ref_hidden.cpu(), scale=pre.cpu(), bar=1.2 * 2.0 ** -7 + 2.0 ** -8)
         out, ref = mlp(x), mlp.fc2(ref_hidden)
         assert (out.float() - ref.float()).abs().max().item() <= 2.0 ** -6 * ref.float().abs().max().item()
-        # not taken: fp32 activations, the tanh approximation, more rows than one frame
+        # not taken: fp32 activations, the tanh approximation; taken: four streams' rows
         assert not mlp._can_fuse_fc1(x.float())
         assert not Mlp(256, 1024, act_layer=lambda: torch.nn.GELU(approximate="tanh")).to(dev).to(torch.bfloat16)._can_fuse_fc1(x)
-        assert not mlp._can_fuse_fc1(torch.zeros(4, 1004, 256, device=dev, dtype=torch.bfloat16))
+        many = torch.randn(4, 1004, 256, device=dev).to(torch.bfloat16)
+        assert mlp._can_fuse_fc1(many)
+        check(mlp.fc1_gelu(many).cpu(), mlp.act(mlp.fc1(many)).cpu(), scale=mlp.fc1(many).cpu(), bar=1.2 * 2.0 ** -7 + 2.0 ** -8)
 
 
 @pytest.mark.parametrize("rope", ["none", "interleaved", "half_split"])
 @pytest.mark.parametrize("norm", [False, True])
-@pytest.mark.parametrize("M,H,K", [(1004, 16, 1024), (70, 3, 128)])
+@pytest.mark.parametrize("M,H,K", [(1004, 16, 1024), (70, 3, 128), (4016, 16, 1024), (3900, 16, 256)])
 def test_qkv_projection_with_the_producer_as_its_epilogue(M, H, K, norm, rope):
     """lbm_qkv_linear_prepare against lbm_linear (bias) followed by lbm_qkv_prepare on its output:
     the same arithmetic on the same rounded projection, so q, k, v and the pool rows are bit-equal.
@@ -276,7 +280,8 @@ def _stats_of(x, tiles):
 
 
 @pytest.mark.parametrize("M,K,Nn,tiles,epilogue", [(1004, 1024, 4096, 16, 1), (1004, 1024, 3072, 8, 0), (200, 256, 128, 4, 1),
-                                                   (77, 2048, 64, 32, 0)])
+                                                   (77, 2048, 64, 32, 0), (4016, 1024, 4096, 8, 1), (4016, 1024, 3072, 16, 0),
+                                                   (2050, 2048, 4096, 32, 0)])
 def test_layernorm_folded_into_the_linear(M, K, Nn, tiles, epilogue):
     """lbm_linear_norm with a_norm (the LayerNorm's affine part folded into weight and bias by the
     caller) against LayerNorm (torch, bf16 in and out) followed by the plain lbm_linear arithmetic
@@ -316,13 +321,14 @@ def test_layernorm_folded_into_the_linear(M, K, Nn, tiles, epilogue):
     assert N.lib.lbm_linear_norm(ptr(xd), N.RowNorm(stats.data_ptr(), None, tiles, 1e-5), ptr(wd), ptr(bd), None, None, ptr(out), None, M, Nn, K, epilogue, None, 0, None) != N.OK
 
 
-def test_layernorm_folded_into_the_qkv_projection_and_producer():
+@pytest.mark.parametrize("M", [1004, 4016])
+def test_layernorm_folded_into_the_qkv_projection_and_producer(M):
     """lbm_qkv_linear_prepare_norm (norm1 folded into the projection) against the same launch fed
     with the LayerNorm computed by torch: q, k, v agree to a bf16 step of the largest values, the
     mean difference a small fraction of that."""
     N = _native()
     dev = torch.device("cuda:0")
-    M, H, K, D, S, tiles = 1004, 16, 1024, 64, 16, 16
+    H, K, D, S, tiles = 16, 1024, 64, 16, 16
     g = torch.Generator().manual_seed(91)
     x = (torch.randn(M, K, generator=g) * 1.7 + 0.2).to(torch.bfloat16)
     lw = (1 + 0.2 * torch.randn(K, generator=g)).to(torch.bfloat16)
