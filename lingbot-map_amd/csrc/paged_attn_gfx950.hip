@@ -611,10 +611,37 @@ __device__ __forceinline__ void lbm_attn_split(const AttnCore& a, const LbmAttnS
       st_vm1 = st_v;                                                                 \
       st_v = st_v1;                                                                  \
     }
+    // The same frame with the ring stages as compile-time constants (the ring has three stages,
+    // so three iterations bring it back to where it started): every LDS address of the
+    // iteration is then one per-lane register plus an immediate offset, and the thirty-odd vector
+    // and scalar instructions per tile that add a run-time stage base to it are gone.
+#define LBM_TILE_ITERATION_AT(U, SK, HALF0, HALF1)                                   \
+    {                                                                                \
+      const int t = t0 + i + (U);                                                    \
+      constexpr int st_k = (SK), st_v = (SK), st_vm1 = ((SK) + 2) % kStages;          \
+      constexpr int st_k1 = ((SK) + 1) % kStages, st_k2 = ((SK) + 2) % kStages;       \
+      constexpr int st_v1 = ((SK) + 1) % kStages;                                    \
+      HALF0                                                                          \
+      HALF1                                                                          \
+      LBM_DMA_LANDED();                                                              \
+      __syncthreads();                                                               \
+    }
     int i = 0;
     // half 0 of tile i: softmax(sA) -> pA | PV(tile i-1, half 1) with pB | QK(tile i, half 1) -> sB
     // half 1 of tile i: softmax(sB) -> pB | PV(tile i, half 0) with pA | QK(tile i+1, half 0) -> sA
-    for (const int n_f = safe ? 0 : n_fast; i < n_f; ++i)
+    const int n_f = safe ? 0 : n_fast;
+#define LBM_FAST_ITERATION_AT(U, SK)                                                              \
+      LBM_TILE_ITERATION_AT(U, SK,                                                                 \
+        LBM_FAST_HALF_STEP(sA, pA, pB, sB, st_vm1, 3, st_k, 1, st_v, 0, LBM_STAGING_HOOK);,        \
+        LBM_FAST_HALF_STEP(sB, pB, pA, sA, st_v, 1, st_k1, 0, st_v, 2, LBM_NO_HOOK);)
+    for (; i + kStages <= n_f; i += kStages) {   // (entered with st_k = st_v = 0, st_vm1 = 2, and left so)
+      LBM_FAST_ITERATION_AT(0, 0)
+      LBM_FAST_ITERATION_AT(1, 1)
+      LBM_FAST_ITERATION_AT(2, 2)
+    }
+#undef LBM_FAST_ITERATION_AT
+#undef LBM_TILE_ITERATION_AT
+    for (; i < n_f; ++i)
       LBM_TILE_ITERATION(
         ,
         LBM_FAST_HALF_STEP(sA, pA, pB, sB, st_vm1, 3, st_k, 1, st_v, 0, LBM_STAGING_HOOK);,
