@@ -439,9 +439,7 @@ def aggregator_step(torch, blocks: int, steps: int, warmup: int, windows=(WINDOW
             "hip_graph": {"value": B / dt_graph, "unit": "frames/s", "ms_per_step": dt_graph * 1e3},
             "what": f"HipAggregatorStream: patch convolution + 24 encoder blocks + {blocks} x (frame block + global block), "
                     f"dim {H * D}, {H} heads, MLP {4 * H * D}, {B} stream(s), {T} tokens/frame, steady-state cache of {kv} "
-                    f"KV tokens; " + ("the package's GEMM with fused LayerNorm / GELU / LayerScale + residual / producer for every "
-                                      "linear" if B == 1 else "PyTorch-ROCm for the linears and GELU, HIP kernels for LayerNorm + residual and "
-                                      "q/k norm + rotary + append") +
+                    f"KV tokens; the package's GEMM with fused LayerNorm / GELU / LayerScale + residual / producer for every linear"
                     ", HIP kernels for the cache path and every block's cache-less attention, PyTorch-ROCm for the patch "
                     "convolution; prediction heads excluded"}
 

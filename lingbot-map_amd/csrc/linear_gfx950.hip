@@ -36,6 +36,7 @@
 // the choice of source address, so the b128 fragment reads are free of bank conflicts.  One
 // workgroup barrier per slice.  The tile leaves through LDS as whole rows: 16-byte stores, and
 // the residual is read the same way.
+#include <type_traits>
 #include <hip/hip_runtime.h>
 #include "lbm_internal.h"
 #include "qkv_math.h"
@@ -135,6 +136,23 @@ __device__ __forceinline__ float gelu_of_bf16(float v, const unsigned short* tab
   return rel < (unsigned)kGeluHalf ? bf16_bits_to_f32(looked_up) : outside;
 }
 
+// Workgroup b's tile.  Workgroups are dealt to the 8 XCDs round-robin (b % 8), 32 of a round of 256
+// to each; an XCD's 32 take consecutive tiles of an order that walks panels of 8 column tiles row
+// by row, i.e. 4 row tiles x 8 column tiles (8 x 4 in a last panel of 4): 12 operand tiles per
+// k-step for the XCD's L2 to hold instead of 17 to 33, which is what sets the latency of the
+// operand loads.
+__device__ __forceinline__ void lbm_tile_of_workgroup(int b, int m_tiles, int n_tiles, int& mt, int& nt) {
+  const int x = b & 7, i = b >> 3;
+  const int base = (i >> 5) * 256;
+  const int in_round = min(m_tiles * n_tiles - base, 256);
+  const int t = base + x * (in_round >> 3) + min(x, in_round & 7) + (i & 31);
+  const int panel_tiles = m_tiles * 8;
+  const int panel = t / panel_tiles, rem = t - panel * panel_tiles;
+  const int width = min(8, n_tiles - panel * 8);
+  mt = rem / width;
+  nt = panel * 8 + rem - mt * width;
+}
+
 // TN: output columns per tile (128 or 64); a wavefront owns 64 x (TN / 2) of the tile.
 // ROPE / NORM: rotary layout (0 none, 1 interleaved, 2 half-split) and qk-LayerNorm of the
 // kEpiQkvPrepare epilogue; 0 / false otherwise.
@@ -149,6 +167,7 @@ __global__ __launch_bounds__(kGThreads, 1) void lbm_linear_bf16_kernel(LinearArg
   __shared__ __attribute__((aligned(16))) unsigned short lds_w[kStagesG][TN * kKS];
   __shared__ __attribute__((aligned(16))) unsigned short gelu_tab[EPI == LBM_LINEAR_BIAS_GELU ? kGeluEntries : 8];
   __shared__ __attribute__((aligned(8))) float ln_rows[LNA ? kGM * 2 : 2];   // per row of the tile: rstd, -mean * rstd
+  __shared__ __attribute__((aligned(16))) float colvec[3][TN];               // bias, column sums of w (LNA), LayerScale
 
   const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int n32 = lane & 31, g = lane >> 5;
@@ -159,13 +178,13 @@ __global__ __launch_bounds__(kGThreads, 1) void lbm_linear_bf16_kernel(LinearArg
   int mt, nt, split = 0;
   {
     const int n_tiles_all = p.m_tiles * p.n_tiles;
-    if ((p.n_tiles & 7) == 0) {
+    if (!SPLITK) {
+      lbm_tile_of_workgroup((int)blockIdx.x, p.m_tiles, p.n_tiles, mt, nt);
+    } else if ((p.n_tiles & 7) == 0) {
       const int x = blockIdx.x & 7;
       int i = blockIdx.x >> 3;
-      if (SPLITK) {
-        split = i / (n_tiles_all >> 3);
-        i -= split * (n_tiles_all >> 3);
-      }
+      split = i / (n_tiles_all >> 3);
+      i -= split * (n_tiles_all >> 3);
       mt = i % p.m_tiles;
       nt = (i / p.m_tiles) * 8 + x;
     } else {
@@ -220,6 +239,20 @@ __global__ __launch_bounds__(kGThreads, 1) void lbm_linear_bf16_kernel(LinearArg
     for (int j = 0; j < kPassW; ++j)
       dma_row(w_base + ((size_t)(64 * j) * p.K + (size_t)ks * kKS) * 2, w_off, &lds_w[stage][(64 * j + 8 * wave) * kKS]);
   };
+  // the same loads one by one, for the loop: M0 values and row offsets as integers, so that
+  // nothing but two scalar adds and the load itself sits between the MFMAs
+  const unsigned m0_a = __builtin_amdgcn_readfirstlane((unsigned)(size_t)(__attribute__((address_space(3))) unsigned short*)&lds_a[0][0] + (unsigned)wave * 1024u);
+  const unsigned m0_w = __builtin_amdgcn_readfirstlane((unsigned)(size_t)(__attribute__((address_space(3))) unsigned short*)&lds_w[0][0] + (unsigned)wave * 1024u);
+  unsigned w_offs[kPassW];
+#pragma unroll
+  for (int j = 0; j < kPassW; ++j) w_offs[j] = w_off + (unsigned)(64 * j) * (unsigned)p.K * 2u;
+  auto dma_one = [&](int ks, int stage, int j) {
+    const char* base = (j < kPassA ? a_base : w_base) + (size_t)ks * (kKS * 2);
+    const unsigned voff = j < kPassA ? a_off[j < kPassA ? j : 0] : w_offs[j < kPassA ? 0 : j - kPassA];
+    const unsigned m0v = j < kPassA ? m0_a + (unsigned)(stage * kGM * kKS * 2 + 64 * j * kKS * 2)
+                                    : m0_w + (unsigned)(stage * TN * kKS * 2 + 64 * (j - kPassA) * kKS * 2);
+    asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1" : : "v"(voff), "s"(base), "s"(m0v) : "memory", "m0");
+  };
   // loads of this wavefront still allowed in flight: N (vmcnt(N); expcnt and lgkmcnt untouched)
   constexpr int kDmaPerStep = kPassA + kPassW;
 #define LBM_DMA_WAIT(N) __builtin_amdgcn_s_waitcnt(0x0F70 | ((N) & 15) | (((N) >> 4) << 14))
@@ -232,32 +265,34 @@ __global__ __launch_bounds__(kGThreads, 1) void lbm_linear_bf16_kernel(LinearArg
 #pragma unroll
       for (int i = 0; i < 16; ++i) acc[a][b][i] = 0.f;
 
-  // One 64-wide step on stage `stage`: each wave group multiplies its 32-wide half, the fragments
-  // of the second 16-wide slice read while the MFMAs of the first run.
+  // One 64-wide step: each wave group multiplies its 32-wide half.  The fragments of a step are
+  // read during the step before it, one read in between two MFMAs (a burst of reads fills the LDS
+  // queue and holds the MFMAs behind it back), into the other half of the fragment registers.
   const int sw_r = (n32 >> 1) & 7;
-  auto step = [&](int stage) {
+  bf16x8 wf[2][2][NT], af[2][2][2];   // [step parity][16-wide slice][block]
+  auto read_one = [&](int stage, int buf, int i) {   // read i of a step's 2 (NT + 2), in the order the MFMAs use them
     const unsigned short* la = &lds_a[stage][0];
     const unsigned short* lw = &lds_w[stage][0];
-    bf16x8 wf[2][NT], af[2][2];
-    auto read = [&](int k16, bf16x8 (&wfr)[NT], bf16x8 (&afr)[2]) {
-      const int pos = ((kh * 4 + k16 * 2 + g) ^ sw_r) * 8;
+    const int k16 = i / (NT + 2), j = i % (NT + 2);
+    const int pos = ((kh * 4 + k16 * 2 + g) ^ sw_r) * 8;
+    if (j == 0) wf[buf][k16][0] = __builtin_bit_cast(bf16x8, *(const u32x4*)&lw[(wn + n32) * kKS + pos]);
+    else if (j <= 2) af[buf][k16][j - 1] = __builtin_bit_cast(bf16x8, *(const u32x4*)&la[(wm + ((j - 1) ^ kh) * 32 + n32) * kKS + pos]);
+    else wf[buf][k16][j - 2] = __builtin_bit_cast(bf16x8, *(const u32x4*)&lw[(wn + (j - 2) * 32 + n32) * kKS + pos]);
+  };
+  auto read_slice = [&](int stage, int buf, int k16) {
 #pragma unroll
-      for (int a = 0; a < NT; ++a)
-        wfr[a] = __builtin_bit_cast(bf16x8, *(const u32x4*)&lw[(wn + a * 32 + n32) * kKS + pos]);
+    for (int i = 0; i < NT + 2; ++i) read_one(stage, buf, k16 * (NT + 2) + i);
+  };
+  auto read_step = [&](int stage, int buf) {
+    read_slice(stage, buf, 0);
+    read_slice(stage, buf, 1);
+  };
+  auto mfma_slice = [&](int buf, int k16) {
+#pragma unroll
+    for (int a = 0; a < NT; ++a)
 #pragma unroll
       for (int b = 0; b < 2; ++b)
-        afr[b] = __builtin_bit_cast(bf16x8, *(const u32x4*)&la[(wm + b * 32 + n32) * kKS + pos]);
-    };
-    read(0, wf[0], af[0]);
-    read(1, wf[1], af[1]);
-#pragma unroll
-    for (int k16 = 0; k16 < 2; ++k16) {
-#pragma unroll
-      for (int a = 0; a < NT; ++a)
-#pragma unroll
-        for (int b = 0; b < 2; ++b)
-          acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wf[k16][a], af[k16][b], acc[a][b], 0, 0, 0);
-    }
+        acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wf[buf][k16][a], af[buf][k16][b], acc[a][b], 0, 0, 0);
   };
 
   // LNA, row statistics: row r of the tile is handled by threads 4 r .. 4 r + 3, each taking every
@@ -273,6 +308,14 @@ __global__ __launch_bounds__(kGThreads, 1) void lbm_linear_bf16_kernel(LinearArg
     for (int i = 0; i < kLnHeld; ++i)
       if ((tid & 3) + 4 * i < p.ln_tiles) ln_part[i] = *(const f32x2*)(ln_st + 2 * ((tid & 3) + 4 * i));
   }
+  // The per-column vectors of the epilogue (bias, column sums of w, LayerScale) are asked for now
+  // and parked in LDS behind the first operand loads; the loop's barriers publish them.
+  float cv_bias = 0.f, cv_sum = 0.f, cv_gamma = 1.f;
+  if (tid < TN) {
+    if (p.bias) cv_bias = p.bias[n0 + tid];
+    if (LNA) cv_sum = p.ln_colsum[n0 + tid];
+    if (EPI == LBM_LINEAR_BIAS_RESIDUAL && p.gamma) cv_gamma = p.gamma[n0 + tid];
+  }
   // The GELU table travels first (480 threads x 16 bytes; the loads return in order, so the wait
   // for the first operand tile covers it and the barrier behind that wait publishes it) ...
   if (EPI == LBM_LINEAR_BIAS_GELU && tid < kGeluEntries / 8)
@@ -281,6 +324,11 @@ __global__ __launch_bounds__(kGThreads, 1) void lbm_linear_bf16_kernel(LinearArg
 #pragma unroll
   for (int i = 0; i < kStagesG - 1; ++i)
     if (i < nk) dma_step(i, i);
+  if (tid < TN) {
+    colvec[0][tid] = cv_bias;
+    colvec[1][tid] = cv_sum;
+    colvec[2][tid] = cv_gamma;
+  }
   if (LNA) {
     const int r = tid >> 2, part = tid & 3;
     float sm = 0.f;
@@ -312,61 +360,54 @@ __global__ __launch_bounds__(kGThreads, 1) void lbm_linear_bf16_kernel(LinearArg
     }
     // (read in the epilogue, many barriers from here)
   }
-  // Step s: wait until its rows have landed (the loads of at most two later steps may still be in
-  // flight), barrier (everyone's rows of step s are there, and everyone is done with step s - 1,
-  // whose stage is the one step s + 3 lands in), ask for step s + 3, multiply step s.
+  // Step 0's fragments: its rows have landed (steps 1 and 2 may still be in flight), barrier, read.
+  if (2 < nk) LBM_DMA_WAIT(2 * kDmaPerStep);
+  else LBM_DMA_WAIT(kDmaPerStep);
+  __syncthreads();
+  read_step(0, 0);
+  if (kStagesG - 1 < nk) dma_step(kStagesG - 1, kStagesG - 1);
+  // Step s: wait until the rows of step s + 1 have landed (the loads of steps s + 2 and s + 3 may
+  // still be in flight), barrier (everyone's rows of step s + 1 are there, and everyone holds the
+  // fragments of step s in registers, so its stage is free), then the MFMAs of step s with the
+  // fragment reads of step s + 1 in between, then the loads of step s + 4 into the freed stage.
+  static_assert(kStagesG == 4, "the loop is written for a ring of four stages");
+#define LBM_SGB(mask, n) __builtin_amdgcn_sched_group_barrier(mask, n, 0)
   for (int s0 = 0; s0 < nk; s0 += kStagesG) {
 #pragma unroll
     for (int st = 0; st < kStagesG; ++st) {
       const int sidx = s0 + st;
       if (sidx < nk) {
-        if (sidx + 2 < nk) LBM_DMA_WAIT(2 * kDmaPerStep);
-        else if (sidx + 1 < nk) LBM_DMA_WAIT(kDmaPerStep);
+        if (sidx + 3 < nk) LBM_DMA_WAIT(2 * kDmaPerStep);
+        else if (sidx + 2 < nk) LBM_DMA_WAIT(kDmaPerStep);
         else LBM_DMA_WAIT(0);
         __syncthreads();
-        if (sidx + kStagesG - 1 < nk) dma_step(sidx + kStagesG - 1, (st + kStagesG - 1) % kStagesG);
-        step(st);
+        __builtin_amdgcn_sched_barrier(0);
+        const bool more = sidx + kStagesG < nk;
+#pragma unroll
+        for (int k16 = 0; k16 < 2; ++k16) {
+          read_slice((st + 1) % kStagesG, (st + 1) & 1, k16);   // (past the last step: stale rows, never used)
+          mfma_slice(st & 1, k16);
+#pragma unroll
+          for (int i = 0; i < NT + 2; ++i) { LBM_SGB(0x008, 1); LBM_SGB(0x100, 1); }
+          __builtin_amdgcn_sched_barrier(0);
+          if (more) {
+#pragma unroll
+            for (int j = 0; j < kDmaPerStep; ++j)
+              if (j * 2 / kDmaPerStep == k16) dma_one(sidx + kStagesG, st, j);
+          }
+        }
       }
     }
   }
+#undef LBM_SGB
   __syncthreads();
 
-  // What the epilogue needs from global memory is asked for here, all at once, and arrives while
-  // the wave groups exchange their sums (asked for where it is used - per column group, per
-  // pass - every load would wait out a trip to L2 or HBM on its own, and behind the stores of
-  // the pass before it; asked for before the multiply, it delays the first operand tiles): the
-  // per-column vectors of this lane's accumulator columns ...
-  f32x4 bias_v[NT][4], colsum_v[NT][4], gamma_v[NT][4];
-#pragma unroll
-  for (int a = 0; a < NT; ++a)
-#pragma unroll
-    for (int c4 = 0; c4 < 4; ++c4) {
-      bias_v[a][c4] = f32x4{0.f, 0.f, 0.f, 0.f};
-      colsum_v[a][c4] = f32x4{0.f, 0.f, 0.f, 0.f};
-      gamma_v[a][c4] = f32x4{1.f, 1.f, 1.f, 1.f};
-    }
-  {
-    const int col0 = n0 + wn + g * 4;     // + a * 32 + c4 * 8: four consecutive output columns
-    if (p.bias) {
-#pragma unroll
-      for (int a = 0; a < NT; ++a)
-#pragma unroll
-        for (int c4 = 0; c4 < 4; ++c4) bias_v[a][c4] = *(const f32x4*)(p.bias + col0 + a * 32 + c4 * 8);
-    }
-    if (LNA) {
-#pragma unroll
-      for (int a = 0; a < NT; ++a)
-#pragma unroll
-        for (int c4 = 0; c4 < 4; ++c4) colsum_v[a][c4] = *(const f32x4*)(p.ln_colsum + col0 + a * 32 + c4 * 8);
-    }
-    if (EPI == LBM_LINEAR_BIAS_RESIDUAL && p.gamma) {
-#pragma unroll
-      for (int a = 0; a < NT; ++a)
-#pragma unroll
-        for (int c4 = 0; c4 < 4; ++c4) gamma_v[a][c4] = *(const f32x4*)(p.gamma + col0 + a * 32 + c4 * 8);
-    }
-  }
-  // ... and the residual rows of the store passes (a workgroup that shares its tile under SPLITK
+  // What the epilogue needs from global memory beyond the per-column vectors is asked for here,
+  // all at once, and arrives while the wave groups exchange their sums (asked for where it is
+  // used - per pass - every load would wait out a trip to L2 or HBM on its own, and behind the
+  // stores of the pass before it; asked for before the multiply, it delays the first operand
+  // tiles):
+  // the residual rows of the store passes (a workgroup that shares its tile under SPLITK
   // asks only once it knows that it is the one to store).
   constexpr int kPieces = TN / 8;                 // 16-byte pieces per row of the tile
   constexpr int kRowsPerPass = kGThreads / kPieces;
@@ -417,24 +458,35 @@ __global__ __launch_bounds__(kGThreads, 1) void lbm_linear_bf16_kernel(LinearArg
   }
   // ---- the two wave groups' sums meet: group 0 finishes row block 0 of every sub-tile, group 1
   // row block 1; each parks the other's half in LDS (the operand buffers are dead)
-  float* xch = (float*)&lds_a[0][0];            // [wave][NT][16][64 lanes] floats
+  float* xch = (float*)&lds_a[0][0];            // [wave][NT][4][64 lanes][4] floats
   static_assert(8 * NT * 16 * 64 * 4 <= (int)sizeof(lds_a), "the exchanged halves fit the activation buffers");
-  // (selects, not indexing by kh: a run-time index would put the accumulators in scratch memory)
+  // (the second wave group reads its activation fragments with the two row blocks swapped, so
+  // for both groups acc[.][0] is the block they finish and acc[.][1] the one they hand over)
   f32x16 fin[NT];
   {
 #pragma unroll
     for (int a = 0; a < NT; ++a)
 #pragma unroll
-      for (int i = 0; i < 16; ++i) {
-        xch[((wave * NT + a) * 16 + i) * 64 + lane] = kh ? acc[a][0][i] : acc[a][1][i];
-        fin[a][i] = kh ? acc[a][1][i] : acc[a][0][i];
+      for (int q = 0; q < 4; ++q) {
+        f32x4 give;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          give[e] = acc[a][1][q * 4 + e];
+          fin[a][q * 4 + e] = acc[a][0][q * 4 + e];
+        }
+        *(f32x4*)&xch[(((wave * NT + a) * 4 + q) * 64 + lane) * 4] = give;
       }
-    __syncthreads();
+    // (a barrier that waits for the LDS writes only: the loads asked for above stay in flight)
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
     const int peer = wave ^ 4;
 #pragma unroll
     for (int a = 0; a < NT; ++a)
 #pragma unroll
-      for (int i = 0; i < 16; ++i) fin[a][i] += xch[((peer * NT + a) * 16 + i) * 64 + lane];
+      for (int q = 0; q < 4; ++q) {
+        const f32x4 got = *(const f32x4*)&xch[(((peer * NT + a) * 4 + q) * 64 + lane) * 4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) fin[a][q * 4 + e] += got[e];
+      }
   }
   const int b = kh;     // the row block this wave finishes
   if (SPLITK) {
@@ -495,7 +547,7 @@ __global__ __launch_bounds__(kGThreads, 1) void lbm_linear_bf16_kernel(LinearArg
 #pragma unroll
     for (int c4 = 0; c4 < 4; ++c4) {
       const int col = wn + a * 32 + c4 * 8 + g * 4;     // four consecutive output columns
-      const f32x4 bias4 = bias_v[a][c4], gamma4 = gamma_v[a][c4], colsum4 = colsum_v[a][c4];
+      const f32x4 bias4 = *(const f32x4*)&colvec[0][col], colsum4 = *(const f32x4*)&colvec[1][col], gamma4 = *(const f32x4*)&colvec[2][col];
       f32x4 y;
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
@@ -599,9 +651,8 @@ __global__ __launch_bounds__(kGThreads, 1) void lbm_linear_bf16_kernel(LinearArg
 // Eight wavefronts, each on 64 rows x 128 columns of the tile (96 x 64 of a 192-row tile) over
 // the whole K slice, no K split inside the workgroup and so no exchange at the end.  Two LDS
 // stages: a 64-wide step is 24-32 MFMAs per wavefront, longer than a trip to memory, so one step
-// of prefetch is enough; the loads of the next step are issued in between the MFMAs of the
-// current one's first three quarters rather than in one burst (they share the LDS with the
-// fragment reads).  Same operand path (global -> LDS directly, swizzled 16-byte chunks), same
+// of prefetch is enough; the loads of a step are issued at the end of the step before the one
+// they replace, right behind the barrier that frees its stage.  Same operand path (global -> LDS directly, swizzled 16-byte chunks), same
 // epilogue arithmetic and rounding sequence.  Epilogues: bias, bias + GELU, and the
 // pre-attention producer; the folded LayerNorm of the activations; not the residual forms (their
 // 1,024 columns make too few such tiles).  The per-column vectors wait in LDS instead of
@@ -630,14 +681,7 @@ __global__ __launch_bounds__(kGThreads, 1) void lbm_linear_bf16_big_kernel(Linea
   const int rg = wave % kRowGroups, cg = wave / kRowGroups;
   const int wm = rg * (RB * 32), wn = cg * (CB * 32);       // this wavefront's corner of the tile
   int mt, nt;
-  if ((p.n_tiles & 7) == 0) {   // an XCD keeps its own column tiles of w and walks the row tiles with them
-    const int x = blockIdx.x & 7, i = blockIdx.x >> 3;
-    mt = i % p.m_tiles;
-    nt = (i / p.m_tiles) * 8 + x;
-  } else {
-    mt = (int)blockIdx.x % p.m_tiles;
-    nt = (int)blockIdx.x / p.m_tiles;
-  }
+  lbm_tile_of_workgroup((int)blockIdx.x, p.m_tiles, p.n_tiles, mt, nt);
   const int m0 = mt * BM, n0 = nt * kBN;
 
   // ---- staging (as in the kernel above: eight 128-byte rows per wavefront and load)
@@ -729,37 +773,83 @@ __global__ __launch_bounds__(kGThreads, 1) void lbm_linear_bf16_big_kernel(Linea
       for (int i = 0; i < 16; ++i) acc[a][b][i] = 0.f;
 
   const int sw_r = (n32 >> 1) & 7;
-  for (int s = 0; s < nk; ++s) {
-    LBM_DMA_WAIT(0);
-    __syncthreads();   // step s has landed everywhere, and everyone is done with step s - 1, whose stage step s + 1 lands in
-    const unsigned short* la = (const unsigned short*)(lds_raw + (s & 1) * kStageBytes);
-    const unsigned short* lw = la + BM * kKS;
-    bf16x8 wf[2][CB], af[2][RB];
-    auto read = [&](int kq, bf16x8 (&wfr)[CB], bf16x8 (&afr)[RB]) {
-      const int pos = ((kq * 2 + g) ^ sw_r) * 8;
+  // M0 values as integers (no pointer cast inside the loop): this wavefront's KB of every block of 64 rows
+  const unsigned m0_wave = __builtin_amdgcn_readfirstlane((unsigned)(size_t)(__attribute__((address_space(3))) unsigned char*)lds_raw + (unsigned)wave * 1024u);
+  unsigned w_offs[kPassW];
 #pragma unroll
-      for (int a = 0; a < CB; ++a)
-        wfr[a] = __builtin_bit_cast(bf16x8, *(const u32x4*)&lw[(wn + a * 32 + n32) * kKS + pos]);
+  for (int j = 0; j < kPassW; ++j) w_offs[j] = w_off + (unsigned)(64 * j) * (unsigned)p.K * 2u;
+  auto dma_at = [&](const char* base, unsigned voff, unsigned m0v) {
+    asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1" : : "v"(voff), "s"(base), "s"(m0v) : "memory", "m0");
+  };
+  auto dma_step = [&](int ks, unsigned stage_bytes) {
+    const char* ab = a_base + (size_t)ks * (kKS * 2);
+    const char* wb = w_base + (size_t)ks * (kKS * 2);
+#pragma unroll
+    for (int j = 0; j < kPassA; ++j) dma_at(ab, a_off[j], m0_wave + stage_bytes + (unsigned)(64 * j * kKS * 2));
+#pragma unroll
+    for (int j = 0; j < kPassW; ++j) dma_at(wb, w_offs[j], m0_wave + stage_bytes + (unsigned)((BM + 64 * j) * kKS * 2));
+  };
+  bf16x8 wf[2][CB], af[2][RB];
+  auto read = [&](unsigned stage_bytes, int kq, bf16x8 (&wfr)[CB], bf16x8 (&afr)[RB]) {
+    const unsigned char* la = lds_raw + stage_bytes;
+    const unsigned char* lw = la + BM * kKS * 2;
+    const int posb = ((kq * 2 + g) ^ sw_r) * 16;
+#pragma unroll
+    for (int a = 0; a < CB; ++a)
+      wfr[a] = __builtin_bit_cast(bf16x8, *(const u32x4*)(lw + (wn + a * 32 + n32) * (kKS * 2) + posb));
+#pragma unroll
+    for (int b = 0; b < RB; ++b)
+      afr[b] = __builtin_bit_cast(bf16x8, *(const u32x4*)(la + (wm + b * 32 + n32) * (kKS * 2) + posb));
+  };
+  auto mfmas = [&](int kq, int from, int to) {
+#pragma unroll
+    for (int a = 0; a < CB; ++a)
 #pragma unroll
       for (int b = 0; b < RB; ++b)
-        afr[b] = __builtin_bit_cast(bf16x8, *(const u32x4*)&la[(wm + b * 32 + n32) * kKS + pos]);
-    };
-    read(0, wf[0], af[0]);
-#pragma unroll
-    for (int kq = 0; kq < 4; ++kq) {
-      if (kq < 3) read(kq + 1, wf[(kq + 1) & 1], af[(kq + 1) & 1]);
-      if (s + 1 < nk) {
-#pragma unroll
-        for (int j = 0; j < kDma; ++j)
-          if (j * 3 / kDma == kq) dma_one(s + 1, (s + 1) & 1, j);   // a third of the next step's loads per quarter step
-      }
-#pragma unroll
-      for (int a = 0; a < CB; ++a)
-#pragma unroll
-        for (int b = 0; b < RB; ++b)
+        if (a * RB + b >= from && a * RB + b < to)
           acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wf[kq & 1][a], af[kq & 1][b], acc[a][b], 0, 0, 0);
+  };
+#define LBM_SGB(mask, n) __builtin_amdgcn_sched_group_barrier(mask, n, 0)
+  // One 64-wide step on the stage at byte `here`.  The fragment reads of a quarter step are
+  // issued one by one in between the MFMAs of the quarter before it (a burst of them fills the
+  // LDS queue and stalls the wavefront's MFMAs behind it).  The barrier that hands the other
+  // stage over sits in the middle of the last quarter: behind it come the first fragment reads
+  // of the next step, covered by the quarter's remaining MFMAs, and at the end of the step the
+  // loads of the step after the next one, which have a whole step to land.
+  constexpr int kQ = CB * RB, kR = CB + RB, kH = kQ / 2;
+  auto step = [&](int s, auto stage_c) {
+    constexpr unsigned here = decltype(stage_c)::value * kStageBytes, there = kStageBytes - here;
+#pragma unroll
+    for (int kq = 0; kq < 3; ++kq) {
+      read(here, kq + 1, wf[(kq + 1) & 1], af[(kq + 1) & 1]);
+      mfmas(kq, 0, kQ);
+#pragma unroll
+      for (int i = 0; i < kR; ++i) { LBM_SGB(0x008, 1); LBM_SGB(0x100, 1); }
+      LBM_SGB(0x008, kQ - kR);
+      __builtin_amdgcn_sched_barrier(0);
     }
+    mfmas(3, 0, kH);
+    __builtin_amdgcn_sched_barrier(0);
+    LBM_DMA_WAIT(0);
+    __syncthreads();   // the other stage has landed everywhere, and everyone has read all of this one
+    __builtin_amdgcn_sched_barrier(0);
+    read(there, 0, wf[0], af[0]);
+    mfmas(3, kH, kQ);
+    LBM_SGB(0x100, kR - (kQ - kH) + 1 > 0 ? kR - (kQ - kH) + 1 : 0);
+#pragma unroll
+    for (int i = 0; i < kQ - kH; ++i) { LBM_SGB(0x008, 1); LBM_SGB(0x100, 1); }
+    __builtin_amdgcn_sched_barrier(0);
+    if (s + 2 < nk) dma_step(s + 2, here);
+  };
+  LBM_DMA_WAIT(0);
+  __syncthreads();
+  dma_step(1, kStageBytes);
+  read(0, 0, wf[0], af[0]);
+  for (int s = 0; s < nk; s += 2) {
+    step(s, std::integral_constant<unsigned, 0>{});
+    step(s + 1, std::integral_constant<unsigned, 1>{});
   }
+#undef LBM_SGB
 
   // ---- epilogue.  What the producer's first passes need from global memory is asked for now and
   // arrives while the tile is staged.
