@@ -1613,9 +1613,14 @@ constexpr double kTileUs = 1.95;      // one 64-token tile iteration of a workgr
 constexpr double kWgTiles = 3.0;      // prologue + epilogue of a workgroup, in tile iterations
 constexpr double kCombineUs = 2.5;    // launch + latency of the combine kernel
 constexpr double kCombineBytesPerUs = 5.0e6;
+// the short-KV kernel (one workgroup per 64 query rows and head, no partial results)
+constexpr double kSmLaunchUs = 1.8;   // launch to first instruction
+constexpr double kSmWgUs = 4.0;       // a workgroup's fixed part: Q rows, range check, merge through LDS, store
+constexpr double kSmTileUs = 0.3625;  // per 64-token tile: 1.45 us per step of eight 32-token pieces
 
 struct ScheduleKey {
   int n_streams = -1, num_heads = 0;
+  bool small = false;
   int q_rows[LBM_MAX_STREAMS], n_tiles[LBM_MAX_STREAMS];
   int order[LBM_MAX_STREAMS], n_splits[LBM_MAX_STREAMS];
 };
@@ -1681,11 +1686,60 @@ void lbm_attn_schedule(const lbm_attn_stream* streams, int n_streams, int num_he
     work += (long long)qt[i] * num_heads * nt[i];
     if (nt[i] > max_nt) max_nt = nt[i];
   }
-  // short KV everywhere: the in-workgroup split kernel, one workgroup per (64 query rows, head),
-  // no partial results
-  bool small = n_streams > 0;
-  for (int i = 0; i < n_streams; ++i) small = small && streams[i].kv_tokens <= kSmMaxKv;
-  if (small) {
+  // Short KV everywhere: the in-workgroup split kernel (one workgroup per 64 query rows and head,
+  // no partial results) is a candidate, priced against the split-KV plan: it wins on one frame's
+  // 1,004 x 1,004 (256 workgroups of 16 tiles: 12 us against 19), the split-KV pair wins once
+  // several streams would take the CUs four rounds of such workgroups (31 against 43 us).
+  bool small_ok = n_streams > 0;
+  for (int i = 0; i < n_streams; ++i) small_ok = small_ok && streams[i].kv_tokens <= kSmMaxKv;
+  ScheduleKey& memo = g_last_schedule;
+  bool hit = memo.n_streams == n_streams && memo.num_heads == num_heads;
+  for (int i = 0; hit && i < n_streams; ++i) hit = memo.q_rows[i] == q_rows[i] && memo.n_tiles[i] == nt[i];
+  if (!hit) {
+    int best_splits[LBM_MAX_STREAMS], cand_splits[LBM_MAX_STREAMS];
+    double best = -1.0;
+    auto consider = [&](long long tps) {
+      if (tps < 2) tps = 2;
+      if (tps > max_nt) tps = max_nt > 0 ? max_nt : 1;
+      const double c = price_candidate(qt, nt, n_streams, num_heads, (int)tps, q_rows, cand_splits);
+      if (best < 0 || c < best) {
+        best = c;
+        for (int i = 0; i < n_streams; ++i) best_splits[i] = cand_splits[i];
+      }
+    };
+    // the longest stream cut into 1..12 pieces, and the total work spread over 1..3 rounds of 256
+    for (int k = 1; k <= 12; ++k) consider((max_nt + k - 1) / k);
+    for (int k = 1; k <= 3; ++k) consider((work + 256LL * k - 1) / (256LL * k));
+    memo.small = false;
+    if (small_ok) {
+      double longest = 0.0, total = 0.0;
+      for (int i = 0; i < n_streams; ++i) {
+        const double dur = kSmWgUs + kSmTileUs * (nt[i] > 0 ? nt[i] : 1);
+        const double wgs = (double)((q_rows[i] + kQPerWave - 1) / kQPerWave) * num_heads;
+        if (wgs > 0 && dur > longest) longest = dur;
+        total += wgs * dur;
+      }
+      const double small_price = kSmLaunchUs + (total / 256.0 > longest ? total / 256.0 : longest);
+      // (the short-KV kernel unless the pair is clearly ahead: it merges its partial results in
+      // fp32 inside the workgroup, the pair rounds them to bf16 on their way through memory)
+      memo.small = best < 0 || 0.85 * small_price <= best;
+    }
+    memo.n_streams = n_streams;
+    memo.num_heads = num_heads;
+    int tiles[LBM_MAX_STREAMS];
+    for (int i = 0; i < n_streams; ++i) {
+      memo.q_rows[i] = q_rows[i];
+      memo.n_tiles[i] = nt[i];
+      memo.n_splits[i] = best_splits[i];
+      memo.order[i] = i;
+      tiles[i] = nt[i] > 0 ? (nt[i] + best_splits[i] - 1) / best_splits[i] : 0;
+    }
+    for (int i = 1; i < n_streams; ++i)
+      for (int j = i; j > 0 && tiles[memo.order[j]] > tiles[memo.order[j - 1]]; --j) {
+        int t = memo.order[j]; memo.order[j] = memo.order[j - 1]; memo.order[j - 1] = t;
+      }
+  }
+  if (memo.small) {
     sch.small = 1;
     int wg = 0;
     for (int i = 0; i < n_streams; ++i) {
@@ -1708,39 +1762,6 @@ void lbm_attn_schedule(const lbm_attn_stream* streams, int n_streams, int num_he
     sch.total_wgs = wg;
     sch.part_rows = 0;
     return;
-  }
-  ScheduleKey& memo = g_last_schedule;
-  bool hit = memo.n_streams == n_streams && memo.num_heads == num_heads;
-  for (int i = 0; hit && i < n_streams; ++i) hit = memo.q_rows[i] == q_rows[i] && memo.n_tiles[i] == nt[i];
-  if (!hit) {
-    int best_splits[LBM_MAX_STREAMS], cand_splits[LBM_MAX_STREAMS];
-    double best = -1.0;
-    auto consider = [&](long long tps) {
-      if (tps < 2) tps = 2;
-      if (tps > max_nt) tps = max_nt > 0 ? max_nt : 1;
-      const double c = price_candidate(qt, nt, n_streams, num_heads, (int)tps, q_rows, cand_splits);
-      if (best < 0 || c < best) {
-        best = c;
-        for (int i = 0; i < n_streams; ++i) best_splits[i] = cand_splits[i];
-      }
-    };
-    // the longest stream cut into 1..12 pieces, and the total work spread over 1..3 rounds of 256
-    for (int k = 1; k <= 12; ++k) consider((max_nt + k - 1) / k);
-    for (int k = 1; k <= 3; ++k) consider((work + 256LL * k - 1) / (256LL * k));
-    memo.n_streams = n_streams;
-    memo.num_heads = num_heads;
-    int tiles[LBM_MAX_STREAMS];
-    for (int i = 0; i < n_streams; ++i) {
-      memo.q_rows[i] = q_rows[i];
-      memo.n_tiles[i] = nt[i];
-      memo.n_splits[i] = best_splits[i];
-      memo.order[i] = i;
-      tiles[i] = nt[i] > 0 ? (nt[i] + best_splits[i] - 1) / best_splits[i] : 0;
-    }
-    for (int i = 1; i < n_streams; ++i)
-      for (int j = i; j > 0 && tiles[memo.order[j]] > tiles[memo.order[j - 1]]; --j) {
-        int t = memo.order[j]; memo.order[j] = memo.order[j - 1]; memo.order[j - 1] = t;
-      }
   }
   int wg = 0;
   long long part = 0;
