@@ -204,3 +204,24 @@ def test_config5_four_ragged_streams_in_one_launch():
         kk, vv = gather_paged(pool, ids[indptr[b]:indptr[b + 1]], lens[indptr[b]:indptr[b + 1]])
         assert kk.shape[0] == kv_tokens[b]
         check(out[b * T:(b + 1) * T], sdpa_nhd(q[b * T:(b + 1) * T], kk, vv), f"stream {b}: {kv_tokens[b]} tokens")
+
+
+@pytest.mark.parametrize("n_streams", [1, 2, 4])
+def test_frame_blocks_of_several_streams_at_full_size(n_streams):
+    """The frame and encoder blocks' cache-less attention (``dense_attention``: 1004 x 1004 per
+    stream, 16 heads) for one, two and four streams in one launch.  The schedule prices the
+    short-KV kernel against the split-KV pair: one and two streams take the short-KV kernel (no
+    workspace), four streams - four rounds of the CUs on the short-KV kernel - take the pair.
+    Either way every stream must match the oracle's SDPA on its own tokens."""
+    from lingbot_map_amd import _native as N, dense_attention
+    from oracle.sdpa_cache import sdpa_nhd
+    dev = torch.device("cuda:0")
+    g = torch.Generator().manual_seed(20 + n_streams)
+    q, k, v = (torch.randn(n_streams * T, H, D, generator=g).to(torch.bfloat16) for _ in range(3))
+    streams = (N.AttnStream * n_streams)(*[N.AttnStream(s * T, T, s * T, T) for s in range(n_streams)])
+    need = int(N.lib.lbm_attn_workspace_bytes(streams, n_streams, H, D))
+    assert (need > 0) == (n_streams == 4), (n_streams, need)
+    out = dense_attention(q.to(dev), k.to(dev), v.to(dev), num_streams=n_streams).cpu()
+    for s in range(n_streams):
+        sl = slice(s * T, (s + 1) * T)
+        check(out[sl], sdpa_nhd(q[sl], k[sl], v[sl]), f"stream {s} of {n_streams}")
