@@ -70,6 +70,20 @@ def test_linear_bias(M, K, Nn):
     check(run_linear(a, w, None, N.LINEAR_BIAS), expected(a, w, None, N.LINEAR_BIAS))
 
 
+def test_linear_tile_counts_that_do_not_fill_rounds_of_the_cus():
+    """Workgroups take tiles in blocks of 4 x 8 per XCD and in rounds of 256; shapes whose tile
+    counts are not multiples of 8, 32 or 256 - one tile, a last panel narrower than 8 column tiles,
+    a last round that does not give every XCD the same number of tiles, more than one round - must
+    still have every tile computed exactly once.  K from the shortest loop (two 64-wide steps) up;
+    both tile widths and both kernels (the last three shapes run on the 256- and 192-row tiles)."""
+    N = _native()
+    for M, K, Nn in [(1, 128, 64), (130, 128, 576), (700, 128, 1152), (1100, 256, 1344), (2300, 128, 2240), (5000, 128, 832),
+                     (390, 384, 4288), (4500, 128, 5120), (9000, 128, 4352), (6100, 256, 3328)]:
+        a, w, bias, _ = _inputs(M, K, Nn, seed=M + Nn)
+        got = run_linear(a, w, bias, N.LINEAR_BIAS)
+        check(got, expected(a, w, bias, N.LINEAR_BIAS))
+
+
 def test_gelu_epilogue_on_every_bf16_pre_activation():
     """One-hot activations make the pre-activation of output (i, n) the weight w[n, i] itself, so
     a 512 x 128 weight matrix puts every finite bf16 bit pattern through the epilogue: the
