@@ -573,13 +573,16 @@ __global__ __launch_bounds__(kGThreads, 1) void lbm_linear_bf16_kernel(LinearArg
       const bool valid = m0 + r < p.M;            // rows past M computed on the last token's entries, never stored
       const u32x2 lo = *(const u32x2*)&stage[r * kCStride + pq.c], hi = *(const u32x2*)&stage[r * kCStride + pq.c + 4];
       const u32x4 raw = {lo[0], lo[1], hi[0], hi[1]};
-      float x[8];
+      bf16x8 o8 = __builtin_bit_cast(bf16x8, raw);   // v rows leave as they are
+      if (pq.which < 2) {
+        // q and k rows: the row's last rounding is the conversion that packs it
+        float x[8];
 #pragma unroll
-      for (int i = 0; i < 8; ++i) x[i] = __builtin_bit_cast(float, (i & 1) ? (raw[i >> 1] & 0xffff0000u) : (raw[i >> 1] << 16));
-      if (pq.which < 2) lbm_qkv::norm_rope<0, ROPE, NORM>(x, pq.w4, pq.b4, pq.cs4[j], pq.c8, p.eps, pq.which == 0 ? p.q_scale : 1.0f);
-      bf16x8 o8;
+        for (int i = 0; i < 8; ++i) x[i] = __builtin_bit_cast(float, (i & 1) ? (raw[i >> 1] & 0xffff0000u) : (raw[i >> 1] << 16));
+        lbm_qkv::norm_rope_unrounded<0, ROPE, NORM>(x, pq.w4, pq.b4, pq.cs4[j], pq.c8, p.eps, pq.which == 0 ? p.q_scale : 1.0f);
 #pragma unroll
-      for (int i = 0; i < 8; ++i) o8[i] = (__bf16)x[i];
+        for (int i = 0; i < 8; ++i) o8[i] = (__bf16)x[i];
+      }
       if (valid) {
         const long long nhd = ((long long)(m0 + r) * H + pq.h) * 64 + pq.c8 * 8;
         if (dst_plain) *(bf16x8*)(dst_plain + nhd) = o8;
@@ -930,13 +933,16 @@ __global__ __launch_bounds__(kGThreads, 1) void lbm_linear_bf16_big_kernel(Linea
         const bool valid = m0 + r < p.M;
         const u32x2 lo = *(const u32x2*)&stage[r * kBCStride + pc], hi = *(const u32x2*)&stage[r * kBCStride + pc + 4];
         const u32x4 raw = {lo[0], lo[1], hi[0], hi[1]};
-        float x[8];
+        bf16x8 o8 = __builtin_bit_cast(bf16x8, raw);   // v rows leave as they are
+        if (which < 2) {
+          // q and k rows: the row's last rounding is the conversion that packs it
+          float x[8];
 #pragma unroll
-        for (int i = 0; i < 8; ++i) x[i] = __builtin_bit_cast(float, (i & 1) ? (raw[i >> 1] & 0xffff0000u) : (raw[i >> 1] << 16));
-        if (which < 2) lbm_qkv::norm_rope<0, ROPE, NORM>(x, w4, b4, cs[j], c8, p.eps, post);
-        bf16x8 o8;
+          for (int i = 0; i < 8; ++i) x[i] = __builtin_bit_cast(float, (i & 1) ? (raw[i >> 1] & 0xffff0000u) : (raw[i >> 1] << 16));
+          lbm_qkv::norm_rope_unrounded<0, ROPE, NORM>(x, w4, b4, cs[j], c8, p.eps, post);
 #pragma unroll
-        for (int i = 0; i < 8; ++i) o8[i] = (__bf16)x[i];
+          for (int i = 0; i < 8; ++i) o8[i] = (__bf16)x[i];
+        }
         if (valid) {
           const long long nhd = ((long long)(m0 + r) * H + ph) * 64 + c8 * 8;
           if (dst_plain) *(bf16x8*)(dst_plain + nhd) = o8;

@@ -59,6 +59,16 @@ __device__ __forceinline__ float sum_of_wave(float s) {
   return (r0 + r1) + (r2 + r3);
 }
 
+// two fp32 values rounded to bf16 and back by ONE conversion (v_cvt_pk_bf16_f32 takes a pair) and
+// two bit operations, where round_bf16 on each would take a conversion and a shift apiece
+__device__ __forceinline__ void round_bf16_pair(float a, float b, float& ra, float& rb) {
+  typedef __attribute__((ext_vector_type(2))) float f32x2;
+  typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
+  const unsigned pk = __builtin_bit_cast(unsigned, __builtin_convertvector(f32x2{a, b}, bf16x2));
+  ra = __builtin_bit_cast(float, pk << 16);
+  rb = __builtin_bit_cast(float, pk & 0xffff0000u);
+}
+
 // x: this lane's elements 8 c .. 8 c + 7 of the row (c = lane % 8; the row's 8 lanes are
 // consecutive and aligned, so the shuffles below stay inside it).  SRC 0: bf16 activations
 // (roundings after the LayerNorm, of cos and sin, and after every product and sum), 1: fp32.
@@ -68,13 +78,15 @@ __device__ __forceinline__ float sum_of_wave(float s) {
 // post: a factor the row is multiplied by in fp32 BEFORE the rounding that ends its last
 // operation (the rotary sum, else the LayerNorm, else the plain copy), so that a scaled q row
 // is rounded once; 1.0f leaves every result as it was (x * 1.0f is exact).
+// norm_rope_unrounded leaves that last rounding of a bf16 row (SRC 0) to the caller, who makes it
+// with the conversion that packs the row for its store; every rounding before it is made here.
 template <int SRC, int ROPE, bool NORM>
-__device__ __forceinline__ void norm_rope(float (&x)[8], const f32x4 (&w4)[2], const f32x4 (&b4)[2],
-                                          const f32x4 (&cs4)[4], int c, float eps, float post = 1.0f) {
+__device__ __forceinline__ void norm_rope_unrounded(float (&x)[8], const f32x4 (&w4)[2], const f32x4 (&b4)[2],
+                                                    const f32x4 (&cs4)[4], int c, float eps, float post = 1.0f) {
   const float post_norm = ROPE == 0 ? post : 1.0f;
   if (!NORM && ROPE == 0) {
 #pragma unroll
-    for (int i = 0; i < 8; ++i) x[i] = SRC == 0 ? round_bf16(mul_rn(x[i], post)) : mul_rn(x[i], post);
+    for (int i = 0; i < 8; ++i) x[i] = mul_rn(x[i], post);
   }
   if (NORM) {
     float s = 0.f;
@@ -88,9 +100,11 @@ __device__ __forceinline__ void norm_rope(float (&x)[8], const f32x4 (&w4)[2], c
     v = sum_of_8(v);
     const float rstd = __builtin_amdgcn_rsqf(v * (1.0f / 64.0f) + eps);  // torch's LayerNorm uses rsqrt too
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      const float y = mul_rn(add_rn(mul_rn(mul_rn(x[i] - mean, rstd), w4[i >> 2][i & 3]), b4[i >> 2][i & 3]), post_norm);
-      x[i] = SRC == 0 ? round_bf16(y) : y;
+    for (int i = 0; i < 8; ++i)
+      x[i] = mul_rn(add_rn(mul_rn(mul_rn(x[i] - mean, rstd), w4[i >> 2][i & 3]), b4[i >> 2][i & 3]), post_norm);
+    if (SRC == 0 && ROPE != 0) {
+#pragma unroll
+      for (int i = 0; i < 8; i += 2) round_bf16_pair(x[i], x[i + 1], x[i], x[i + 1]);
     }
   }
   if (ROPE == 1) {
@@ -103,10 +117,12 @@ __device__ __forceinline__ void norm_rope(float (&x)[8], const f32x4 (&w4)[2], c
         float co = q4[2 * j], si = q4[2 * j + 1];
         const float x1 = x[i], x2 = x[i + 1];
         if (SRC == 0) {
-          co = round_bf16(co);
-          si = round_bf16(si);
-          x[i] = round_bf16(mul_rn(sub_rn(round_bf16(mul_rn(x1, co)), round_bf16(mul_rn(x2, si))), post));
-          x[i + 1] = round_bf16(mul_rn(add_rn(round_bf16(mul_rn(x1, si)), round_bf16(mul_rn(x2, co))), post));
+          round_bf16_pair(co, si, co, si);
+          float cc, ss, sc, cs;
+          round_bf16_pair(mul_rn(x1, co), mul_rn(x2, si), cc, ss);
+          round_bf16_pair(mul_rn(x1, si), mul_rn(x2, co), sc, cs);
+          x[i] = mul_rn(sub_rn(cc, ss), post);
+          x[i + 1] = mul_rn(add_rn(sc, cs), post);
         } else {
           x[i] = mul_rn(sub_rn(mul_rn(x1, co), mul_rn(x2, si)), post);
           x[i + 1] = mul_rn(add_rn(mul_rn(x1, si), mul_rn(x2, co)), post);
@@ -116,8 +132,9 @@ __device__ __forceinline__ void norm_rope(float (&x)[8], const f32x4 (&w4)[2], c
   } else if (ROPE != 0) {
     // half-split pairs: in each 32-element half, element j < 16 rotates with element j + 16
     // (x * cos + rotate(x) * sin with rotate = (-second, first), rope.py:123-152); the partner
-    // sits two lanes away in the 8-lane group
-    const bool first = (c & 2) == 0;
+    // sits two lanes away in the 8-lane group.  a - b is a + (-b) bit for bit, so the lanes of
+    // the first 16 flip the sign of the second product instead of choosing between two results.
+    const unsigned flip = (c & 2) == 0 ? 0x80000000u : 0u;
 #pragma unroll
     for (int p = 0; p < 4; ++p) {
       const f32x4 q4 = cs4[p];  // (cos, sin) of two elements
@@ -127,17 +144,28 @@ __device__ __forceinline__ void norm_rope(float (&x)[8], const f32x4 (&w4)[2], c
         float co = q4[2 * j], si = q4[2 * j + 1];
         const float own = x[i];
         const float other = lane_xor2(own);
+        float a0, b0;
         if (SRC == 0) {
-          co = round_bf16(co);
-          si = round_bf16(si);
-          const float a0 = round_bf16(mul_rn(own, co)), b0 = round_bf16(mul_rn(other, si));
-          x[i] = round_bf16(mul_rn(first ? sub_rn(a0, b0) : add_rn(a0, b0), post));
+          round_bf16_pair(co, si, co, si);
+          round_bf16_pair(mul_rn(own, co), mul_rn(other, si), a0, b0);
         } else {
-          const float a0 = mul_rn(own, co), b0 = mul_rn(other, si);
-          x[i] = mul_rn(first ? sub_rn(a0, b0) : add_rn(a0, b0), post);
+          a0 = mul_rn(own, co), b0 = mul_rn(other, si);
         }
+        b0 = __builtin_bit_cast(float, __builtin_bit_cast(unsigned, b0) ^ flip);
+        x[i] = mul_rn(add_rn(a0, b0), post);
       }
     }
+  }
+}
+
+// the same with the last rounding of a bf16 row made here: x holds bf16 values as fp32
+template <int SRC, int ROPE, bool NORM>
+__device__ __forceinline__ void norm_rope(float (&x)[8], const f32x4 (&w4)[2], const f32x4 (&b4)[2],
+                                          const f32x4 (&cs4)[4], int c, float eps, float post = 1.0f) {
+  norm_rope_unrounded<SRC, ROPE, NORM>(x, w4, b4, cs4, c, eps, post);
+  if (SRC == 0) {
+#pragma unroll
+    for (int i = 0; i < 8; i += 2) round_bf16_pair(x[i], x[i + 1], x[i], x[i + 1]);
   }
 }
 
