@@ -7,7 +7,7 @@
 if it has not been built: there is no CPU path.
 """
 from . import _native  # noqa: F401  (loads the library, fails loudly when missing)
-from .aggregator import GraphedAggregator, HipAggregatorStream, PatchConv, PatchTrunk
+from .aggregator import GraphedAggregator, HipAggregatorStream, PatchConv, PatchTrunk, PipelinedAggregator
 from .block import (HipPagedAttention, HipPagedBlock, PositionGetter, RotaryPositionEmbedding2D,
                     RotaryPositionEmbedding3D, WanRotaryPosEmbed, keyframe_flags, set_skip_append)
 from .dense import dense_attention
@@ -16,4 +16,4 @@ from .manager import HipPagedKVCacheManager
 
 __all__ = ["HipAggregatorStream", "PatchConv", "PatchTrunk", "HipPagedKVCacheManager", "HipPagedAttention", "HipPagedBlock", "RotaryPositionEmbedding2D",
            "RotaryPositionEmbedding3D", "WanRotaryPosEmbed", "PositionGetter",
-           "dense_attention", "GraphedFrame", "GraphedStream", "GraphedAggregator", "keyframe_flags", "set_skip_append"]
+           "dense_attention", "GraphedFrame", "GraphedStream", "GraphedAggregator", "PipelinedAggregator", "keyframe_flags", "set_skip_append"]

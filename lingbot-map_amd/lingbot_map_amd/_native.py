@@ -3,6 +3,7 @@
 There is no CPU fallback: importing this module without the built library raises."""
 from __future__ import annotations
 
+import contextlib
 import ctypes as C
 import os
 
@@ -23,6 +24,27 @@ HDR = {"frame_count": 0, "n_anchor": 1, "win_head": 2, "win_count": 3, "n_free_p
        "n_memory_pages": 9, "error": 10, "plan_kv_tokens": 11, "plan_n_pages": 12}
 HDR_WORDS = 16
 ABI_VERSION = 7
+
+
+# Scratch memory that the package keeps per device (the K-split workspace of the GEMM, the
+# workspace of the cache-less attention) serves one chain of launches at a time.  Code that runs a
+# second chain which may overlap the first on the same GPU (another branch of a HIP graph) runs it
+# under ``scratch_lane(1)``: every lane has scratch areas of its own.
+_scratch_lane = 0
+
+
+def current_scratch_lane() -> int:
+    return _scratch_lane
+
+
+@contextlib.contextmanager
+def scratch_lane(lane: int):
+    global _scratch_lane
+    before, _scratch_lane = _scratch_lane, int(lane)
+    try:
+        yield
+    finally:
+        _scratch_lane = before
 
 
 class CacheGeom(C.Structure):

@@ -276,14 +276,20 @@ class HipAggregatorStream(nn.Module):
 
     def forward(self, images: Tensor, selected_idx: Optional[List[int]] = None,
                 num_frame_for_scale: Optional[int] = None, sliding_window_size: Optional[int] = None,
-                num_frame_per_block: int = 1, *, pos3d: Optional[Tensor] = None) -> Tuple[List[Tensor], int]:
+                num_frame_per_block: int = 1, *, pos3d: Optional[Tensor] = None,
+                tokens: Optional[Tensor] = None) -> Tuple[List[Tensor], int]:
         """``images`` ``[streams, S, 3, H, W]`` in [0, 1]; ``S`` is 1 in streaming (more only for
         the anchor pass of a single stream).  Returns the groups' outputs ``[streams, S, P, 2C]``
         (all groups, or those in ``selected_idx``) and the index of the first patch token.
         ``pos3d``: the global blocks' rotary table of this call, for a caller that keeps the frame
-        index itself (graph replay); the stream's frame counter is then left alone."""
+        index itself (graph replay); the stream's frame counter is then left alone.
+        ``tokens``: what ``_embed_images`` returned for these images, ``[streams * S, P, C]``, for
+        a caller that ran the image encoder ahead of time; ``images`` then only gives the sizes."""
         H, W = images.shape[-2:]
-        tokens, B, S, P, C = self._embed_images(images, num_frame_for_scale)
+        if tokens is None:
+            tokens, B, S, P, C = self._embed_images(images, num_frame_for_scale)
+        else:
+            (B, S), (P, C) = images.shape[:2], tokens.shape[-2:]
         pos = self._get_positions(B * S, H, W, images.device)
         manager = self._get_manager(tokens.device, tokens.dtype, P)
         scale_frames = self.num_frame_for_scale if num_frame_for_scale is None else num_frame_for_scale
@@ -382,6 +388,76 @@ class GraphedAggregator:
         assert tuple(images.shape[-2:]) == self._hw, "the graphs were captured for another image size"
         extra = [self._table(images.device)] if self.model.rope3d is not None else []
         out = self.stream(images, *extra, keyframe=keyframe)
+        if keyframe:
+            self.model.total_frames_processed += 1
+        return out
+
+
+class PipelinedAggregator:
+    """Steady-state streaming with one frame of look-ahead.  The image encoder (normalisation,
+    patch convolution, encoder blocks, special tokens: ``_embed_images``) reads nothing of the
+    cache, so the encoder of frame t + 1 does not depend on the frame and global blocks of frame
+    t.  Here the two are branches of one HIP graph on two streams: one frame's kernels leave CUs
+    idle (128 to 192 workgroups of a GEMM on 256 CUs, the gaps between dependent launches) which
+    the other branch's kernels fill.  Results are those of ``GraphedAggregator`` bit for bit; what
+    changes is when an image must be there: a call hands in the NEXT frame's images and returns
+    the outputs of the frame handed in by the call before (``prime`` hands in the first).
+
+    The encoder branch runs under ``scratch_lane(1)``, i.e. on scratch memory of its own.  The cache
+    must be in its steady state, as for ``GraphedAggregator``."""
+
+    def __init__(self, model: HipAggregatorStream, example_images: Tensor,
+                 selected_idx: Optional[List[int]] = None) -> None:
+        from . import _native as N
+        from .graph import GraphedStream
+        if model.kv_cache_manager is None:
+            raise RuntimeError("PipelinedAggregator: stream the anchor and window frames eagerly first")
+        self.model = model
+        self._hw = tuple(example_images.shape[-2:])
+        self._side = torch.cuda.Stream()
+        self._primed = False
+        dev = example_images.device
+        with torch.no_grad():
+            self._next = torch.empty_like(model._embed_images(example_images)[0])   # tokens of the frame in waiting
+
+        def frame_fn(images_next: Tensor, table: Optional[Tensor] = None) -> Tensor:
+            main = torch.cuda.current_stream()
+            current = self._next.clone()
+            self._side.wait_stream(main)          # fork: the encoder may overwrite the buffer from here on
+            with torch.cuda.stream(self._side), N.scratch_lane(1):
+                self._next.copy_(model._embed_images(images_next)[0])
+            pos3d = torch.view_as_complex(table) if table is not None else None
+            outs, _ = model(images_next, selected_idx=selected_idx, pos3d=pos3d, tokens=current)
+            out = torch.stack(outs)
+            main.wait_stream(self._side)          # join
+            return out
+
+        inputs = [example_images]
+        if model.rope3d is not None:
+            inputs.append(self._table(dev))
+        self.stream = GraphedStream(model.kv_cache_manager, frame_fn, inputs, model.kv_cache_cross_frame_special,
+                                    model.kv_cache_camera_only)
+
+    def _table(self, device) -> Tensor:
+        t = self.model.stream_table(1, self._hw[0], self._hw[1], device)
+        return torch.view_as_real(t.to(torch.complex64)).contiguous()
+
+    @torch.no_grad()
+    def prime(self, images: Tensor) -> None:
+        """Encode the first frame of the pipeline (eagerly); its outputs come out of the next call."""
+        assert tuple(images.shape[-2:]) == self._hw, "the graphs were captured for another image size"
+        self._next.copy_(self.model._embed_images(images)[0])
+        self._primed = True
+
+    def __call__(self, next_images: Tensor, keyframe: bool = True) -> Tensor:
+        """Outputs ``[groups, streams, 1, P, 2C]`` of the frame in waiting (a keyframe or not), while
+        ``next_images`` are encoded and take its place.  The result buffer is overwritten by the next
+        call of the same kind."""
+        if not self._primed:
+            raise RuntimeError("PipelinedAggregator: prime() the first frame before the first call")
+        assert tuple(next_images.shape[-2:]) == self._hw, "the graphs were captured for another image size"
+        extra = [self._table(next_images.device)] if self.model.rope3d is not None else []
+        out = self.stream(next_images, *extra, keyframe=keyframe)
         if keyframe:
             self.model.total_frames_processed += 1
         return out

@@ -195,18 +195,21 @@ _split_workspaces = {}
 
 def _split_workspace(device, nbytes: int) -> Optional[Tensor]:
     """Zero-filled device memory for launches that split K (``lbm_linear_norm``'s workspace; the
-    launches leave its counters at zero), one per device; None when nothing is needed.  The
-    blocks' launches on one device are serialised (one manager, one stream at a time), so they
-    share it.  It is never allocated or filled under stream capture: a graph would own the
-    memory and replay the fill."""
+    launches leave its counters at zero), one per device and scratch lane; None when nothing is
+    needed.  The blocks' launches of one lane on one device are serialised (one manager, one
+    stream at a time), so they share it; a chain that may overlap them runs under
+    ``_native.scratch_lane``.  It is never allocated or filled under stream capture: a graph would
+    own the memory and replay the fill."""
     if nbytes <= 0:
         return None
-    ws = _split_workspaces.get(device)
+    from . import _native as N
+    lane = (device, N.current_scratch_lane())
+    ws = _split_workspaces.get(lane)
     if ws is None or ws.numel() < nbytes:
         if torch.cuda.is_current_stream_capturing():
             raise RuntimeError("the K-split workspace must exist before a frame is captured: run the frame once "
                                "eagerly first (GraphedFrame does)")
-        ws = _split_workspaces[device] = torch.zeros(nbytes, dtype=torch.uint8, device=device)
+        ws = _split_workspaces[lane] = torch.zeros(nbytes, dtype=torch.uint8, device=device)
     return ws
 
 

@@ -42,10 +42,11 @@ def dense_attention(q: Tensor, k: Tensor, v: Tensor, num_streams: int = 1, q_pre
         need = int(N.lib.lbm_attn_workspace_bytes(streams, num_streams, H, D))
         plan = _plans[key] = (kv_rows, streams, need)
     kv_rows, streams, need = plan
-    ws = _workspace.get(q.device)
+    lane = (q.device, N.current_scratch_lane())     # one workspace per chain of launches that may overlap another
+    ws = _workspace.get(lane)
     if ws is None or ws.numel() < max(need, 16):
         ws = torch.empty(max(int(need * 1.25), 1 << 20), dtype=torch.uint8, device=q.device)
-        _workspace[q.device] = ws
+        _workspace[lane] = ws
     out = torch.empty_like(q)
     p = lambda t: C.c_void_p(t.data_ptr())
     N.check(N.lib.lbm_attn_run(

@@ -213,3 +213,40 @@ def test_graphed_aggregator_equals_eager_aggregator():
     for x, y in zip(ma.kv_caches, mb.kv_caches):
         assert torch.equal(x, y)
     mb.check_device_errors()
+
+
+def test_pipelined_aggregator_equals_eager_aggregator():
+    """The next frame's image encoder as a second branch of the graph that takes the present frame
+    through its frame and global blocks: the outputs are those of the eager aggregator bit for
+    bit, one call later; keyframes and read-only frames mixed, two ragged streams, an encoder
+    with blocks of its own (whose fc2 splits K, so both branches use a K-split workspace)."""
+    from lingbot_map_amd import HipAggregatorStream, PipelinedAggregator, set_skip_append
+    dev = torch.device("cuda:0")
+    torch.manual_seed(11)
+    kw = dict(img_size=56, patch_size=14, embed_dim=128, depth=2, num_heads=2, init_values=0.5, patch_embed="vit",
+              encoder_depth=2, enable_3d_rope=True, max_frame_num=64, kv_cache_sliding_window=[2, 3], kv_cache_scale_frames=1,
+              kv_cache_cross_frame_special=False, use_scale_token=False, page_size=4, layout="frame_pages", num_streams=2)
+    a = HipAggregatorStream(**kw).to(dev, torch.bfloat16).eval()
+    b = HipAggregatorStream(**kw).to(dev, torch.bfloat16).eval()
+    b.load_state_dict(a.state_dict())
+    g = torch.Generator(device=dev).manual_seed(12)
+    imgs = [torch.rand(2, 1, 3, 42, 56, generator=g, device=dev).to(torch.bfloat16) for _ in range(5)]
+    with torch.no_grad():
+        for i in range(6):                       # anchor and both windows full
+            a(imgs[i % 5]); b(imgs[i % 5])
+        piped = PipelinedAggregator(b, imgs[0], selected_idx=[1])
+        with pytest.raises(RuntimeError):
+            piped(imgs[0])
+        frames = [imgs[(2 * i + 1) % 5] for i in range(10)]
+        piped.prime(frames[0])
+        for i in range(9):
+            keyframe = i % 3 != 1
+            set_skip_append(a.kv_cache_manager, not keyframe)
+            want = a(frames[i], selected_idx=[1])[0][0]
+            got = piped(frames[i + 1], keyframe=keyframe)[0]       # frame i comes out while frame i + 1 is encoded
+            torch.cuda.synchronize()
+            assert torch.equal(got, want), (i, keyframe)
+    assert a.total_frames_processed == b.total_frames_processed == 12
+    for x, y in zip(a.kv_cache_manager.kv_caches, b.kv_cache_manager.kv_caches):
+        assert torch.equal(x, y)
+    b.kv_cache_manager.check_device_errors()
