@@ -593,7 +593,46 @@ def main() -> None:
                 ours(); theirs()
             sweep.append({"M": M, "N": Nn, "K": K, "lbm_linear_us": kernel_time_ms(ours, 50, torch) * 1e3,
                           "torch_us": kernel_time_ms(theirs, 50, torch) * 1e3})
-        print(json.dumps({"mode": "linear", "rows": rows, "chained": chained, "k_sweep": sweep}))
+        # the qkv projection with the producer as its store, form by form (what the q/k LayerNorm,
+        # the rotary layouts and the pool copy add to the launch), one and four frames' rows
+        forms = []
+        K, Nn = 1024, 3 * H * D
+        for M in (4 * T, T):
+            a = torch.randn(M, K, generator=g, device=dev).to(torch.bfloat16)
+            w = (torch.randn(Nn, K, generator=g, device=dev) / K ** 0.5).to(torch.bfloat16)
+            b32 = torch.randn(Nn, generator=g, device=dev)
+            tiles = 16
+            xs = a.float().reshape(M, tiles, -1)
+            mean = xs.mean(-1)
+            stats = torch.stack([mean, ((xs - mean[..., None]) ** 2).sum(-1)], -1).contiguous()
+            colsum = w.float().sum(1).contiguous()
+            ln = N.RowNorm(stats.data_ptr(), colsum.data_ptr(), tiles, 1e-5)
+            qk_norm = [torch.randn(D, generator=g, device=dev) for _ in range(4)]
+            pairs = torch.randn(M, D // 2, 2, generator=g, device=dev)
+            halves = torch.randn(M, D, 2, generator=g, device=dev)
+            q, k, v = (torch.empty(M, H, D, dtype=torch.bfloat16, device=dev) for _ in range(3))
+            pool = torch.empty((M + PAGE - 1) // PAGE + 1, 2, PAGE, H, D, dtype=torch.bfloat16, device=dev)
+            t_idx = torch.arange(M, device=dev, dtype=torch.int32)
+            pool_rows = (t_idx // PAGE * 2 * PAGE + t_idx % PAGE).contiguous()
+            stream = lambda: C.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+            def form(norm, table, layout, plain, pooled):
+                nw = [vp(t) for t in qk_norm] if norm else [None] * 4
+                return lambda: N.check(N.lib.lbm_qkv_linear_prepare_norm(
+                    vp(a), ln, vp(w), vp(b32), M, K, nw[0], nw[1], nw[2], nw[3], 1e-5, 0.18, vp(table) if table is not None else None,
+                    layout, vp(q), vp(k) if plain else None, vp(v) if plain else None, vp(pool) if pooled else None,
+                    vp(pool_rows) if pooled else None, H, D, PAGE, stream()))
+            for name, fn in (("no q/k norm, no rotary, plain q/k/v", form(False, None, N.ROPE_INTERLEAVED, True, False)),
+                             ("q/k norm", form(True, None, N.ROPE_INTERLEAVED, True, False)),
+                             ("interleaved rotary", form(False, pairs, N.ROPE_INTERLEAVED, True, False)),
+                             ("interleaved rotary + q/k norm", form(True, pairs, N.ROPE_INTERLEAVED, True, False)),
+                             ("half-split rotary + q/k norm", form(True, halves, N.ROPE_HALF_SPLIT, True, False)),
+                             ("half-split rotary + q/k norm, K/V into pool pages only", form(True, halves, N.ROPE_HALF_SPLIT, False, True)),
+                             ("half-split rotary + q/k norm, plain q/k/v and pool pages", form(True, halves, N.ROPE_HALF_SPLIT, True, True))):
+                for _ in range(10):
+                    fn()
+                forms.append({"form": name, "M": M, "lbm_qkv_linear_prepare_norm_us": kernel_time_ms(fn, 50, torch) * 1e3})
+        print(json.dumps({"mode": "linear", "rows": rows, "chained": chained, "k_sweep": sweep, "producer_forms": forms}))
         return
     blocks = args.blocks
     m = HipPagedKVCacheManager(blocks, ANCHOR + WINDOW + 16, T, H, D, torch.bfloat16, dev,
