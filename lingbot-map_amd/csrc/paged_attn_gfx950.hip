@@ -1071,6 +1071,36 @@ __global__ __launch_bounds__(kSmThreads, 1) void lbm_attn_bf16_d64_small_kernel(
 
 // Merge split-KV partial results: out = sum_s w_s * o_s with w_s = 2^(lse_s - max) / sum.
 // One thread per (query row, head, 8 consecutive d).
+//
+// Up to NJ splits (n <= NJ): all 2 NJ loads - the log-sum-exps and the partial rows - are issued
+// before the first use of any of them, one round trip of memory latency instead of three.  NJ is
+// the next of 2, 4, 8 above the split count, so that a launch with two splits (several streams'
+// frame blocks) does not load its last split seven times over.
+template <int NJ>
+__device__ __forceinline__ void lbm_combine_upto(const float* lse, const unsigned short* po, long long split_stride, int n,
+                                                 float& wsum, f32x8& acc) {
+  float t[NJ];
+  bf16x8 v[NJ];
+#pragma unroll
+  for (int j = 0; j < NJ; ++j) {
+    const long long s = min(j, n - 1);
+    t[j] = lse[s * split_stride];
+    v[j] = *(const bf16x8*)(po + s * split_stride * 64);
+  }
+  float mx = -INFINITY;
+#pragma unroll
+  for (int j = 0; j < NJ; ++j) mx = fmaxf(mx, t[j]);
+  if (mx == -INFINITY) mx = 0.f;  // every split empty (no visible token): weights 0, output 0
+#pragma unroll
+  for (int j = 0; j < NJ; ++j) {
+    const float w = j < n ? __builtin_amdgcn_exp2f(t[j] - mx) : 0.f;
+    const f32x8 vf = __builtin_convertvector(v[j], f32x8);
+    wsum += w;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) acc[e] += w * vf[e];
+  }
+}
+
 __global__ __launch_bounds__(256) void lbm_attn_combine_bf16_kernel(AttnArgs a) {
   const LbmAttnStreamPlan sp = a.sch.s[blockIdx.y];
   if (sp.n_splits <= 1) return;
@@ -1087,30 +1117,12 @@ __global__ __launch_bounds__(256) void lbm_attn_combine_bf16_kernel(AttnArgs a) 
   f32x8 acc;
 #pragma unroll
   for (int e = 0; e < 8; ++e) acc[e] = 0.f;
-  if (n <= 8) {
-    // up to eight splits (every schedule of one frame's queries): all sixteen loads - the
-    // log-sum-exps and the partial rows - are issued before the first use of any of them, one
-    // round trip of memory latency instead of three
-    float t[8];
-    bf16x8 v[8];
-#pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      const long long s = min(j, n - 1);
-      t[j] = lse[s * split_stride];
-      v[j] = *(const bf16x8*)(po + s * split_stride * 64);
-    }
-    float mx = -INFINITY;
-#pragma unroll
-    for (int j = 0; j < 8; ++j) mx = fmaxf(mx, t[j]);
-    if (mx == -INFINITY) mx = 0.f;  // every split empty (no visible token): weights 0, output 0
-#pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      const float w = j < n ? __builtin_amdgcn_exp2f(t[j] - mx) : 0.f;
-      const f32x8 vf = __builtin_convertvector(v[j], f32x8);
-      wsum += w;
-#pragma unroll
-      for (int e = 0; e < 8; ++e) acc[e] += w * vf[e];
-    }
+  if (n <= 2) {
+    lbm_combine_upto<2>(lse, po, split_stride, n, wsum, acc);
+  } else if (n <= 4) {
+    lbm_combine_upto<4>(lse, po, split_stride, n, wsum, acc);
+  } else if (n <= 8) {
+    lbm_combine_upto<8>(lse, po, split_stride, n, wsum, acc);
   } else {
     // loads are issued in batches (the split count is a run-time value, a plain loop would
     // wait for each load in turn)
