@@ -104,3 +104,20 @@ def test_rope3d_module_equals_the_oracle_table():
         m(ppf=1, pph=2, ppw=2, patch_start_idx=0, device="cpu", f_start=511, f_end=513)
     pos = PositionGetter()(2, 3, 4, "cpu")
     assert pos.shape == (2, 12, 2) and pos[1, 7].tolist() == [1, 3] and pos[0, 11].tolist() == [2, 3]
+
+
+def test_scratch_lanes_nest_and_restore():
+    """The lane that keys the package's per-device scratch memory: 0 by default, set for the span
+    of a `with`, restored on the way out, also when the body raises."""
+    from lingbot_map_amd import _native as N
+    assert N.current_scratch_lane() == 0
+    with N.scratch_lane(1):
+        assert N.current_scratch_lane() == 1
+        with N.scratch_lane(2):
+            assert N.current_scratch_lane() == 2
+        assert N.current_scratch_lane() == 1
+    assert N.current_scratch_lane() == 0
+    with pytest.raises(ValueError):
+        with N.scratch_lane(3):
+            raise ValueError("body fails")
+    assert N.current_scratch_lane() == 0
