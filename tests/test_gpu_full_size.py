@@ -225,3 +225,42 @@ def test_frame_blocks_of_several_streams_at_full_size(n_streams):
     for s in range(n_streams):
         sl = slice(s * T, (s + 1) * T)
         check(out[sl], sdpa_nhd(q[sl], k[sl], v[sl]), f"stream {s} of {n_streams}")
+
+
+@pytest.mark.parametrize("n_streams", [1, 2])
+def test_lookahead_replay_at_full_width(n_streams):
+    """The look-ahead replay (next frame's encoder beside the present frame's blocks) at the real
+    widths - 1,004 tokens per frame, dim 1,024, MLP 4,096, so that fc2 splits K over workgroups in
+    both branches (each on the workspace of its own scratch lane) and the launches of the two
+    branches share the CUs - against the plain replay of a twin model: bit-equal outputs, frame by
+    frame, and equal pools."""
+    from lingbot_map_amd import GraphedAggregator, HipAggregatorStream, PipelinedAggregator
+    dev = torch.device("cuda:0")
+    kw = dict(img_size=518, patch_size=14, embed_dim=1024, depth=3, num_heads=16, mlp_ratio=4.0, num_register_tokens=4,
+              qk_norm=True, init_values=0.01, patch_embed="vit", encoder_depth=3, enable_3d_rope=True, max_frame_num=64,
+              kv_cache_sliding_window=[3, 2][:n_streams] if n_streams > 1 else 3, kv_cache_scale_frames=1,
+              kv_cache_cross_frame_special=False, use_scale_token=False, page_size=16, layout="frame_pages",
+              num_streams=n_streams)
+    torch.manual_seed(21)
+    a = HipAggregatorStream(**kw).to(dev, torch.bfloat16).eval()
+    b = HipAggregatorStream(**kw).to(dev, torch.bfloat16).eval()
+    b.load_state_dict(a.state_dict())
+    g = torch.Generator(device=dev).manual_seed(22)
+    imgs = [torch.rand(n_streams, 1, 3, 378, 518, generator=g, device=dev).to(torch.bfloat16) for _ in range(4)]
+    with torch.no_grad():
+        for i in range(5):                       # anchor and windows full
+            a(imgs[i % 4]); b(imgs[i % 4])
+        plain = GraphedAggregator(a, imgs[0])
+        piped = PipelinedAggregator(b, imgs[0])
+        frames = [imgs[(3 * i + 1) % 4] for i in range(8)]
+        piped.prime(frames[0])
+        for i in range(7):
+            keyframe = i % 4 != 2
+            want = plain(frames[i], keyframe=keyframe).clone()
+            got = piped(frames[i + 1], keyframe=keyframe)
+            torch.cuda.synchronize()
+            assert torch.isfinite(got.float()).all()
+            assert torch.equal(got, want), (i, keyframe)
+    for x, y in zip(a.kv_cache_manager.kv_caches, b.kv_cache_manager.kv_caches):
+        assert torch.equal(x, y)
+    b.kv_cache_manager.check_device_errors()
