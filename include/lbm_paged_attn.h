@@ -24,7 +24,7 @@
 extern "C" {
 #endif
 
-#define LBM_ABI_VERSION 7
+#define LBM_ABI_VERSION 8
 
 #define LBM_OK 0
 #define LBM_ERR_INVALID 1     /* bad argument (null pointer, negative size, bad enum)      */
@@ -254,6 +254,19 @@ int lbm_linear_norm(const void* a, const lbm_row_norm* a_norm, const void* w, co
 /* Bytes of workspace with which lbm_linear_norm would split K for this shape and epilogue; 0 when
  * it would not. */
 size_t lbm_linear_workspace_bytes(int32_t M, int32_t N, int32_t K, int32_t epilogue);
+
+/* No counterpart in the reference (ABI 8).  A model's weights do not stay in any cache from one
+ * frame to the next, and a GEMM of one frame's rows that finds its weights in HBM takes 0.6 to 5 us
+ * longer than one that finds them in a cache.  A caller that knows which memory the launch AFTER
+ * the next one will read - the weights of the layer that follows - names it here: the next
+ * lbm_linear, lbm_linear_norm, lbm_qkv_linear_prepare or lbm_qkv_linear_prepare_norm call of the
+ * calling host thread then also reads one dword of every 128-byte line of [next_read, next_read +
+ * bytes) while it computes (a ninth wavefront per workgroup that does nothing else), which leaves
+ * the lines in the memory-side cache.  The hint is consumed by that one call (launches on
+ * 256-row tiles ignore it); results are the same with and without it.  The memory must be
+ * readable device memory for as long as that launch can run, replays of a captured graph
+ * included.  bytes below 128 or next_read = NULL withdraws a pending hint. */
+int lbm_linear_prefetch_hint(const void* next_read, size_t bytes);
 
 /* lbm_qkv_linear_prepare with a_norm (NULL = none) applied to the activations: norm1 of the
  * block (folded as described at lbm_row_norm), its qkv projection and the pre-attention producer

@@ -136,6 +136,11 @@ int lbm_linear_norm(const void* a, const lbm_row_norm* a_norm, const void* w, co
                            workspace_bytes, (hipStream_t)stream);
 }
 
+int lbm_linear_prefetch_hint(const void* next_read, size_t bytes) {
+  lbm_set_prefetch_hint(next_read, next_read ? bytes : 0);
+  return LBM_OK;
+}
+
 size_t lbm_linear_workspace_bytes(int32_t M, int32_t N, int32_t K, int32_t epilogue) {
   if (M <= 0 || N <= 0 || K <= 0 || N % 64 != 0 || K % 128 != 0) return 0;
   return lbm_linear_workspace_for(M, N, K, epilogue);

@@ -37,6 +37,7 @@ int lbm_launch_linear(const void* a, const lbm_row_norm* a_norm, const void* w, 
                       const void* residual, void* out, float* out_stats, int M, int N, int K, int epilogue,
                       void* workspace, size_t workspace_bytes, hipStream_t stream);
 int lbm_linear_stats_tiles_for(int M, int N);
+void lbm_set_prefetch_hint(const void* ptr, size_t bytes);
 size_t lbm_linear_workspace_for(int M, int N, int K, int epilogue);
 
 int lbm_launch_qkv_linear_prepare(const void* a, const lbm_row_norm* a_norm, const void* w, const float* bias, int M, int K,

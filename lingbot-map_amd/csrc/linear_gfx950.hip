@@ -56,6 +56,7 @@ typedef __attribute__((ext_vector_type(2))) unsigned int u32x2;
 constexpr int kGK = 128;         // K granularity the launches accept
 constexpr int kGM = 128;         // activation rows per tile
 constexpr int kGThreads = 512;
+constexpr int kGTouchThreads = 64;   // lbm_linear_bf16_kernel: one more wavefront that only asks for weight lines ahead of the loop
 constexpr int kKS = 64;          // K elements per LDS stage
 constexpr int kStagesG = 4;      // LDS stages: three being loaded while one is multiplied (six stages for the 64-column tile,
                                  // which has the room: slower, 8.4 -> 8.8 us for proj - the longer prologue costs more than the depth gains)
@@ -97,6 +98,10 @@ struct LinearArgs {
   // parks its fp32 partial tile in `split_part` and takes a ticket from the tile's counter; the
   // one that draws the last ticket sums the partials in slice order (the same sum whoever is
   // last) and runs the epilogue.  Counters start at zero and are left at zero.
+  // memory the launch after this one will read (lbm_linear_prefetch_hint): the ninth wavefronts of
+  // lbm_linear_bf16_kernel ask for it
+  const char* touch;
+  unsigned touch_lines;          // 128-byte lines
   int k_splits;
   unsigned* split_counters;      // [m_tiles * n_tiles]
   float* split_part;             // [m_tiles * n_tiles][k_splits][8 waves][NT * 16][64 lanes]
@@ -159,7 +164,7 @@ __device__ __forceinline__ void lbm_tile_of_workgroup(int b, int m_tiles, int n_
 // LNA: the activations' rows are standardised by the store (see LinearArgs).
 // SPLITK: several workgroups per tile, each over a slice of K (see LinearArgs).
 template <int EPI, int TN, int ROPE = 0, bool NORM = false, bool LNA = false, bool SPLITK = false>
-__global__ __launch_bounds__(kGThreads, 1) void lbm_linear_bf16_kernel(LinearArgs p) {
+__global__ __launch_bounds__(kGThreads + kGTouchThreads, 1) void lbm_linear_bf16_kernel(LinearArgs p) {
   constexpr int NT = TN / 64;   // 32-column blocks of W per wavefront
   // [buffer][k half][row][64 + pad]
   // [stage][row][64]: 64-wide slices of K, kStagesG of them in flight or in use
@@ -217,6 +222,33 @@ __global__ __launch_bounds__(kGThreads, 1) void lbm_linear_bf16_kernel(LinearArg
   const size_t k_first = SPLITK ? (size_t)split * nk * kKS : 0;
   const char* a_base = (const char*)(p.a + k_first);
   const char* w_base = (const char*)(p.w + (size_t)n0 * p.K + k_first);
+  if (wave >= kGThreads / 64) {   // (a scalar condition: the whole wavefront branches)
+    // The ninth wavefront holds no operand and joins no barrier (a wavefront that has ended is not
+    // waited for).  In a model every launch finds its weights in HBM - a frame walks through far
+    // more weight bytes than the caches hold - and the loop's three steps of look-ahead do not
+    // cover that latency: the same launch takes 0.6 to 5 us longer on weights that no cache holds.
+    // A caller that knows which memory the launch AFTER this one will read says so
+    // (lbm_linear_prefetch_hint), and these wavefronts, all workgroups' together, read one dword of
+    // every 128-byte line of it: the lines are then in the memory-side cache (or an L2) when that
+    // launch starts, having travelled while this one computed.
+    // (plain loads whose results the compiler sees - a load whose result it does not know of could
+    // land in a register it has reused: eight in flight per lane, their values folded into a word
+    // that is stored only under a condition that never holds)
+    unsigned folded = 0;
+    const unsigned stride = gridDim.x * 64u;
+    for (unsigned first = blockIdx.x * 64u + (unsigned)lane; first < p.touch_lines; first += 8u * stride) {
+      unsigned got[8];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const unsigned line = first + (unsigned)j * stride;
+        got[j] = line < p.touch_lines ? *(const unsigned*)(p.touch + (size_t)line * 128) : 0u;
+      }
+#pragma unroll
+      for (int j = 0; j < 8; ++j) folded ^= got[j];
+    }
+    if (folded == 0x5bd1e995u && p.M < 0) p.out[lane] = (unsigned short)folded;   // (M is never negative)
+    return;
+  }
   // The loads are written as inline assembly: the compiler would otherwise wait for every
   // LDS-direct load in flight before any LDS read that might alias it (it cannot tell the two
   // buffers apart), which serialises load and multiply.  M0 carries the LDS address of the
@@ -1058,10 +1090,30 @@ int lbm_linear_stats_tiles_for(int M, int N) {
   return p.n_tiles;
 }
 
+namespace {
+// what the calling thread's next GEMM launch is to ask for on behalf of the launch after it
+thread_local const char* g_prefetch_hint = nullptr;
+thread_local size_t g_prefetch_hint_bytes = 0;
+void lbm_take_prefetch_hint(LinearArgs& p) {
+  p.touch = g_prefetch_hint;
+  p.touch_lines = (unsigned)(g_prefetch_hint ? g_prefetch_hint_bytes / 128 : 0);
+  g_prefetch_hint = nullptr;
+  g_prefetch_hint_bytes = 0;
+}
+}  // namespace
+
+void lbm_set_prefetch_hint(const void* ptr, size_t bytes) {
+  g_prefetch_hint = bytes >= 128 ? (const char*)ptr : nullptr;
+  g_prefetch_hint_bytes = g_prefetch_hint ? bytes : 0;
+}
+
 int lbm_launch_linear(const void* a, const lbm_row_norm* a_norm, const void* w, const float* bias, const float* gamma,
                       const void* residual, void* out, float* out_stats, int M, int N, int K, int epilogue,
                       void* workspace, size_t workspace_bytes, hipStream_t stream) {
-  if (M == 0) return LBM_OK;
+  if (M == 0) {
+    lbm_set_prefetch_hint(nullptr, 0);   // a hint is for the next call, whatever that call does
+    return LBM_OK;
+  }
   if (K % kGK != 0 || N % 64 != 0)
     return lbm_fail(LBM_ERR_UNSUPPORTED, "lbm_linear: K must be a multiple of 128 and N of 64 (got K %d, N %d)", K, N);
   if (!lbm_offsets_fit(M, N, K))
@@ -1079,9 +1131,10 @@ int lbm_launch_linear(const void* a, const lbm_row_norm* a_norm, const void* w, 
   p.res = (const unsigned short*)residual;
   p.out = (unsigned short*)out;
   p.M = M; p.N = N; p.K = K;
+  lbm_take_prefetch_hint(p);
   if (int rc = lbm_set_row_norm(p, a_norm, "lbm_linear_norm")) return rc;
   const bool lna = a_norm != nullptr;
-  const dim3 block(kGThreads);
+  const dim3 block(kGThreads), block_s(kGThreads + kGTouchThreads);
   if (epilogue == LBM_LINEAR_BIAS || epilogue == LBM_LINEAR_BIAS_GELU) {
     if (const int bm = lbm_linear_big_tiles(p)) {
       const dim3 grid_b((unsigned)(p.m_tiles * p.n_tiles));
@@ -1108,16 +1161,16 @@ int lbm_launch_linear(const void* a, const lbm_row_norm* a_norm, const void* w, 
       p.split_counters = (unsigned*)workspace;
       p.split_part = (float*)((char*)workspace + lbm_linear_counter_bytes(p));
       const dim3 grid_s((unsigned)(p.m_tiles * p.n_tiles * splits));
-      if (wide) hipLaunchKernelGGL((lbm_linear_bf16_kernel<LBM_LINEAR_BIAS_RESIDUAL, 128, 0, false, false, true>), grid_s, block, 0, stream, p);
-      else hipLaunchKernelGGL((lbm_linear_bf16_kernel<LBM_LINEAR_BIAS_RESIDUAL, 64, 0, false, false, true>), grid_s, block, 0, stream, p);
+      if (wide) hipLaunchKernelGGL((lbm_linear_bf16_kernel<LBM_LINEAR_BIAS_RESIDUAL, 128, 0, false, false, true>), grid_s, block_s, 0, stream, p);
+      else hipLaunchKernelGGL((lbm_linear_bf16_kernel<LBM_LINEAR_BIAS_RESIDUAL, 64, 0, false, false, true>), grid_s, block_s, 0, stream, p);
       return lbm_check_launch("lbm_linear_bf16_kernel<split K>");
     }
   }
   const dim3 grid((unsigned)(p.m_tiles * p.n_tiles));
 #define LBM_LINEAR_LAUNCH(E, L)                                                                                  \
   {                                                                                                              \
-    if (wide) hipLaunchKernelGGL((lbm_linear_bf16_kernel<E, 128, 0, false, L>), grid, block, 0, stream, p);      \
-    else hipLaunchKernelGGL((lbm_linear_bf16_kernel<E, 64, 0, false, L>), grid, block, 0, stream, p);            \
+    if (wide) hipLaunchKernelGGL((lbm_linear_bf16_kernel<E, 128, 0, false, L>), grid, block_s, 0, stream, p);    \
+    else hipLaunchKernelGGL((lbm_linear_bf16_kernel<E, 64, 0, false, L>), grid, block_s, 0, stream, p);          \
   }
   if (epilogue == LBM_LINEAR_BIAS && lna) LBM_LINEAR_LAUNCH(LBM_LINEAR_BIAS, true)
   else if (epilogue == LBM_LINEAR_BIAS) LBM_LINEAR_LAUNCH(LBM_LINEAR_BIAS, false)
@@ -1145,6 +1198,7 @@ int lbm_launch_qkv_linear_prepare(const void* a, const lbm_row_norm* a_norm, con
   p.bias = bias;
   p.out = (unsigned short*)q_out;
   p.M = M; p.N = N; p.K = K;
+  lbm_take_prefetch_hint(p);
   p.q_norm_w = q_norm_w; p.q_norm_b = q_norm_b; p.k_norm_w = k_norm_w; p.k_norm_b = k_norm_b;
   p.rope_cs = rope_cs;
   p.k_out = (unsigned short*)k_out; p.v_out = (unsigned short*)v_out;
@@ -1185,7 +1239,7 @@ int lbm_launch_qkv_linear_prepare(const void* a, const lbm_row_norm* a_norm, con
     wide = false;
     p.n_tiles = N / 64;
   }
-  const dim3 grid((unsigned)(p.m_tiles * p.n_tiles)), block(kGThreads);
+  const dim3 grid((unsigned)(p.m_tiles * p.n_tiles)), block(kGThreads + kGTouchThreads);
 #define LBM_QKV_LAUNCH_L(R, NRM, L)                                                                                   \
   {                                                                                                                   \
     if (wide) hipLaunchKernelGGL((lbm_linear_bf16_kernel<kEpiQkvPrepare, 128, R, NRM, L>), grid, block, 0, stream, p); \

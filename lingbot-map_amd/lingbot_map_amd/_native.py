@@ -23,7 +23,7 @@ HDR = {"frame_count": 0, "n_anchor": 1, "win_head": 2, "win_count": 3, "n_free_p
        "n_free_special": 5, "n_special_pages": 6, "special_tokens": 7, "n_memory": 8,
        "n_memory_pages": 9, "error": 10, "plan_kv_tokens": 11, "plan_n_pages": 12}
 HDR_WORDS = 16
-ABI_VERSION = 7
+ABI_VERSION = 8
 
 
 # Scratch memory that the package keeps per device (the K-split workspace of the GEMM, the
@@ -69,7 +69,7 @@ class RowNorm(C.Structure):
 
 
 SYMBOLS = ("lbm_abi_version", "lbm_last_error", "lbm_tables_words", "lbm_tables_step",
-           "lbm_rows_from_pages", "lbm_kv_append", "lbm_qkv_prepare", "lbm_residual_norm", "lbm_linear", "lbm_linear_norm", "lbm_linear_stats_tiles", "lbm_linear_workspace_bytes", "lbm_qkv_linear_prepare", "lbm_qkv_linear_prepare_norm", "lbm_attn_workspace_bytes", "lbm_attn_run", "lbm_attn_run_live",
+           "lbm_rows_from_pages", "lbm_kv_append", "lbm_qkv_prepare", "lbm_residual_norm", "lbm_linear", "lbm_linear_norm", "lbm_linear_stats_tiles", "lbm_linear_workspace_bytes", "lbm_linear_prefetch_hint", "lbm_qkv_linear_prepare", "lbm_qkv_linear_prepare_norm", "lbm_attn_workspace_bytes", "lbm_attn_run", "lbm_attn_run_live",
            "lbm_attn_run_static")
 
 
@@ -100,6 +100,8 @@ def _load():
     lib.lbm_linear_norm.argtypes = [vp, p(RowNorm), vp, vp, vp, vp, vp, vp, i32, i32, i32, i32, vp, C.c_size_t, vp]
     lib.lbm_linear_workspace_bytes.restype = C.c_size_t
     lib.lbm_linear_workspace_bytes.argtypes = [i32, i32, i32, i32]
+    lib.lbm_linear_prefetch_hint.restype = C.c_int
+    lib.lbm_linear_prefetch_hint.argtypes = [vp, C.c_size_t]
     lib.lbm_linear_stats_tiles.restype = i32
     lib.lbm_linear_stats_tiles.argtypes = [i32, i32]
     lib.lbm_qkv_linear_prepare_norm.restype = C.c_int

@@ -193,6 +193,20 @@ class LayerScale(nn.Module):
 _split_workspaces = {}
 
 
+def _prefetch_hint(t: Optional[Tensor]) -> None:
+    """Tell the next GEMM launch of the package which memory the launch AFTER it will read
+    (``lbm_linear_prefetch_hint``): the weights of the layer that follows, which would otherwise
+    come from HBM when that layer starts - a frame walks through far more weight bytes than the
+    caches hold.  The blocks' chain names, in front of each of its GEMMs, the weights of the one
+    after it: proj's in front of the qkv projection, fc1's in front of proj, fc2's in front of fc1,
+    and in front of fc2 the qkv projection's of the block that follows."""
+    if t is None or not t.is_cuda:
+        return
+    import ctypes as C
+    from . import _native as N
+    N.lib.lbm_linear_prefetch_hint(C.c_void_p(t.data_ptr()), t.numel() * t.element_size())
+
+
 def _split_workspace(device, nbytes: int) -> Optional[Tensor]:
     """Zero-filled device memory for launches that split K (``lbm_linear_norm``'s workspace; the
     launches leave its counters at zero), one per device and scratch lane; None when nothing is
@@ -437,6 +451,7 @@ class HipPagedAttention(nn.Module):
             from . import _native as N
             rows = x.numel() // x.shape[-1]
             w, colsum, bias = FoldedNorm.of(self, norm, self.qkv)
+            norm.__dict__["_lbm_folded_qkv_weight"] = w    # where the block before this one finds it (_prefetch_hint)
             row_norm = N.RowNorm(stats.stats.data_ptr(), colsum.data_ptr(), stats.tiles, float(norm.eps))
             return x.reshape(rows, x.shape[-1]).contiguous(), w, bias, row_norm, (stats, colsum)
         w = self.qkv.weight
@@ -693,8 +708,11 @@ class HipPagedBlock(nn.Module):
         """Everything after the attention kernel (block.py:283-285) in three launches;
         ``heads_out`` is the attention's output before ``proj``.  With ``next_norm`` the result is
         ``(x, RowStats)``: the statistics the next block folds its ``norm1`` from."""
+        _prefetch_hint(FoldedNorm.of(self.mlp, self.norm2, self.mlp.fc1)[0])
         x, stats = self._linear_residual(heads_out, self.attn.proj, self.ls1, x, True)
+        _prefetch_hint(self.mlp.fc2.weight)
         hidden = self.mlp.fc1_gelu(x, self.norm2, stats)
+        _prefetch_hint(getattr(next_norm, "_lbm_folded_qkv_weight", None))
         x, stats = self._linear_residual(hidden, self.mlp.fc2, self.ls2, x, next_norm is not None)
         return x if next_norm is None else (x, stats)
 
@@ -723,6 +741,7 @@ class HipPagedBlock(nn.Module):
                 a_in, kw = x, dict(norm=self.norm1, stats=stats)
             else:
                 a_in, kw = (self.norm1(x) if (normed is None or stats is not None) else normed), {}
+            _prefetch_hint(self.attn.proj.weight)
             if is_streaming:
                 heads = self.attn.stream_attend_fused(kv_cache, global_idx, a_in, pos, **kw)
             else:

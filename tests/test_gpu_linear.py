@@ -418,3 +418,43 @@ def test_residual_epilogue_with_k_split_over_workgroups(M, K, Nn):
     check(out.cpu(), ref, scale=scale, bar=2.0 ** -6)
     assert N.lib.lbm_linear_norm(ptr(ad), None, ptr(wd), ptr(bd), ptr(gd), ptr(rd), ptr(rd), None, M, Nn, K,
                                  N.LINEAR_BIAS_RESIDUAL, ptr(ws), need, None) != N.OK
+
+
+@pytest.mark.parametrize("M,K,Nn,epilogue", [(1004, 1024, 3072, "bias"), (1004, 4096, 1024, "residual"), (70, 128, 64, "gelu"),
+                                             (4016, 1024, 4096, "gelu"), (1004, 1024, 1024, "residual")])
+def test_prefetch_hint_changes_no_result(M, K, Nn, epilogue):
+    """lbm_linear_prefetch_hint: the launch that consumes a hint reads the named memory besides its
+    own work - whole buffers, buffers that end inside a 128-byte line, a single line, one shorter
+    than a line (ignored) - and writes what it writes without the hint, bit for bit; the 256-row
+    tiles (4,016 rows into 4,096 columns) ignore the hint; a withdrawn hint is no hint."""
+    N = _native()
+    dev = torch.device("cuda:0")
+    a, w, bias, g = _inputs(M, K, Nn, seed=M + K + Nn)
+    epi = {"bias": N.LINEAR_BIAS, "gelu": N.LINEAR_BIAS_GELU, "residual": N.LINEAR_BIAS_RESIDUAL}[epilogue]
+    gamma = torch.rand(Nn, generator=g).to(torch.bfloat16) if epilogue == "residual" else None
+    res = torch.randn(M, Nn, generator=g).to(torch.bfloat16) if epilogue == "residual" else None
+    plain = run_linear(a, w, bias, epi, gamma, res)
+    big = torch.randn(3_000_000, generator=g).to(torch.bfloat16).to(dev)      # 6 MB, like a layer's weights
+    for nbytes in (big.numel() * 2, 1_000_003, 128, 127):
+        assert N.lib.lbm_linear_prefetch_hint(ptr(big), nbytes) == N.OK
+        hinted = run_linear(a, w, bias, epi, gamma, res)
+        assert torch.equal(hinted, plain), nbytes
+    assert N.lib.lbm_linear_prefetch_hint(ptr(big), big.numel() * 2) == N.OK
+    assert N.lib.lbm_linear_prefetch_hint(None, 0) == N.OK                     # withdrawn
+    assert torch.equal(run_linear(a, w, bias, epi, gamma, res), plain)
+    # through the split-K launch too (fc2 of one frame)
+    need = N.lib.lbm_linear_workspace_bytes(M, Nn, K, epi)
+    if need:
+        f32 = lambda t: t.float().to(dev).contiguous()
+        a_d, w_d, b_d, g_d, r_d = a.to(dev), w.to(dev), f32(bias), f32(gamma), res.to(dev)
+        ws = torch.zeros(need, dtype=torch.uint8, device=dev)
+        outs = []
+        for hint in (False, True):
+            o = torch.full((M, Nn), float("nan"), dtype=torch.bfloat16, device=dev)
+            if hint:
+                assert N.lib.lbm_linear_prefetch_hint(ptr(big), big.numel() * 2) == N.OK
+            N.check(N.lib.lbm_linear_norm(ptr(a_d), None, ptr(w_d), ptr(b_d), ptr(g_d), ptr(r_d), ptr(o), None, M, Nn, K, epi,
+                                          ptr(ws), need, None))
+            torch.cuda.synchronize()
+            outs.append(o.cpu())
+        assert torch.equal(outs[0], outs[1]) and torch.isfinite(outs[0].float()).all()
