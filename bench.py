@@ -632,7 +632,40 @@ def main() -> None:
                 for _ in range(10):
                     fn()
                 forms.append({"form": name, "M": M, "lbm_qkv_linear_prepare_norm_us": kernel_time_ms(fn, 50, torch) * 1e3})
-        print(json.dumps({"mode": "linear", "rows": rows, "chained": chained, "k_sweep": sweep, "producer_forms": forms}))
+        # weights that no cache holds (a model walks through far more weight bytes per frame than the
+        # caches hold): the same launch on one weight matrix every time, on weights rotating through
+        # 640 MB, and on the rotating weights with each launch told (lbm_linear_prefetch_hint) what
+        # the launch after it will read
+        cold = []
+        M = T
+        for name, Nn, K, epi in (("qkv", 3072, 1024, N.LINEAR_BIAS), ("proj", 1024, 1024, N.LINEAR_BIAS),
+                                 ("fc1 + gelu", 4096, 1024, N.LINEAR_BIAS_GELU), ("fc2", 1024, 4096, N.LINEAR_BIAS)):
+            copies = max(2, (640 << 20) // (Nn * K * 2))
+            a = torch.randn(M, K, generator=g, device=dev).to(torch.bfloat16)
+            ws = [(torch.randn(Nn, K, generator=g, device=dev) / K ** 0.5).to(torch.bfloat16) for _ in range(copies)]
+            b32 = torch.randn(Nn, generator=g, device=dev)
+            out = torch.empty(M, Nn, dtype=torch.bfloat16, device=dev)
+            stream = lambda: C.c_void_p(torch.cuda.current_stream().cuda_stream)
+            at = [0]
+
+            def launch(rotate: bool, hint: bool):
+                if rotate:
+                    at[0] = (at[0] + 1) % copies
+                if hint:
+                    nxt = ws[(at[0] + 1) % copies]
+                    N.check(N.lib.lbm_linear_prefetch_hint(vp(nxt), nxt.numel() * 2))
+                N.check(N.lib.lbm_linear(vp(a), vp(ws[at[0]]), vp(b32), None, None, vp(out), M, Nn, K, epi, stream()))
+            times = {}
+            for label, rotate, hint in (("same_weights_us", False, False), ("rotating_weights_us", True, False),
+                                        ("rotating_weights_hinted_us", True, True)):
+                fn = lambda: launch(rotate, hint)
+                for _ in range(3):
+                    fn()
+                times[label] = kernel_time_ms(fn, 100, torch) * 1e3
+            cold.append({"layer": name, "M": M, "K": K, "N": Nn, "weight_copies": copies, **times})
+            del ws
+        print(json.dumps({"mode": "linear", "rows": rows, "chained": chained, "k_sweep": sweep, "producer_forms": forms,
+                          "cold_weights": cold}))
         return
     blocks = args.blocks
     m = HipPagedKVCacheManager(blocks, ANCHOR + WINDOW + 16, T, H, D, torch.bfloat16, dev,
