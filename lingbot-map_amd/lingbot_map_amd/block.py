@@ -199,7 +199,9 @@ def _prefetch_hint(t: Optional[Tensor]) -> None:
     come from HBM when that layer starts - a frame walks through far more weight bytes than the
     caches hold.  The blocks' chain names, in front of each of its GEMMs, the weights of the one
     after it: proj's in front of the qkv projection, fc1's in front of proj, fc2's in front of fc1,
-    and in front of fc2 the qkv projection's of the block that follows."""
+    and in front of fc2 the qkv projection's of the block that follows - while a frame is being
+    captured into a HIP graph, where the GPU sets the pace; an eager frame is bound by the host's
+    launches and is spared the four extra calls per block."""
     if t is None or not t.is_cuda:
         return
     import ctypes as C
@@ -704,15 +706,19 @@ class HipPagedBlock(nn.Module):
                                       N.stream_ptr(a.device)))
         return out.reshape(residual.shape), stats
 
-    def _finish_chain(self, x: Tensor, heads_out: Tensor, next_norm):
+    def _finish_chain(self, x: Tensor, heads_out: Tensor, next_norm, hints: bool = False):
         """Everything after the attention kernel (block.py:283-285) in three launches;
         ``heads_out`` is the attention's output before ``proj``.  With ``next_norm`` the result is
-        ``(x, RowStats)``: the statistics the next block folds its ``norm1`` from."""
-        _prefetch_hint(FoldedNorm.of(self.mlp, self.norm2, self.mlp.fc1)[0])
+        ``(x, RowStats)``: the statistics the next block folds its ``norm1`` from.  ``hints``: name
+        the next launch's weights in front of each launch (``_prefetch_hint``)."""
+        if hints:
+            _prefetch_hint(FoldedNorm.of(self.mlp, self.norm2, self.mlp.fc1)[0])
         x, stats = self._linear_residual(heads_out, self.attn.proj, self.ls1, x, True)
-        _prefetch_hint(self.mlp.fc2.weight)
+        if hints:
+            _prefetch_hint(self.mlp.fc2.weight)
         hidden = self.mlp.fc1_gelu(x, self.norm2, stats)
-        _prefetch_hint(getattr(next_norm, "_lbm_folded_qkv_weight", None))
+        if hints:
+            _prefetch_hint(getattr(next_norm, "_lbm_folded_qkv_weight", None))
         x, stats = self._linear_residual(hidden, self.mlp.fc2, self.ls2, x, next_norm is not None)
         return x if next_norm is None else (x, stats)
 
@@ -741,13 +747,17 @@ class HipPagedBlock(nn.Module):
                 a_in, kw = x, dict(norm=self.norm1, stats=stats)
             else:
                 a_in, kw = (self.norm1(x) if (normed is None or stats is not None) else normed), {}
-            _prefetch_hint(self.attn.proj.weight)
+            # (hints only where the GPU sets the pace: an eager frame is bound by the host's launches,
+            # and four more calls per block would slow it)
+            hints = torch.cuda.is_current_stream_capturing()
+            if hints:
+                _prefetch_hint(self.attn.proj.weight)
             if is_streaming:
                 heads = self.attn.stream_attend_fused(kv_cache, global_idx, a_in, pos, **kw)
             else:
                 heads = self.attn.dense_attend_fused(a_in, pos, enable_3d_rope, **kw)
             heads = heads.reshape(x.shape[0], x.shape[1], self.attn.num_heads * self.attn.head_dim).to(x.dtype)
-            return self._finish_chain(x, heads, next_norm)
+            return self._finish_chain(x, heads, next_norm, hints)
         n1 = self.norm1(x) if (normed is None or stats is not None) else normed
         if is_streaming:
             if self.attn.can_fuse(kv_cache, pos, enable_3d_rope):
