@@ -23,6 +23,7 @@ reference's method-by-method sequence is used.
 from __future__ import annotations
 
 import math
+import os
 from typing import Callable, Optional
 
 import torch
@@ -588,6 +589,10 @@ class HipPagedAttention(nn.Module):
 
 
 class HipPagedBlock(nn.Module):
+    #: name the next launch's weights in front of every GEMM of a captured frame (``_prefetch_hint``);
+    #: a switch for measurements - results do not depend on it
+    PREFETCH_HINTS = os.environ.get("LBM_PREFETCH_HINTS", "1") != "0"
+
     def __init__(self, dim: int, num_heads: int, mlp_ratio: float = 4.0, qkv_bias: bool = True,
                  proj_bias: bool = True, ffn_bias: bool = True, drop: float = 0.0, attn_drop: float = 0.0,
                  init_values=None, drop_path: float = 0.0, act_layer: Callable[..., nn.Module] = nn.GELU,
@@ -749,7 +754,7 @@ class HipPagedBlock(nn.Module):
                 a_in, kw = (self.norm1(x) if (normed is None or stats is not None) else normed), {}
             # (hints only where the GPU sets the pace: an eager frame is bound by the host's launches,
             # and four more calls per block would slow it)
-            hints = torch.cuda.is_current_stream_capturing()
+            hints = self.PREFETCH_HINTS and torch.cuda.is_current_stream_capturing()
             if hints:
                 _prefetch_hint(self.attn.proj.weight)
             if is_streaming:
