@@ -153,6 +153,7 @@ def config3_stream(torch) -> dict:
     for _ in range(5):
         m.step(0, q, k, v, keyframe=[True])
     step_ms = event_time_ms(lambda: m.step(0, q, k, v, keyframe=[True]), 20, torch)
+    m._plan(0, [False])   # every visible row in the pool again (a step's table names its new frame by the caller's rows)
     attn_ms = event_time_ms(lambda: m._attend_planned(0, q, None, None), 50, torch)
     m.check_device_errors()
     kv_now = m._plan_tokens[0][0]
@@ -817,6 +818,8 @@ def main() -> None:
 
     # ---- per-kernel timings with HIP events on the launch stream
     flops = 4.0 * T * kv_tokens * H * D
+    m._plan(0, [False])   # the row table of the same visible tokens with every row in the pool (the steps' tables name the newest frame by the caller's rows)
+    assert m._plan_tokens[0][0] == kv_tokens
     attn_ms = event_time_ms(lambda: m._attend_planned(1, qs[0], None, None), 500, torch)
     append_ms = kernel_time_ms(lambda: m._scatter(1, m._append_rows[0], ks[0], vs[0]), 100, torch)
     ops = m._ops([{"ops": 16, "expect_kv_tokens": kv_tokens}])

@@ -24,7 +24,7 @@
 extern "C" {
 #endif
 
-#define LBM_ABI_VERSION 8
+#define LBM_ABI_VERSION 9
 
 #define LBM_OK 0
 #define LBM_ERR_INVALID 1     /* bad argument (null pointer, negative size, bad enum)      */
@@ -59,6 +59,11 @@ extern "C" {
 #define LBM_OP_APPEND 4
 #define LBM_OP_EVICT 8
 #define LBM_OP_PLAN 16
+/* with LBM_OP_PLAN, frame_pages layout (ABI 9): the rows of the newest cached frame - the one
+ * this step's LBM_OP_APPEND stored - name the caller's own K/V rows (q_begin + t, as self_tokens
+ * rows do) instead of its pool rows, in the same place of the row table.  For a step whose append
+ * is carried out by the attention call itself (lbm_attn_run_append), after the pool was read. */
+#define LBM_OP_PLAN_NEWEST_SELF 32
 
 /* Sticky bits of the device-side error word (header word LBM_HDR_ERROR). */
 #define LBM_TERR_PATCH_POOL 1   /* flashinfer_cache.py:489-494 */
@@ -291,6 +296,21 @@ int lbm_attn_run_live(const void* q, const void* pool, void* out, const void* se
                       const lbm_attn_stream* streams, int32_t n_streams, int32_t num_heads,
                       int32_t head_dim, int32_t page_size, int32_t dtype, float sm_scale,
                       void* workspace, size_t workspace_bytes, void* stream);
+
+/* lbm_attn_run followed by the append of the current frames' K/V, as one call (ABI 9): new_k /
+ * new_v are the self_k / self_v of lbm_attn_run (rows the table names by negative entries are read
+ * from them) and, once the attention has read the pool, row t of them is also stored in pool row
+ * append_rows[t] (a negative entry stores nothing), t < append_tokens - by the launch that merges
+ * the split-KV partial results where there is one, so that the append costs no launch of its own,
+ * by a launch of its own otherwise.  Replaces append_frame (flashinfer_cache.py:474-553, its
+ * writes) and prefill_wrapper.run (:418-421) of one streamed frame as lbm_kv_append + lbm_attn_run
+ * do, with the same results, for a step whose row table names the newest frame by the caller's
+ * rows (LBM_OP_PLAN_NEWEST_SELF); pool and new_k / new_v share the dtype. */
+int lbm_attn_run_append(const void* q, void* pool, void* out, const void* new_k, const void* new_v,
+                        const int32_t* kv_rows, const int32_t* append_rows, int32_t append_tokens,
+                        const lbm_attn_stream* streams, int32_t n_streams, int32_t num_heads,
+                        int32_t head_dim, int32_t page_size, int32_t dtype, float sm_scale,
+                        void* workspace, size_t workspace_bytes, void* stream);
 
 /* Fused pre-attention producer: per-head LayerNorm of q and k, rotary embedding of q and k
  * (interleaved pairs), [token][head][dim] layout and the keyframe-gated paged append of k and

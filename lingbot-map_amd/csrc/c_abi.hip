@@ -43,8 +43,12 @@ int lbm_tables_step(int32_t* tables, const lbm_cache_geom* geom, int32_t n_strea
     return lbm_fail(LBM_ERR_INVALID, "lbm_tables_step: n_streams %d outside [1, %d]", n_streams, LBM_MAX_STREAMS);
   for (int i = 0; i < n_streams; ++i) {
     const lbm_step_op& o = ops[i];
-    if (o.ops & ~(LBM_OP_RESET | LBM_OP_ROLLBACK | LBM_OP_APPEND | LBM_OP_EVICT | LBM_OP_PLAN))
+    if (o.ops & ~(LBM_OP_RESET | LBM_OP_ROLLBACK | LBM_OP_APPEND | LBM_OP_EVICT | LBM_OP_PLAN | LBM_OP_PLAN_NEWEST_SELF))
       return lbm_fail(LBM_ERR_INVALID, "lbm_tables_step: stream %d has unknown op bits 0x%x", i, o.ops);
+    if ((o.ops & LBM_OP_PLAN_NEWEST_SELF) &&
+        ((o.ops & (LBM_OP_APPEND | LBM_OP_PLAN)) != (LBM_OP_APPEND | LBM_OP_PLAN) || geom->layout != LBM_LAYOUT_FRAME_PAGES))
+      return lbm_fail(LBM_ERR_INVALID, "lbm_tables_step: stream %d: LBM_OP_PLAN_NEWEST_SELF goes with LBM_OP_APPEND | "
+                      "LBM_OP_PLAN in the frame_pages layout", i);
     if ((o.ops & LBM_OP_PLAN) && !kv_rows && !(kv_page_ids && kv_page_lens))
       return lbm_fail(LBM_ERR_INVALID, "lbm_tables_step: PLAN needs kv_rows or the page table outputs");
     if ((o.ops & LBM_OP_PLAN) && (o.expect_kv_tokens == INT32_MIN || o.kv_row_begin < 0 || o.page_out_begin < 0))
@@ -219,7 +223,8 @@ static int lbm_attn_run_impl(const char* who, const void* q, const void* pool, v
                              const void* self_v, const int32_t* kv_rows, const int32_t* live_kv_tokens,
                              const lbm_attn_stream* streams, int32_t n_streams, int32_t num_heads,
                              int32_t head_dim, int32_t page_size, int32_t dtype, float sm_scale,
-                             void* workspace, size_t workspace_bytes, void* stream) {
+                             void* workspace, size_t workspace_bytes, void* stream,
+                             const int32_t* append_rows = nullptr, int32_t append_tokens = 0) {
   int rc = lbm_check_attn_streams(streams, n_streams, who);
   if (rc != LBM_OK) return rc;
   if (!q || !pool || !out || !kv_rows) return lbm_fail(LBM_ERR_INVALID, "%s: null q, pool, out or kv_rows", who);
@@ -235,7 +240,7 @@ static int lbm_attn_run_impl(const char* who, const void* q, const void* pool, v
   if (need > 0 && (!workspace || workspace_bytes < need))
     return lbm_fail(LBM_ERR_WORKSPACE, "%s: workspace of %zu bytes, %zu needed", who, workspace_bytes, need);
   return lbm_launch_attention(q, pool, out, self_k, self_v, kv_rows, live_kv_tokens, sch, num_heads, head_dim,
-                              page_size, dtype, sm_scale, workspace, (hipStream_t)stream);
+                              page_size, dtype, sm_scale, workspace, (hipStream_t)stream, append_rows, append_tokens);
 }
 
 int lbm_attn_run(const void* q, const void* pool, void* out, const void* self_k,
@@ -245,6 +250,19 @@ int lbm_attn_run(const void* q, const void* pool, void* out, const void* self_k,
                  void* stream) {
   return lbm_attn_run_impl("lbm_attn_run", q, pool, out, self_k, self_v, kv_rows, nullptr, streams, n_streams,
                            num_heads, head_dim, page_size, dtype, sm_scale, workspace, workspace_bytes, stream);
+}
+
+int lbm_attn_run_append(const void* q, void* pool, void* out, const void* new_k, const void* new_v,
+                        const int32_t* kv_rows, const int32_t* append_rows, int32_t append_tokens,
+                        const lbm_attn_stream* streams, int32_t n_streams, int32_t num_heads,
+                        int32_t head_dim, int32_t page_size, int32_t dtype, float sm_scale,
+                        void* workspace, size_t workspace_bytes, void* stream) {
+  if (!new_k || !new_v || !append_rows)
+    return lbm_fail(LBM_ERR_INVALID, "lbm_attn_run_append: null new_k, new_v or append_rows");
+  if (append_tokens < 0) return lbm_fail(LBM_ERR_INVALID, "lbm_attn_run_append: negative append_tokens");
+  return lbm_attn_run_impl("lbm_attn_run_append", q, pool, out, new_k, new_v, kv_rows, nullptr, streams, n_streams,
+                           num_heads, head_dim, page_size, dtype, sm_scale, workspace, workspace_bytes, stream,
+                           append_rows, append_tokens);
 }
 
 int lbm_attn_run_live(const void* q, const void* pool, void* out, const void* self_k,

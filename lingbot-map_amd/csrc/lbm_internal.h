@@ -68,7 +68,8 @@ int lbm_launch_attention(const void* q, const void* pool, void* out, const void*
                          const void* self_v, const int32_t* kv_rows, const int32_t* live_kv_tokens,
                          const LbmAttnSchedule& sch,
                          int num_heads, int head_dim, int page_size, int dtype, float sm_scale,
-                         void* workspace, hipStream_t stream);
+                         void* workspace, hipStream_t stream,
+                         const int32_t* append_rows = nullptr, int append_tokens = 0);
 
 // Address and size of the library's static device scratch array on the current device (looked
 // up once per device; no allocation).

@@ -80,6 +80,10 @@ struct AttnCore {
   int num_heads;
   int page_size;
   float scale_log2;
+  // the append carried by the merging launch: row t of self_k / self_v to pool row append_rows[t]
+  const int32_t* append_rows;
+  int append_tokens;
+  int combine_blocks;      // blocks (per stream) of that launch that merge; those beyond them append
 };
 struct AttnArgs : AttnCore {
   LbmAttnSchedule sch;
@@ -1102,6 +1106,25 @@ __device__ __forceinline__ void lbm_combine_upto(const float* lse, const unsigne
 }
 
 __global__ __launch_bounds__(256) void lbm_attn_combine_bf16_kernel(AttnArgs a) {
+  if ((int)blockIdx.x >= a.combine_blocks) {
+    // The append's share of the launch (lbm_attn_run_append): the main kernel has read the pool,
+    // the new frames' rows - attended to from the caller's tensors - now go into their pages.  One
+    // 16-byte piece of a K row and of the matching V row per thread, as lbm_kv_append_kernel.
+    if (blockIdx.y != 0) return;
+    const int pieces = a.num_heads * 8;
+    const long long idx = (long long)((int)blockIdx.x - a.combine_blocks) * 256 + threadIdx.x;
+    if (idx >= (long long)a.append_tokens * pieces) return;
+    const int t = (int)(idx / pieces), piece = (int)(idx % pieces);
+    const int row = a.append_rows[t];
+    if (row < 0) return;
+    const long long row_elems = (long long)a.num_heads * 64;
+    const long long src = t * row_elems + piece * 8, dk = row * row_elems + piece * 8;
+    unsigned short* pool = const_cast<unsigned short*>(a.pool);
+    const u32x4 kk = *(const u32x4*)(a.self_k + src), vv = *(const u32x4*)(a.self_v + src);
+    *(u32x4*)(pool + dk) = kk;
+    *(u32x4*)(pool + dk + (long long)a.page_size * row_elems) = vv;
+    return;
+  }
   const LbmAttnStreamPlan sp = a.sch.s[blockIdx.y];
   if (sp.n_splits <= 1) return;
   const int H = a.num_heads;
@@ -1809,11 +1832,36 @@ size_t lbm_attn_schedule_bytes(const LbmAttnSchedule& sch, int num_heads, int he
   return split_kv > few_q ? split_kv : few_q;
 }
 
+namespace {
+int lbm_launch_attention_only(const void* q, const void* pool, void* out, const void* self_k,
+                              const void* self_v, const int32_t* kv_rows, const int32_t* live_kv_tokens,
+                              const LbmAttnSchedule& sch, int num_heads, int head_dim, int page_size, int dtype,
+                              float sm_scale, void* workspace, hipStream_t stream, const int32_t* append_rows,
+                              int append_tokens, bool* appended);
+}  // namespace
+
+// append_rows (lbm_attn_run_append): rows of self_k / self_v that are stored in the pool after the
+// attention has read it - inside the launch that merges the split-KV partials when the schedule has
+// one, by lbm_kv_append_kernel behind the attention otherwise.
 int lbm_launch_attention(const void* q, const void* pool, void* out, const void* self_k,
                          const void* self_v, const int32_t* kv_rows, const int32_t* live_kv_tokens,
                          const LbmAttnSchedule& sch,
                          int num_heads, int head_dim, int page_size, int dtype, float sm_scale,
-                         void* workspace, hipStream_t stream) {
+                         void* workspace, hipStream_t stream, const int32_t* append_rows, int append_tokens) {
+  bool appended = false;
+  int rc = lbm_launch_attention_only(q, pool, out, self_k, self_v, kv_rows, live_kv_tokens, sch, num_heads, head_dim,
+                                     page_size, dtype, sm_scale, workspace, stream, append_rows, append_tokens, &appended);
+  if (rc != LBM_OK || !append_rows || append_tokens <= 0 || appended) return rc;
+  return lbm_launch_append(self_k, self_v, dtype, const_cast<void*>(pool), dtype, append_rows, append_tokens, num_heads,
+                           head_dim, page_size, stream);
+}
+
+namespace {
+int lbm_launch_attention_only(const void* q, const void* pool, void* out, const void* self_k,
+                              const void* self_v, const int32_t* kv_rows, const int32_t* live_kv_tokens,
+                              const LbmAttnSchedule& sch, int num_heads, int head_dim, int page_size, int dtype,
+                              float sm_scale, void* workspace, hipStream_t stream, const int32_t* append_rows,
+                              int append_tokens, bool* appended) {
   if (head_dim != 64 && !(head_dim == 128 && dtype == LBM_DTYPE_F32))
     return lbm_fail(LBM_ERR_UNSUPPORTED, "attention kernels cover head_dim 64 (bf16, fp32) and 128 (fp32), got %d", head_dim);
   if (dtype == LBM_DTYPE_F32) {
@@ -1885,6 +1933,9 @@ int lbm_launch_attention(const void* q, const void* pool, void* out, const void*
   a.num_heads = num_heads;
   a.page_size = page_size;
   a.scale_log2 = sm_scale == 0.f ? 1.0f : sm_scale * 1.4426950408889634f;   // 0: q already carries scale * log2(e)
+  a.append_rows = nullptr;
+  a.append_tokens = 0;
+  a.combine_blocks = 0x7fffffff;
   a.sch = sch;
   if (sch.total_wgs == 0) return LBM_OK;
   if (sch.small) {
@@ -1899,12 +1950,20 @@ int lbm_launch_attention(const void* q, const void* pool, void* out, const void*
     for (int i = 0; i < sch.n_streams; ++i)
       if (sch.s[i].n_splits > 1 && sch.s[i].q_rows > max_rows) max_rows = sch.s[i].q_rows;
     const long long threads = (long long)max_rows * num_heads * 8;
-    hipLaunchKernelGGL(lbm_attn_combine_bf16_kernel, dim3((unsigned)((threads + 255) / 256), sch.n_streams),
-                       dim3(256), 0, stream, a);
+    unsigned blocks = (unsigned)((threads + 255) / 256);
+    a.combine_blocks = (int)blocks;
+    if (append_rows && append_tokens > 0) {
+      a.append_rows = append_rows;
+      a.append_tokens = append_tokens;
+      blocks += (unsigned)(((long long)append_tokens * num_heads * 8 + 255) / 256);
+      *appended = true;
+    }
+    hipLaunchKernelGGL(lbm_attn_combine_bf16_kernel, dim3(blocks, sch.n_streams), dim3(256), 0, stream, a);
     rc = lbm_check_launch("lbm_attn_combine_bf16_kernel");
   }
   return rc;
 }
+}  // namespace
 
 // ---------------------------------------------------------------------------- static scratch
 // Workspace for callers that cannot allocate (lbm_attn_run_static): split-KV partials and the

@@ -226,6 +226,9 @@ LBM_HD void lbm_phase_plan(int32_t* st, const lbm_cache_geom& g, const LbmTables
   const int nfr = h.na + h.wc;
   const int frame_tokens = nfr * L.tpf;
   const int self_n = op.self_tokens > 0 ? op.self_tokens : 0;
+  // LBM_OP_PLAN_NEWEST_SELF: the newest cached frame (the one this step appended: the last of the
+  // frame list) is named by the caller's own rows, in the place its pool rows would take
+  const bool newest_self = (op.ops & LBM_OP_PLAN_NEWEST_SELF) != 0 && !two && nfr > 0;
   int total = frame_tokens + h.stc + self_n;
   // expect_kv_tokens >= 0: the host's own count, which must agree; < 0: the host does not track
   // the count and gives the capacity of this stream's part of kv_rows instead
@@ -262,7 +265,8 @@ LBM_HD void lbm_phase_plan(int32_t* st, const lbm_cache_geom& g, const LbmTables
 #endif
         for (int k = 0; k < 8; ++k) {
           const int i = (f0 + k) * L.tpf + t;
-          if (f0 + k < nfr && i < limit) out[i] = page[k] * 2 * S + slot;
+          if (f0 + k < nfr && i < limit)
+            out[i] = (newest_self && f0 + k == nfr - 1) ? -1 - (op.q_begin + t) : page[k] * 2 * S + slot;
         }
       }
     }

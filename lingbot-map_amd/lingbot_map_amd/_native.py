@@ -16,14 +16,14 @@ ROPE_INTERLEAVED, ROPE_HALF_SPLIT = 0, 1
 LINEAR_BIAS, LINEAR_BIAS_GELU, LINEAR_BIAS_RESIDUAL = 0, 1, 2
 MAX_STREAMS = 16
 STATIC_SCRATCH_MIB = 64
-OP_RESET, OP_ROLLBACK, OP_APPEND, OP_EVICT, OP_PLAN = 1, 2, 4, 8, 16
+OP_RESET, OP_ROLLBACK, OP_APPEND, OP_EVICT, OP_PLAN, OP_PLAN_NEWEST_SELF = 1, 2, 4, 8, 16, 32
 TERR_NAMES = {1: "patch page pool exhausted", 2: "special page pool exhausted", 4: "window ring full",
               8: "trajectory memory full", 16: "rollback underflow", 32: "visible token count mismatch"}
 HDR = {"frame_count": 0, "n_anchor": 1, "win_head": 2, "win_count": 3, "n_free_patch": 4,
        "n_free_special": 5, "n_special_pages": 6, "special_tokens": 7, "n_memory": 8,
        "n_memory_pages": 9, "error": 10, "plan_kv_tokens": 11, "plan_n_pages": 12}
 HDR_WORDS = 16
-ABI_VERSION = 8
+ABI_VERSION = 9
 
 
 # Scratch memory that the package keeps per device (the K-split workspace of the GEMM, the
@@ -69,7 +69,7 @@ class RowNorm(C.Structure):
 
 
 SYMBOLS = ("lbm_abi_version", "lbm_last_error", "lbm_tables_words", "lbm_tables_step",
-           "lbm_rows_from_pages", "lbm_kv_append", "lbm_qkv_prepare", "lbm_residual_norm", "lbm_linear", "lbm_linear_norm", "lbm_linear_stats_tiles", "lbm_linear_workspace_bytes", "lbm_linear_prefetch_hint", "lbm_qkv_linear_prepare", "lbm_qkv_linear_prepare_norm", "lbm_attn_workspace_bytes", "lbm_attn_run", "lbm_attn_run_live",
+           "lbm_rows_from_pages", "lbm_kv_append", "lbm_qkv_prepare", "lbm_residual_norm", "lbm_linear", "lbm_linear_norm", "lbm_linear_stats_tiles", "lbm_linear_workspace_bytes", "lbm_linear_prefetch_hint", "lbm_qkv_linear_prepare", "lbm_qkv_linear_prepare_norm", "lbm_attn_workspace_bytes", "lbm_attn_run", "lbm_attn_run_append", "lbm_attn_run_live",
            "lbm_attn_run_static")
 
 
@@ -113,6 +113,9 @@ def _load():
     lib.lbm_attn_run.restype = C.c_int
     lib.lbm_attn_run.argtypes = [vp, vp, vp, vp, vp, vp, p(AttnStream), i32, i32, i32, i32, i32,
                                  C.c_float, vp, C.c_size_t, vp]
+    lib.lbm_attn_run_append.restype = C.c_int
+    lib.lbm_attn_run_append.argtypes = [vp, vp, vp, vp, vp, vp, vp, i32, p(AttnStream), i32, i32, i32, i32, i32,
+                                        C.c_float, vp, C.c_size_t, vp]
     lib.lbm_attn_run_live.restype = C.c_int
     lib.lbm_attn_run_live.argtypes = [vp, vp, vp, vp, vp, vp, vp, p(AttnStream), i32, i32, i32, i32, i32,
                                       C.c_float, vp, C.c_size_t, vp]

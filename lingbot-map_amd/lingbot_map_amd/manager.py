@@ -180,6 +180,10 @@ class HipPagedKVCacheManager:
         self._plan_valid = [False] * self._n_sets
         # append rows of frames block 0 wrote while other blocks were still behind (anchor pass)
         self._rows_log: Dict[int, Tensor] = {}
+        #: step(): the attention call stores the new frame itself (lbm_attn_run_append), reading it
+        #: from the caller's tensors meanwhile - no append launch in front of the attention
+        self.fuse_append = True
+        self._newest_self = [False] * self._n_sets   # the set's row table names the newest frame by the caller's rows
         self._n_appends: List[int] = [0] * num_blocks    # appends ever made per block (rollbacks do not count down)
         self.reset()
 
@@ -426,6 +430,7 @@ class HipPagedKVCacheManager:
                         "expect_kv_tokens": self._expect(n)})
         self._tables_step(ts, self._ops(per), kv_rows=True, pages=pages)
         self._plan_valid[ts] = True
+        self._newest_self[ts] = False
 
     def compute_attention(self, block_idx: int, q: Tensor, self_k: Optional[Tensor] = None,
                           self_v: Optional[Tensor] = None) -> Tensor:
@@ -451,7 +456,14 @@ class HipPagedKVCacheManager:
         k, v = self._check_frame("k", k), self._check_frame("v", v)
         if v.dtype != k.dtype:
             v = v.to(k.dtype)
-        ts, keyframe, tail = self._step_tables(block_idx, keyframe, cross_frame_special, camera_only)
+        want = self.fuse_append and self.layout == "frame_pages" and not self.device_token_counts
+        ts, keyframe, tail = self._step_tables(block_idx, keyframe, cross_frame_special, camera_only, newest_self=want)
+        if self._newest_self[ts]:
+            # the row table names the keyframes' new rows by k and v themselves: attend, then store
+            # them, in one call
+            self.frame_count[block_idx] += 1
+            self._n_appends[block_idx] += 1
+            return self._attend_planned(block_idx, q, k, v, append_rows=self._append_rows[ts])
         if any(keyframe):
             self._scatter(block_idx, self._append_rows[ts], k, v)
             self.frame_count[block_idx] += 1
@@ -587,9 +599,12 @@ class HipPagedKVCacheManager:
                 self._plan_tokens[ts][b] = self._visible_tokens(c)
 
     def _step_tables(self, block_idx: int, keyframe: Optional[Sequence[bool]], cross_frame_special: bool,
-                     camera_only: bool):
+                     camera_only: bool, newest_self: bool = False):
         """Table work of one streamed frame (allocate, evict, visible rows; one launch on the
-        leading block).  Returns the table set and the per-stream keyframe / read-only flags."""
+        leading block).  Returns the table set and the per-stream keyframe / read-only flags.
+        ``newest_self`` (leading block): the row table names the rows a keyframe appends by the
+        caller's own K/V rows; every block of the frame then attends and appends with
+        ``lbm_attn_run_append`` (``step`` does), which ``_newest_self`` remembers."""
         if keyframe is None:
             keyframe = [not self._skip_append] * self.num_streams
         keyframe = [bool(x) and self._active[b] for b, x in enumerate(keyframe)]
@@ -606,7 +621,7 @@ class HipPagedKVCacheManager:
                 ops, n = 0, 0
                 if keyframe[b]:
                     self._mirror_append(c, block_idx)
-                    ops = N.OP_APPEND | N.OP_PLAN
+                    ops = N.OP_APPEND | N.OP_PLAN | (N.OP_PLAN_NEWEST_SELF if newest_self else 0)
                     if not self._defer_eviction:
                         self._mirror_evict(c, self._windows[b], keep, block_idx)
                         ops |= N.OP_EVICT
@@ -620,15 +635,21 @@ class HipPagedKVCacheManager:
                             "expect_kv_tokens": self._expect(n)})
             self._tables_step(ts, self._ops(per), append_rows=True, kv_rows=True)
             self._plan_valid[ts] = True
+            self._newest_self[ts] = bool(newest_self and any(keyframe))
         elif self._n_appends[block_idx] + (1 if any(keyframe) else 0) != self._n_appends[0]:
             raise RuntimeError(f"step: block {block_idx} has made {self._n_appends[block_idx]} appends, block 0 "
                                f"{self._n_appends[0]}: with shared page tables every block takes the frame block 0 took")
         return ts, keyframe, tail
 
     def _attend_planned(self, block_idx: int, q: Tensor, self_k: Optional[Tensor], self_v: Optional[Tensor],
-                        q_prescaled: bool = False) -> Tensor:
-        """``q_prescaled``: q already carries 1 / sqrt(D) and log2(e) (``step_qkv``'s producer)."""
+                        q_prescaled: bool = False, append_rows: Optional[Tensor] = None) -> Tensor:
+        """``q_prescaled``: q already carries 1 / sqrt(D) and log2(e) (``step_qkv``'s producer).
+        ``append_rows``: ``self_k`` / ``self_v`` are also stored, row t in pool row
+        ``append_rows[t]``, once the attention has read the pool (``lbm_attn_run_append``)."""
         ts = self._set(block_idx)
+        if self._newest_self[ts] and append_rows is None:
+            raise RuntimeError("this frame's row table names its newest frame by the caller's K/V rows (step() led "
+                               "the frame): every block of the frame takes it through step()")
         rows = self.num_streams * self.tokens_per_frame
         assert q.dim() == 3 and tuple(q.shape) == (rows, self.num_heads, self.head_dim), (
             f"q: expected [{rows}, {self.num_heads}, {self.head_dim}], got {tuple(q.shape)}")
@@ -648,6 +669,8 @@ class HipPagedKVCacheManager:
         if n < self.num_streams:
             out.zero_()
         if n == 0:
+            if append_rows is not None:
+                self._scatter(block_idx, append_rows, self_k, self_v)
             return out
         need = N.lib.lbm_attn_workspace_bytes(streams, n, self.num_heads, self.head_dim)
         if need > self.workspace_buffer.numel():
@@ -659,7 +682,9 @@ class HipPagedKVCacheManager:
         tensors = (C.c_void_p(qc.data_ptr()), C.c_void_p(self.kv_caches[block_idx].data_ptr()), C.c_void_p(out.data_ptr()),
                    C.c_void_p(self_k.data_ptr()) if has_tail else None, C.c_void_p(self_v.data_ptr()) if has_tail else None,
                    C.c_void_p(self._kv_rows[ts].data_ptr()))
-        if self.device_token_counts:
+        if append_rows is not None:
+            N.check(N.lib.lbm_attn_run_append(*tensors, C.c_void_p(append_rows.data_ptr()), self_k.shape[0], *common))
+        elif self.device_token_counts:
             # the kernels read each stream's visible-token count from its table header, where the
             # last plan left it; the host's count above only sizes the launch
             live = self._tables[ts].data_ptr() + 4 * N.HDR["plan_kv_tokens"]
@@ -678,6 +703,7 @@ class HipPagedKVCacheManager:
             self._counts[ts] = [_StreamCounts(self.max_patch_pages, self.max_special_pages)
                                 for _ in range(self.num_streams)]
             self._plan_valid[ts] = False
+            self._newest_self[ts] = False
             self._plan_tokens[ts] = [0] * self.num_streams
         for i in range(self.num_blocks):
             self.frame_count[i] = 0

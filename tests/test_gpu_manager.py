@@ -264,3 +264,47 @@ def test_flow_keyframe_protocol_of_the_windowed_driver(layout, page_size):
         for p in pol:
             p.reset()
         assert m.num_frames == 0 and m.build_visible_page_table(0) == []
+
+
+@pytest.mark.parametrize("T,H,streams,dtype", [(1004, 16, 1, torch.bfloat16), (203, 4, 3, torch.bfloat16),
+                                               (70, 2, 2, torch.float32), (7, 2, 1, torch.bfloat16)])
+def test_step_that_appends_inside_the_attention_call(T, H, streams, dtype):
+    """step() with the append carried by the attention call (the row table names the new frame by
+    the caller's rows, lbm_attn_run_append stores them once the pool was read) against step() with
+    the append as a launch of its own in front (fuse_append = False): the same outputs bit for bit,
+    the same pools, the same tables - anchor, sliding windows of different lengths, evictions that
+    hand pages out again, keyframes and read-only frames mixed per stream, an inactive stream,
+    three blocks behind one table; split-KV with the combine launch (1,004 tokens), the short-KV
+    kernel and the fp32 kernels (append behind the attention), and one stream of 7 tokens."""
+    from lingbot_map_amd import HipPagedKVCacheManager
+    dev = torch.device("cuda:0")
+    kw = dict(num_special_tokens=3, scale_frames=1, sliding_window=[4, 2, 3][:streams] if streams > 1 else 4,
+              max_total_frames=64, page_size=16, layout="frame_pages", num_streams=streams, force_fp32=dtype == torch.float32)
+    a = HipPagedKVCacheManager(3, 24, T, H, 64, dtype, dev, **kw)
+    b = HipPagedKVCacheManager(3, 24, T, H, 64, dtype, dev, **kw)
+    b.fuse_append = False
+    g = torch.Generator(device=dev).manual_seed(T + H)
+    for i in range(9):
+        keyframe = [(i + s) % 4 != 2 or i < 2 for s in range(streams)]
+        if streams == 3 and i == 5:
+            a.set_active_streams([True, False, True]); b.set_active_streams([True, False, True])
+        if streams == 3 and i == 6:
+            a.set_active_streams(None); b.set_active_streams(None)
+        for blk in range(3):
+            q, k, v = (torch.randn(streams * T, H, 64, generator=g, device=dev).to(dtype) / (2 if j else 1) for j in range(3))
+            oa = a.step(blk, q, k, v, keyframe=keyframe, cross_frame_special=False)
+            ob = b.step(blk, q, k, v, keyframe=keyframe, cross_frame_special=False)
+            torch.cuda.synchronize()
+            assert torch.isfinite(oa.float()).all() and torch.equal(oa, ob), (i, blk)
+        assert a._newest_self[0] == any(keyframe) and not b._newest_self[0]
+    for x, y in zip(a.kv_caches, b.kv_caches):
+        assert torch.equal(x, y)
+    assert torch.equal(a._tables, b._tables)
+    for s in range(streams):
+        assert a.build_visible_page_table(0, stream=s) == b.build_visible_page_table(0, stream=s)
+    a.check_device_errors(); b.check_device_errors()
+    # a block that does not go through step() on a frame that step() led is refused
+    q, k, v = (torch.randn(streams * T, H, 64, generator=g, device=dev).to(dtype) for _ in range(3))
+    a.step(0, q, k, v, keyframe=[True] * streams, cross_frame_special=False)
+    with pytest.raises(RuntimeError):
+        a._attend_planned(1, q, None, None)

@@ -206,3 +206,38 @@ def test_error_word_instead_of_corruption(host_lib):
     ht.step([{"ops": OP_RESET}]); ht.step([{"ops": OP_APPEND}], append=True)
     _, _, rows = ht.visible(7 + 3)
     assert ht.hdr()[10] == 32 and rows[7:] == [0, 0, 0]
+
+
+@pytest.mark.parametrize("page_size", [4, 16, 3])
+def test_plan_with_the_newest_frame_named_by_the_callers_rows(host_lib, page_size):
+    """LBM_OP_PLAN_NEWEST_SELF: the row table of a step that appends, evicts and plans is the
+    ordinary one except for the rows of the frame just appended, which name the caller's rows
+    (-1 - (q_begin + t)) in the same place; page lists, counts and the table state are the same.
+    Two streams, the second with its own q_begin; anchor frames, a sliding window with evictions
+    and trajectory-memory tokens behind the frames."""
+    T, n_special = 11, 3
+    pols = [PagePolicy(T, n_special, page_size, 1, 3, max_total_frames=12, layout=LAYOUT_FRAME_PAGES) for _ in range(2)]
+    keep = pols[0]._keep_tokens(True, False)          # evicted frames leave their special tokens behind
+    plain = HostTables(host_lib, pols[0], n_streams=2, max_total_frames=12)
+    flagged = HostTables(host_lib, pols[0], n_streams=2, max_total_frames=12)
+    visible = [0, 0]
+    for frame in range(9):
+        for b in range(2):
+            if b == 1 and frame % 3 == 2:
+                continue      # the second stream skips some frames
+            pols[b].append_frame(); pols[b].evict_frames(1, 3)
+            visible[b] = pols[b].visible_tokens()
+            base = {"sliding_window": 3, "keep_tokens": keep, "expect_kv_tokens": visible[b]}
+            per = lambda extra: [dict(base, ops=OP_APPEND | OP_EVICT | OP_PLAN | extra) if i == b else {"ops": 0} for i in range(2)]
+            plain.step(per(0), append=True, plan=True)
+            flagged.step(per(32), append=True, plan=True)
+            assert np.array_equal(plain.tables, flagged.tables) and np.array_equal(plain.append_rows, flagged.append_rows)
+            assert np.array_equal(plain.ids, flagged.ids) and np.array_equal(plain.lens, flagged.lens)
+            lo = b * plain.rows_cap
+            want = plain.kv_rows[lo: lo + visible[b]].copy()
+            n_frames = int(plain.hdr(b)[1]) + int(plain.hdr(b)[3])          # anchor + window frames
+            first = (n_frames - 1) * T
+            assert want[first: first + T].tolist() == plain.append_rows[b * T: (b + 1) * T].tolist()   # the newest frame's pool rows
+            want[first: first + T] = -1 - (b * T + np.arange(T))
+            assert flagged.kv_rows[lo: lo + visible[b]].tolist() == want.tolist()
+            assert flagged.hdr(b)[10] == 0
