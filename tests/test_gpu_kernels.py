@@ -547,3 +547,54 @@ def test_fp32_running_maximum_covers_every_lane_group():
     want = v[c > 0].mean(dim=0)                                # [H, D]
     assert torch.isfinite(out).all()
     assert (out.cpu() - want[None]).abs().max().item() <= 1e-5
+
+
+@pytest.mark.parametrize("rows,H,cached,dtype", [(1004, 16, 6000, "bf16"), (300, 4, 900, "bf16"), (70, 2, 200, "f32")])
+def test_attn_run_append_equals_append_then_run(rows, H, cached, dtype):
+    """lbm_attn_run_append through the C ABI: the new rows are attended to from the caller's
+    tensors (row-table entries -1 - r where their pool rows would stand) and stored afterwards,
+    against lbm_kv_append followed by lbm_attn_run over a table that names the stored rows: equal
+    outputs and equal pools - with a merging launch to carry the copy (split KV), without one
+    (short KV), and on the fp32 kernels; gated rows (negative entries) are not stored; argument
+    checks."""
+    N = _native()
+    dev = torch.device("cuda:0")
+    D, S = 64, 16
+    td = torch.bfloat16 if dtype == "bf16" else torch.float32
+    dt = N.DTYPE_BF16 if dtype == "bf16" else N.DTYPE_F32
+    g = torch.Generator(device=dev).manual_seed(rows + cached)
+    n_pages = (cached + rows) // S + 8
+    pool0 = torch.randn(n_pages, 2, S, H, D, generator=g, device=dev).to(td)
+    q, k, v = (torch.randn(rows, H, D, generator=g, device=dev).to(td) for _ in range(3))
+    slots = torch.randperm(n_pages * S, generator=g, device=dev)
+    to_row = lambda s: ((s // S) * 2 * S + s % S).to(torch.int32)
+    old_rows, new_rows = to_row(slots[:cached]), to_row(slots[cached:cached + rows])
+    gated = new_rows.clone()
+    gated[::5] = -1                                                    # rows that are not stored
+    arr = (N.AttnStream * 1)(N.AttnStream(0, rows, 0, cached + rows))
+    need = N.lib.lbm_attn_workspace_bytes(arr, 1, H, D)
+    ws = torch.empty(max(int(need), 16), dtype=torch.uint8, device=dev)
+    scale = 1.0 / math.sqrt(D)
+    for append_rows in (new_rows, gated):
+        # the two-call way: store, then attend to a table of pool rows (gated rows from the caller's tensors)
+        pool_a = pool0.clone()
+        N.check(N.lib.lbm_kv_append(ptr(k), ptr(v), dt, ptr(pool_a), dt, ptr(append_rows), rows, H, D, S, None))
+        own = (-1 - torch.arange(rows, device=dev, dtype=torch.int32))
+        table_a = torch.cat([old_rows, torch.where(append_rows >= 0, append_rows, own)]).contiguous()
+        out_a = torch.full_like(q, float("nan"))
+        N.check(N.lib.lbm_attn_run(ptr(q), ptr(pool_a), ptr(out_a), ptr(k), ptr(v), ptr(table_a), arr, 1, H, D, S, dt, scale,
+                                   ptr(ws), ws.numel(), None))
+        # the one-call way
+        pool_b = pool0.clone()
+        table_b = torch.cat([old_rows, own]).contiguous()
+        out_b = torch.full_like(q, float("nan"))
+        N.check(N.lib.lbm_attn_run_append(ptr(q), ptr(pool_b), ptr(out_b), ptr(k), ptr(v), ptr(table_b), ptr(append_rows), rows,
+                                          arr, 1, H, D, S, dt, scale, ptr(ws), ws.numel(), None))
+        torch.cuda.synchronize()
+        assert torch.isfinite(out_b.float()).all() and torch.equal(out_a, out_b)
+        assert torch.equal(pool_a, pool_b) and not torch.equal(pool_b, pool0)
+    bad = lambda *a: N.lib.lbm_attn_run_append(*a) != N.OK
+    common = (arr, 1, H, D, S, dt, scale, ptr(ws), ws.numel(), None)
+    assert bad(ptr(q), ptr(pool_b), ptr(out_b), None, ptr(v), ptr(table_b), ptr(new_rows), rows, *common)
+    assert bad(ptr(q), ptr(pool_b), ptr(out_b), ptr(k), ptr(v), ptr(table_b), None, rows, *common)
+    assert bad(ptr(q), ptr(pool_b), ptr(out_b), ptr(k), ptr(v), ptr(table_b), ptr(new_rows), -1, *common)
